@@ -1,0 +1,127 @@
+/*
+ * tessera_qmm.h -- C ABI of the MI355X (gfx950) quantized-matmul kernel library.
+ *
+ * The library is the device side of a tessera `Backend` for the quantized matmul
+ * path only.  Tessera has no C ABI of its own: its backends are C++ classes linked
+ * into the binary (tessera::CreateBackend, include/tessera/backend.hpp:1062-1071).
+ * Each entry point below therefore names the Backend virtual, or the piece of
+ * RocmBackend, that a thin C++ adapter implements by calling it.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every device pointer is a HIP device address
+ *     on the device chosen by qmm_init;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All work
+ *     is asynchronous on that stream, like RocmBackend's single stream
+ *     (src/backends/rocm/rocm_backend.cpp:311-330,716-722);
+ *   - every function returns a qmm_status whose integer values are identical to
+ *     tessera::StatusCode (include/tessera/types.hpp:36-48);
+ *   - no exceptions cross the boundary and nothing here allocates device memory
+ *     except qmm_alloc.
+ */
+#ifndef TESSERA_QMM_H_
+#define TESSERA_QMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t qmm_status;
+enum {
+  QMM_OK = 0,
+  QMM_INVALID_ARGUMENT = 1,
+  QMM_FILE_NOT_FOUND = 2,
+  QMM_MALFORMED_FILE = 3,
+  QMM_UNSUPPORTED_FEATURE = 4,
+  QMM_OUT_OF_MEMORY = 5,
+  QMM_DEVICE_ERROR = 6,
+  QMM_NON_FINITE = 7,
+  QMM_NETWORK_ERROR = 8
+};
+
+/* Binding limits of one launch (include/tessera/backend.hpp:45-48). */
+#define QMM_MAX_BOUND_BUFFERS 16
+#define QMM_MAX_SCALARS 16
+
+/* Opaque kernel handle: table index + 1, never 0 for a loaded kernel.  Same
+ * representation as RocmBackend (src/backends/rocm/rocm_backend.cpp:639-670). */
+typedef uintptr_t qmm_kernel;
+
+/* Backend::SetDeviceIndex + Backend::Init (backend.hpp:869-889;
+ * rocm_backend.cpp:270-333).  Selects the device, checks that it is a gfx950 part
+ * and that the library's code object loads.  Ok when already initialised on the same
+ * device; InvalidArgument for an index out of range; UnsupportedFeature on a device
+ * that is not gfx950; DeviceError for any HIP failure. */
+qmm_status qmm_init(int device);
+
+/* Backend::DeviceName (backend.hpp:853-854).  Valid after qmm_init; "" before. */
+const char* qmm_device_name(void);
+
+/* Backend::MemoryInfo (backend.hpp:856-859). */
+qmm_status qmm_memory_info(uint64_t* total_bytes, uint64_t* free_bytes);
+
+/* Backend::AllocateBuffer(bytes, MemoryKind::Device) / Backend::FreeBuffer
+ * (backend.hpp:891-906; rocm_backend.cpp:335-376).  0 bytes is InvalidArgument;
+ * hipErrorOutOfMemory maps to OutOfMemory. */
+qmm_status qmm_alloc(size_t bytes, void** out_device_ptr);
+qmm_status qmm_free(void* device_ptr);
+
+/* Backend::CopyH2DAt / CopyD2HAt / CopyD2D (backend.hpp:912-965;
+ * rocm_backend.cpp:378-408,523-550).  The adapter does the bounds check against its
+ * Buffer sizes and passes already-offset pointers.  H2D and D2H return after the
+ * copy has completed (they synchronise the stream, as the reference does); D2D is
+ * asynchronous. */
+qmm_status qmm_copy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
+qmm_status qmm_copy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
+qmm_status qmm_copy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
+
+/* Backend::LoadKernel(name, {}) for built-ins (backend.hpp:1004-1017;
+ * rocm_backend.cpp:639-670).  An id this library does not implement returns
+ * UnsupportedFeature, which the callers rely on to fall through to another regime
+ * (src/models/qwen3_5/project.cpp:109-112,285,303,319,331). */
+qmm_status qmm_load(const char* id, qmm_kernel* out);
+
+/* Kernel::Id() of a loaded handle; NULL for a bad handle. */
+const char* qmm_kernel_id(qmm_kernel kernel);
+
+/* The ids qmm_load accepts, for diagnostics: count, then name by index. */
+size_t qmm_kernel_count(void);
+const char* qmm_kernel_name(size_t index);
+
+/* Backend::LaunchKernel (backend.hpp:1022-1026; rocm_backend.cpp:672-729) with
+ * KernelLaunch flattened: grid[3], block[3], buffers in kernel parameter order, then
+ * 64-bit scalars (floats travel as fp32 bit patterns in the low 32 bits).
+ *
+ * Validation happens before any device work and returns InvalidArgument: zero grid or
+ * block dimensions, more than 16 buffers or scalars (ValidateLaunch,
+ * backend.hpp:138-148), the per-id argument counts and shape rules of
+ * CheckBuiltInArgs (backend.hpp:391-841), a NULL buffer, and -- when `buf_bytes` is
+ * not NULL -- any buffer smaller than the launch's scalars require.  `buf_bytes[i]` is
+ * Buffer::Size() of buffer i; pass NULL to skip the size check.
+ *
+ * Geometry: the ids keep the reference's argument contracts, but a gfx950 kernel has
+ * its own natural launch shape, so `grid` and `block` are validated and otherwise
+ * ignored: the library picks the launch shape from the scalars.  (The Vulkan backend
+ * ignores block_* the same way, backend.hpp:50-55.)  Split-K ids
+ * ("gemm_q4k_vec", "gemm_q4k_rows{2..5}", "gemm_mxfp4_wmma") honour the `split` scalar
+ * of their contract: the sum over the `split` output regions equals the result, so the
+ * reference's reduce pass ("gemm_vec_reduce", "gemm_mxfp4_wmma_reduce") still works.
+ */
+qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                      void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
+                      const uint64_t* scalars, size_t nscalars, void* stream);
+
+/* Backend::Synchronize (backend.hpp:1028-1029; rocm_backend.cpp:731-739). */
+qmm_status qmm_sync(void* stream);
+
+/* Text of the last HIP error seen by this thread ("" if none), for the adapter's
+ * diagnostics channel (Backend::SetDiagnostics, backend.hpp:861-863). */
+const char* qmm_last_error(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* TESSERA_QMM_H_ */

@@ -1,0 +1,295 @@
+"""ctypes front-end of the CPU oracle (``qmm_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the
+CPU-baseline leg of ``bench.py``.  The product package never imports this module.
+
+All functions take and return numpy arrays; byte buffers are ``uint8``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+Q4K_ELEMS = 256
+Q4K_BYTES = 144
+
+
+def build(force: bool = False) -> str:
+    """Compile ``qmm_oracle.c`` into ``liboracle.so`` with gcc."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = C.CDLL(_LIB_PATH)
+    f32p, u8p, u32p = C.POINTER(C.c_float), C.POINTER(C.c_uint8), C.POINTER(C.c_uint32)
+    sz = C.c_size_t
+    sig = {
+        "orc_fp16_to_float": (C.c_float, [C.c_uint16]),
+        "orc_fp32_to_half_bits": (C.c_uint16, [C.c_float]),
+        "orc_round_bf16": (None, [f32p, sz]),
+        "orc_fp8_e4m3_to_float": (C.c_float, [C.c_uint8]),
+        "orc_e8m0_to_float": (C.c_float, [C.c_uint8]),
+        "orc_f4e2m1_to_float": (C.c_float, [C.c_uint8]),
+        "orc_fp32_to_fp8_e4m3": (C.c_uint8, [C.c_float]),
+        "orc_get_scale_min": (None, [sz, u8p, u8p, u8p]),
+        "orc_dequantize_q4k": (None, [u8p, f32p]),
+        "orc_dequantize_q4k_rows": (None, [u8p, f32p, sz]),
+        "orc_quantize_q4k": (None, [f32p, u8p]),
+        "orc_quantize_fp8_ref": (C.c_int, [f32p, f32p, sz, sz]),
+        "orc_quantize_fp8_pack_ref": (C.c_int, [f32p, u8p, f32p, sz, sz]),
+        "orc_gemm_q4k_ref": (C.c_int, [f32p, u8p, f32p, sz, sz, sz]),
+        "orc_gemm_q4k_ref_omp": (C.c_int, [f32p, u8p, f32p, sz, sz, sz]),
+        "orc_gemm_mxfp4_ref": (C.c_int, [f32p, u8p, u8p, f32p, sz, sz, sz]),
+        "orc_dequantize_mxfp4": (C.c_int, [u8p, f32p, sz, sz]),
+        "orc_gemm_fp8_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
+        "orc_fold_entry": (C.c_uint8, [C.c_uint, C.c_uint]),
+        "orc_fold_entry_rne": (C.c_uint8, [C.c_uint, C.c_uint]),
+        "orc_fold_mxfp4_to_fp8": (C.c_int, [u8p, u8p, u8p, u8p, sz, sz]),
+        "orc_gemm_mxfp4_fp8_ref": (C.c_int, [u8p, f32p, u8p, u8p, f32p, sz, sz, sz]),
+        "orc_gemm_mxfp4_w4a8_ref": (C.c_int, [u8p, f32p, u8p, u8p, f32p, sz, sz, sz]),
+        "orc_moe_gate": (None, [f32p, f32p, sz]),
+        "orc_top_k_row": (None, [f32p, sz, sz, u32p, f32p]),
+        "orc_moe_expert_forward_q4k": (C.c_int, [f32p, u8p, u8p, u8p, sz, sz, f32p]),
+        "orc_moe_experts_forward_q4k": (
+            C.c_int, [f32p, u32p, f32p, sz, u8p, sz, u8p, sz, u8p, sz, sz, sz, f32p]),
+        "orc_moe_batch_forward_q4k": (
+            C.c_int, [f32p, u32p, f32p, sz, sz, u8p, sz, u8p, sz, u8p, sz, sz, sz, f32p]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+_lib = _load()
+
+
+class OracleError(RuntimeError):
+    """A routine returned a non-zero tessera StatusCode."""
+
+    def __init__(self, code: int):
+        super().__init__(f"oracle status {code}")
+        self.code = code
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise OracleError(code)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+def _p(a: np.ndarray, ty):
+    return a.ctypes.data_as(C.POINTER(ty))
+
+
+# ---- scalar codecs -------------------------------------------------------
+def fp16_to_float(bits: int) -> float:
+    return _lib.orc_fp16_to_float(bits)
+
+
+def fp32_to_half_bits(v: float) -> int:
+    return _lib.orc_fp32_to_half_bits(v)
+
+
+def fp8_e4m3_to_float(code: int) -> float:
+    return _lib.orc_fp8_e4m3_to_float(code)
+
+
+def e8m0_to_float(code: int) -> float:
+    return _lib.orc_e8m0_to_float(code)
+
+
+def f4e2m1_to_float(nib: int) -> float:
+    return _lib.orc_f4e2m1_to_float(nib)
+
+
+def fp32_to_fp8_e4m3(v: float) -> int:
+    return _lib.orc_fp32_to_fp8_e4m3(v)
+
+
+def fold_entry(d: int, mag: int) -> int:
+    return _lib.orc_fold_entry(d, mag)
+
+
+def fold_entry_rne(d: int, mag: int) -> int:
+    return _lib.orc_fold_entry_rne(d, mag)
+
+
+def round_bf16(x) -> np.ndarray:
+    out = _f32(x).copy()
+    _lib.orc_round_bf16(_p(out, C.c_float), out.size)
+    return out
+
+
+def get_scale_min(j: int, scales12) -> tuple[int, int]:
+    s = _u8(scales12)
+    assert s.size == 12
+    sc, mn = C.c_uint8(), C.c_uint8()
+    _lib.orc_get_scale_min(j, _p(s, C.c_uint8), C.byref(sc), C.byref(mn))
+    return sc.value, mn.value
+
+
+# ---- Q4_K ----------------------------------------------------------------
+def dequantize_q4k(w) -> np.ndarray:
+    """Any whole number of 144-byte super-blocks -> fp32, 256 values per block."""
+    w = _u8(w).reshape(-1)
+    assert w.size % Q4K_BYTES == 0
+    nb = w.size // Q4K_BYTES
+    out = np.empty(nb * Q4K_ELEMS, dtype=np.float32)
+    _lib.orc_dequantize_q4k_rows(_p(w, C.c_uint8), _p(out, C.c_float), nb)
+    return out
+
+
+def quantize_q4k(x) -> np.ndarray:
+    x = _f32(x).reshape(-1)
+    assert x.size % Q4K_ELEMS == 0
+    nb = x.size // Q4K_ELEMS
+    out = np.zeros(nb * Q4K_BYTES, dtype=np.uint8)
+    for b in range(nb):
+        xb = x[b * Q4K_ELEMS:(b + 1) * Q4K_ELEMS]
+        ob = out[b * Q4K_BYTES:(b + 1) * Q4K_BYTES]
+        _lib.orc_quantize_q4k(_p(xb, C.c_float), _p(ob, C.c_uint8))
+    return out
+
+
+def gemm_q4k(a, w, m: int, n: int, k: int, threads: bool = False) -> np.ndarray:
+    a, w = _f32(a), _u8(w)
+    if k % Q4K_ELEMS == 0 and k and n and m:
+        assert a.size == m * k and w.size == n * (k // Q4K_ELEMS) * Q4K_BYTES
+    c = np.empty((m, n), dtype=np.float32)
+    fn = _lib.orc_gemm_q4k_ref_omp if threads else _lib.orc_gemm_q4k_ref
+    _check(fn(_p(a, C.c_float), _p(w, C.c_uint8), _p(c, C.c_float), m, n, k))
+    return c
+
+
+# ---- MXFP4 / FP8 ----------------------------------------------------------
+def split_mxfp4(packed, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:
+    """Packed device layout -> (blob n*k/2 bytes, scales n*k/32 bytes)."""
+    packed = _u8(packed).reshape(-1)
+    assert packed.size == n * k // 2 + n * k // 32
+    return packed[: n * k // 2], packed[n * k // 2:]
+
+
+def gemm_mxfp4(a, packed, m: int, n: int, k: int) -> np.ndarray:
+    a = _f32(a)
+    blob, s = split_mxfp4(packed, n, k)
+    c = np.empty((m, n), dtype=np.float32)
+    _check(_lib.orc_gemm_mxfp4_ref(_p(a, C.c_float), _p(blob, C.c_uint8), _p(s, C.c_uint8),
+                                   _p(c, C.c_float), m, n, k))
+    return c
+
+
+def dequantize_mxfp4(packed, n: int, k: int) -> np.ndarray:
+    packed = _u8(packed).reshape(-1)
+    out = np.empty((n, k), dtype=np.float32)
+    _check(_lib.orc_dequantize_mxfp4(_p(packed, C.c_uint8), _p(out, C.c_float), n, k))
+    return out
+
+
+def gemm_fp8(a, w, s, m: int, n: int, k: int) -> np.ndarray:
+    a, w, s = _f32(a), _u8(w), _f32(s)
+    assert a.size == m * k and w.size == n * k and s.size == n
+    c = np.empty((m, n), dtype=np.float32)
+    _check(_lib.orc_gemm_fp8_ref(_p(a, C.c_float), _p(w, C.c_uint8), _p(s, C.c_float),
+                                 _p(c, C.c_float), m, n, k))
+    return c
+
+
+def quantize_fp8(data, rows: int, cols: int) -> tuple[np.ndarray, np.ndarray]:
+    """Quantize-dequantize; returns (qdq data, scales)."""
+    out = _f32(data).copy().reshape(rows, cols)
+    scale = np.empty(rows, dtype=np.float32)
+    _check(_lib.orc_quantize_fp8_ref(_p(out, C.c_float), _p(scale, C.c_float), rows, cols))
+    return out, scale
+
+
+def quantize_fp8_pack(data, rows: int, cols: int) -> tuple[np.ndarray, np.ndarray]:
+    """Returns (e4m3 codes rows x cols, scales)."""
+    src = _f32(data).reshape(rows, cols)
+    codes = np.empty((rows, cols), dtype=np.uint8)
+    scale = np.empty(rows, dtype=np.float32)
+    _check(_lib.orc_quantize_fp8_pack_ref(_p(src, C.c_float), _p(codes, C.c_uint8),
+                                          _p(scale, C.c_float), rows, cols))
+    return codes, scale
+
+
+def fold_mxfp4_to_fp8(packed, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:
+    blob, s = split_mxfp4(packed, n, k)
+    out = np.empty((n, k), dtype=np.uint8)
+    wref = np.empty(n, dtype=np.uint8)
+    _check(_lib.orc_fold_mxfp4_to_fp8(_p(blob, C.c_uint8), _p(s, C.c_uint8), _p(out, C.c_uint8),
+                                      _p(wref, C.c_uint8), n, k))
+    return out, wref
+
+
+def gemm_mxfp4_fp8(a8, a_scale, w8, wref, m: int, n: int, k: int) -> np.ndarray:
+    a8, a_scale, w8, wref = _u8(a8), _f32(a_scale), _u8(w8), _u8(wref)
+    c = np.empty((m, n), dtype=np.float32)
+    _check(_lib.orc_gemm_mxfp4_fp8_ref(_p(a8, C.c_uint8), _p(a_scale, C.c_float),
+                                       _p(w8, C.c_uint8), _p(wref, C.c_uint8),
+                                       _p(c, C.c_float), m, n, k))
+    return c
+
+
+def gemm_mxfp4_w4a8(a8, a_scale, packed, m: int, n: int, k: int) -> np.ndarray:
+    a8, a_scale = _u8(a8), _f32(a_scale)
+    blob, s = split_mxfp4(packed, n, k)
+    c = np.empty((m, n), dtype=np.float32)
+    _check(_lib.orc_gemm_mxfp4_w4a8_ref(_p(a8, C.c_uint8), _p(a_scale, C.c_float),
+                                        _p(blob, C.c_uint8), _p(s, C.c_uint8),
+                                        _p(c, C.c_float), m, n, k))
+    return c
+
+
+# ---- MoE -------------------------------------------------------------------
+def moe_gate(vals) -> np.ndarray:
+    v = _f32(vals).reshape(-1)
+    out = np.empty_like(v)
+    _lib.orc_moe_gate(_p(v, C.c_float), _p(out, C.c_float), v.size)
+    return out
+
+
+def top_k_row(logits, top_k: int) -> tuple[np.ndarray, np.ndarray]:
+    lg = _f32(logits).reshape(-1)
+    ids = np.empty(top_k, dtype=np.uint32)
+    vals = np.empty(top_k, dtype=np.float32)
+    _lib.orc_top_k_row(_p(lg, C.c_float), lg.size, top_k, _p(ids, C.c_uint32), _p(vals, C.c_float))
+    return ids, vals
+
+
+def moe_batch_forward_q4k(x, ids, wts, gate, up, down, hidden: int, inter: int) -> np.ndarray:
+    """Routed-expert sum per token.  gate/up: [E][inter][hidden/256] blocks; down:
+    [E][hidden][inter/256] blocks; ids/wts: rows x top_k."""
+    x = _f32(x).reshape(-1, hidden)
+    rows = x.shape[0]
+    ids = np.ascontiguousarray(ids, dtype=np.uint32).reshape(rows, -1)
+    wts = _f32(wts).reshape(rows, -1)
+    top_k = ids.shape[1]
+    gate, up, down = _u8(gate).reshape(-1), _u8(up).reshape(-1), _u8(down).reshape(-1)
+    gs = inter * (hidden // Q4K_ELEMS) * Q4K_BYTES
+    ds = hidden * (inter // Q4K_ELEMS) * Q4K_BYTES
+    out = np.empty((rows, hidden), dtype=np.float32)
+    _check(_lib.orc_moe_batch_forward_q4k(
+        _p(x, C.c_float), _p(ids, C.c_uint32), _p(wts, C.c_float), rows, top_k,
+        _p(gate, C.c_uint8), gs, _p(up, C.c_uint8), gs, _p(down, C.c_uint8), ds,
+        hidden, inter, _p(out, C.c_float)))
+    return out

@@ -1,0 +1,593 @@
+/*
+ * CPU oracle for the quantized-matmul path: TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain-C restatement of the host reference numerics of Quackster/tessera
+ * (src/core/numerics/{quant,gemm,moe_cpu}.cpp).  Nothing in the product may
+ * call into this file: it is the checker used by tests/, by the smoke check
+ * and by the CPU-baseline leg of the benchmark, never the thing shipped or
+ * measured as the product.
+ *
+ * Every routine cites the reference lines it follows.  Each is pinned by
+ * tests/test_oracle_*.py against closed forms, exhaustive sweeps against
+ * numpy/torch IEEE conversions, brute-force layout extraction and the few
+ * known-answer values the reference documents (see the test files).  The
+ * reference ships no test fixtures for this path, and its own sources do not
+ * compile in this image (they need the C++23 <expected> header), so no
+ * compiled-reference cross-check exists.
+ *
+ * Pin status:
+ *   fp16/bf16/e4m3/e8m0/e2m1 codecs ......... pinned (exhaustive)
+ *   Q4_K scale unpack + block decode ........ pinned (bit-serial brute force, closed form)
+ *   fp8 per-row quantize (QDQ and pack) ..... pinned (invariants + torch.float8_e4m3fn)
+ *   gemm_* sequential-fma references ........ pinned (one-hot identity, float64 bound)
+ *   MXFP4->e4m3 fold table .................. pinned (the reference's literal 16x8 table, kept
+ *                                             as a golden fixture; equals the encoder except 3
+ *                                             tie entries)
+ *   MoE expert forward / gate ............... pinned (composition of pinned parts; softmax
+ *                                             vs torch)
+ *
+ * Status codes mirror tessera::StatusCode (include/tessera/types.hpp:36-48).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_OK 0
+#define ORC_INVALID_ARGUMENT 1
+#define ORC_UNSUPPORTED 4
+#define ORC_OOM 5
+
+#define Q4K_ELEMS 256u
+#define Q4K_BYTES 144u
+#define MX_BLOCK 32u
+
+/* quant.hpp:58-64 */
+static const float kE4M3Max = 448.0f;
+static const float kE4M3MinScale = 1.0f / (448.0f * 512.0f);
+
+static uint32_t f32_bits(float v) {
+  uint32_t b;
+  memcpy(&b, &v, 4);
+  return b;
+}
+static float bits_f32(uint32_t b) {
+  float v;
+  memcpy(&v, &b, 4);
+  return v;
+}
+
+/* ---- IEEE binary16 -> binary32, exact (quant.cpp:74-91) ---- */
+float orc_fp16_to_float(uint16_t h) {
+  const uint32_t s = h >> 15, e = (h >> 10) & 31u, m = h & 1023u;
+  float v;
+  if (e == 0) {
+    v = (float)m * 0x1p-24f;
+  } else if (e == 31) {
+    v = m ? nanf("") : INFINITY;
+  } else {
+    v = (1.0f + (float)m / 1024.0f) * ldexpf(1.0f, (int)e - 15);
+  }
+  return s ? -v : v;
+}
+
+/* Right shift with round-to-nearest-even (quant.cpp:42-52). */
+static uint32_t shift_rne(uint32_t v, int sh) {
+  const uint32_t rem = v & ((1u << sh) - 1u), half = 1u << (sh - 1);
+  uint32_t r = v >> sh;
+  if (rem > half || (rem == half && (r & 1u))) ++r;
+  return r;
+}
+
+/* ---- binary32 -> binary16 bits, RNE (quant.cpp:606-654) ---- */
+uint16_t orc_fp32_to_half_bits(float v) {
+  const uint32_t b = f32_bits(v);
+  const uint32_t s = b >> 31, ef = (b >> 23) & 255u, m = b & 0x7FFFFFu;
+  const uint16_t inf = (uint16_t)((s << 15) | 0x7C00u);
+  if (ef == 255u) return (uint16_t)(inf | (m ? 0x200u : 0u));
+  if (ef == 0u) return (uint16_t)(s << 15);
+  const int e = (int)ef - 127;
+  if (e > 15) return inf;
+  if (e < -14) {
+    const int sh = -e - 1;
+    if (sh >= 32) return (uint16_t)(s << 15);
+    const uint32_t r = shift_rne(m + (1u << 23), sh);
+    if (r > 1023u) return (uint16_t)((s << 15) | 0x0400u);
+    return (uint16_t)((s << 15) | r);
+  }
+  const uint32_t m10 = shift_rne(m, 13);
+  if (m10 > 1023u) {
+    if (e + 1 > 15) return inf;
+    return (uint16_t)((s << 15) | ((uint32_t)(e + 1 + 15) << 10));
+  }
+  return (uint16_t)((s << 15) | ((uint32_t)(e + 15) << 10) | m10);
+}
+
+/* ---- fp32 -> nearest bf16 value kept in fp32 storage (quant.cpp:231-243) ---- */
+void orc_round_bf16(float* x, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    uint32_t b = f32_bits(x[i]);
+    b += 0x7FFFu + ((b >> 16) & 1u);
+    b &= 0xFFFF0000u;
+    x[i] = bits_f32(b);
+  }
+}
+
+/* ---- OCP FP8 E4M3 byte -> fp32 (quant.cpp:258-277) ---- */
+float orc_fp8_e4m3_to_float(uint8_t c) {
+  const uint32_t s = c >> 7, e = (c >> 3) & 15u, m = c & 7u;
+  float v;
+  if (e == 0) {
+    v = (float)m * 0x1p-9f;
+  } else if (e == 15) {
+    if (m == 7) return nanf("");
+    v = (1.0f + (float)m / 8.0f) * 256.0f;
+  } else {
+    v = (1.0f + (float)m / 8.0f) * ldexpf(1.0f, (int)e - 7);
+  }
+  return s ? -v : v;
+}
+
+/* ---- E8M0 shared exponent -> fp32: 2^(s-127) (quant.cpp:279-281) ---- */
+float orc_e8m0_to_float(uint8_t s) { return ldexpf(1.0f, (int)s - 127); }
+
+/* ---- OCP E2M1 nibble -> fp32 (quant.cpp:283-297) ---- */
+float orc_f4e2m1_to_float(uint8_t nib) {
+  const uint32_t s = (nib >> 3) & 1u, e = (nib >> 1) & 3u, m = nib & 1u;
+  float v;
+  if (e == 0) {
+    v = (float)m * 0.5f;
+  } else {
+    v = (1.0f + (float)m / 2.0f) * ldexpf(1.0f, (int)e - 1);
+  }
+  return s ? -v : v;
+}
+
+/* ---- fp32 -> OCP FP8 E4M3 byte, RNE, NaN and |x|>448 -> 0x7F (quant.cpp:299-342) ---- */
+uint8_t orc_fp32_to_fp8_e4m3(float v) {
+  const uint32_t b = f32_bits(v);
+  const uint32_t s = b >> 31;
+  if ((b & 0x7FFFFFFFu) > 0x7F800000u) return (uint8_t)((s << 7) | 0x7Fu);
+  const float a = v < 0 ? -v : v;
+  if (a == 0.0f) return (uint8_t)(s << 7);
+  if (a > 448.0f) return (uint8_t)((s << 7) | 0x7Fu);
+  int ex = 0;
+  const float fr = frexpf(a, &ex); /* a = fr * 2^ex, fr in [0.5, 1) */
+  int field = ex + 6;
+  if (field < 1) {
+    long long m = llrintf(a * 512.0f);
+    if (m > 7) m = 7;
+    return (uint8_t)((s << 7) | (uint32_t)m);
+  }
+  long long m = llrintf((fr * 2.0f - 1.0f) * 8.0f);
+  if (m == 8) {
+    m = 0;
+    ++field;
+  }
+  if (field > 15) field = 15;
+  if (field == 15 && m > 6) m = 6;
+  return (uint8_t)((s << 7) | ((uint32_t)field << 3) | (uint32_t)m);
+}
+
+/* ---- Q4_K 6-bit (scale, min) pair of sub-block j from the 12-byte packing
+ *      (quant.cpp:58-70; layout text quant.hpp:11-15) ---- */
+void orc_get_scale_min(size_t j, const uint8_t* p, uint8_t* sc, uint8_t* mn) {
+  if (j < 4) {
+    *sc = p[j] & 63u;
+    *mn = p[j + 4] & 63u;
+  } else {
+    *sc = (uint8_t)((p[j + 4] & 15u) | ((p[j - 4] >> 6) << 4));
+    *mn = (uint8_t)((p[j + 4] >> 4) | ((p[j] >> 6) << 4));
+  }
+}
+
+/* ---- one 144-byte Q4_K super-block -> 256 fp32 (quant.cpp:656-675) ---- */
+void orc_dequantize_q4k(const uint8_t* blk, float* out) {
+  const float d = orc_fp16_to_float((uint16_t)(blk[0] | (blk[1] << 8)));
+  const float dmin = orc_fp16_to_float((uint16_t)(blk[2] | (blk[3] << 8)));
+  const uint8_t* sp = blk + 4;
+  const uint8_t* qs = blk + 16;
+  for (size_t g = 0; g < 4; ++g) {
+    uint8_t sc0, mn0, sc1, mn1;
+    orc_get_scale_min(2 * g, sp, &sc0, &mn0);
+    orc_get_scale_min(2 * g + 1, sp, &sc1, &mn1);
+    const float s0 = d * (float)sc0, o0 = dmin * (float)mn0;
+    const float s1 = d * (float)sc1, o1 = dmin * (float)mn1;
+    for (size_t l = 0; l < 32; ++l) {
+      const uint8_t q = qs[32 * g + l];
+      out[64 * g + l] = s0 * (float)(q & 15u) - o0;
+      out[64 * g + 32 + l] = s1 * (float)(q >> 4) - o1;
+    }
+  }
+}
+
+void orc_dequantize_q4k_rows(const uint8_t* w, float* out, size_t nblocks) {
+  for (size_t b = 0; b < nblocks; ++b) orc_dequantize_q4k(w + b * Q4K_BYTES, out + b * Q4K_ELEMS);
+}
+
+static uint32_t round_half_even_u32(float v) {
+  const long long r = llrint((double)v);
+  return r < 0 ? 0u : (uint32_t)r;
+}
+
+/* ---- 256 fp32 -> one Q4_K super-block, fixture builder (quant.cpp:677-739) ---- */
+void orc_quantize_q4k(const float* x, uint8_t* blk) {
+  memset(blk, 0, Q4K_BYTES);
+  float amax = 0.0f;
+  for (size_t i = 0; i < Q4K_ELEMS; ++i) amax = fmaxf(amax, fabsf(x[i]));
+  if (amax == 0.0f) return;
+  const uint16_t db = orc_fp32_to_half_bits(amax / 32.0f);
+  const float d = orc_fp16_to_float(db), dm = d;
+  blk[0] = blk[2] = (uint8_t)(db & 255u);
+  blk[1] = blk[3] = (uint8_t)(db >> 8);
+  uint8_t* sp = blk + 4;
+  uint8_t* qs = blk + 16;
+  for (size_t j = 0; j < 8; ++j) {
+    const float* sub = x + 32 * j;
+    float lo = sub[0], hi = sub[0];
+    for (size_t i = 1; i < 32; ++i) {
+      lo = fminf(lo, sub[i]);
+      hi = fmaxf(hi, sub[i]);
+    }
+    const float emin = fminf(lo, 0.0f);
+    const float step = (hi - emin) / 15.0f;
+    uint32_t sc = round_half_even_u32(step / d);
+    if (sc > 63u) sc = 63u;
+    uint32_t m = 0;
+    if (lo < 0.0f) {
+      m = round_half_even_u32(-lo / dm);
+      if (m > 63u) m = 63u;
+    }
+    if (j < 4) {
+      sp[j] = (uint8_t)sc;
+      sp[j + 4] = (uint8_t)m;
+    } else {
+      sp[j + 4] = (uint8_t)((sc & 15u) | ((m & 15u) << 4));
+      sp[j - 4] |= (uint8_t)((sc >> 4) << 6);
+      sp[j] |= (uint8_t)((m >> 4) << 6);
+    }
+    const float off = dm * (float)m, scale = d * (float)sc;
+    for (size_t i = 0; i < 32; ++i) {
+      uint32_t q = 0;
+      if (sc != 0) {
+        q = round_half_even_u32((sub[i] + off) / scale);
+        if (q > 15u) q = 15u;
+      }
+      const size_t el = 32 * j + i;
+      const size_t at = 32 * (el / 64) + el % 32;
+      if ((el / 32) % 2 == 1) {
+        qs[at] |= (uint8_t)(q << 4);
+      } else {
+        qs[at] |= (uint8_t)(q & 15u);
+      }
+    }
+  }
+}
+
+/* ---- per-row dynamic E4M3 quantize-dequantize in place (quant.cpp:180-205) ---- */
+int orc_quantize_fp8_ref(float* data, float* scale, size_t rows, size_t cols) {
+  if (rows == 0 || cols == 0) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    float* row = data + r * cols;
+    float amax = 0.0f;
+    for (size_t c = 0; c < cols; ++c) amax = fmaxf(amax, fabsf(row[c]));
+    const float s = fmaxf(amax / kE4M3Max, kE4M3MinScale);
+    scale[r] = s;
+    for (size_t c = 0; c < cols; ++c) {
+      float q = row[c] / s;
+      q = q < -kE4M3Max ? -kE4M3Max : (q > kE4M3Max ? kE4M3Max : q);
+      row[c] = orc_fp8_e4m3_to_float(orc_fp32_to_fp8_e4m3(q)) * s;
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- per-row dynamic E4M3 quantize to packed bytes + scale (quant.cpp:207-229) ---- */
+int orc_quantize_fp8_pack_ref(const float* in, uint8_t* out, float* scale, size_t rows,
+                              size_t cols) {
+  if (rows == 0 || cols == 0 || cols % 4 != 0) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    const float* row = in + r * cols;
+    float amax = 0.0f;
+    for (size_t c = 0; c < cols; ++c) amax = fmaxf(amax, fabsf(row[c]));
+    const float s = fmaxf(amax / kE4M3Max, kE4M3MinScale);
+    scale[r] = s;
+    for (size_t c = 0; c < cols; ++c) {
+      float q = row[c] / s;
+      q = q < -kE4M3Max ? -kE4M3Max : (q > kE4M3Max ? kE4M3Max : q);
+      out[r * cols + c] = orc_fp32_to_fp8_e4m3(q);
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- C = A . deq(W)^T, Q4_K rows, sequential fp32 fma over t = 0..k-1
+ *      (gemm.cpp:18-41,62-73) ---- */
+int orc_gemm_q4k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0 || k % Q4K_ELEMS != 0) return ORC_INVALID_ARGUMENT;
+  const size_t bpr = k / Q4K_ELEMS;
+  float* row = (float*)malloc(k * sizeof(float));
+  if (!row) return ORC_OOM;
+  for (size_t j = 0; j < n; ++j) {
+    orc_dequantize_q4k_rows(w + j * bpr * Q4K_BYTES, row, bpr);
+    for (size_t i = 0; i < m; ++i) {
+      const float* ar = a + i * k;
+      float acc = 0.0f;
+      for (size_t t = 0; t < k; ++t) acc = fmaf(ar[t], row[t], acc);
+      c[i * n + j] = acc;
+    }
+  }
+  free(row);
+  return ORC_OK;
+}
+
+/* Same arithmetic, weight rows spread over OpenMP threads.  Each output keeps
+ * the sequential-t fma chain, so results equal orc_gemm_q4k_ref bit for bit.
+ * Used only to time a multi-core CPU baseline. */
+int orc_gemm_q4k_ref_omp(const float* a, const uint8_t* w, float* c, size_t m, size_t n,
+                         size_t k) {
+  if (m == 0 || n == 0 || k == 0 || k % Q4K_ELEMS != 0) return ORC_INVALID_ARGUMENT;
+  const size_t bpr = k / Q4K_ELEMS;
+  int failed = 0;
+#pragma omp parallel
+  {
+    float* row = (float*)malloc(k * sizeof(float));
+    if (!row) {
+#pragma omp atomic write
+      failed = 1;
+    }
+#pragma omp for schedule(static)
+    for (long long j = 0; j < (long long)n; ++j) {
+      if (!row) continue;
+      orc_dequantize_q4k_rows(w + (size_t)j * bpr * Q4K_BYTES, row, bpr);
+      for (size_t i = 0; i < m; ++i) {
+        const float* ar = a + i * k;
+        float acc = 0.0f;
+        for (size_t t = 0; t < k; ++t) acc = fmaf(ar[t], row[t], acc);
+        c[i * n + (size_t)j] = acc;
+      }
+    }
+    free(row);
+  }
+  return failed ? ORC_OOM : ORC_OK;
+}
+
+/* ---- C = A . deq(W)^T, MXFP4 blob + E8M0 scales given separately
+ *      (gemm.cpp:311-344); low nibble = even element ---- */
+int orc_gemm_mxfp4_ref(const float* a, const uint8_t* w, const uint8_t* s, float* c, size_t m,
+                       size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0 || k % MX_BLOCK != 0) return ORC_INVALID_ARGUMENT;
+  const size_t nb = k / MX_BLOCK;
+  for (size_t i = 0; i < m; ++i) {
+    for (size_t j = 0; j < n; ++j) {
+      float acc = 0.0f;
+      for (size_t b = 0; b < nb; ++b) {
+        const float sc = orc_e8m0_to_float(s[j * nb + b]);
+        for (size_t l = 0; l < MX_BLOCK; ++l) {
+          const size_t t = b * MX_BLOCK + l;
+          const uint8_t byte = w[(j * k + t) / 2];
+          const uint8_t nib = (t % 2 == 0) ? (byte & 15u) : (byte >> 4);
+          acc = fmaf(a[i * k + t], sc * orc_f4e2m1_to_float(nib), acc);
+        }
+      }
+      c[i * n + j] = acc;
+    }
+  }
+  return ORC_OK;
+}
+
+/* MXFP4 weights -> fp32, n x k, from the packed device layout (blob then scales,
+ * include/tessera/backend.hpp:195-201). */
+int orc_dequantize_mxfp4(const uint8_t* packed, float* out, size_t n, size_t k) {
+  if (n == 0 || k == 0 || k % MX_BLOCK != 0) return ORC_INVALID_ARGUMENT;
+  const uint8_t* s = packed + n * k / 2;
+  const size_t nb = k / MX_BLOCK;
+  for (size_t j = 0; j < n; ++j) {
+    for (size_t t = 0; t < k; ++t) {
+      const uint8_t byte = packed[(j * k + t) / 2];
+      const uint8_t nib = (t % 2 == 0) ? (byte & 15u) : (byte >> 4);
+      out[j * k + t] = orc_e8m0_to_float(s[j * nb + t / MX_BLOCK]) * orc_f4e2m1_to_float(nib);
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- C = A . (diag(s) W)^T, E4M3 weights with one fp32 scale per row
+ *      (gemm.cpp:253-277) ---- */
+int orc_gemm_fp8_ref(const float* a, const uint8_t* w, const float* s, float* c, size_t m,
+                     size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0) return ORC_INVALID_ARGUMENT;
+  for (size_t i = 0; i < m; ++i) {
+    for (size_t j = 0; j < n; ++j) {
+      const float sc = s[j];
+      float acc = 0.0f;
+      for (size_t t = 0; t < k; ++t) {
+        acc = fmaf(a[i * k + t], sc * orc_fp8_e4m3_to_float(w[j * k + t]), acc);
+      }
+      c[i * n + j] = acc;
+    }
+  }
+  return ORC_OK;
+}
+
+/* e4m3 byte of (E2M1 magnitude code mag) * 2^-d, derived from the encoder with
+ * round-to-nearest-even.  Agrees with the reference's literal table below except in
+ * three tie entries (the tests list them). */
+uint8_t orc_fold_entry_rne(unsigned d, unsigned mag) {
+  const float v = ldexpf(orc_f4e2m1_to_float((uint8_t)(mag & 7u)), -(int)d);
+  return orc_fp32_to_fp8_e4m3(v);
+}
+
+/* The reference's fold table as data (quant.cpp:846-863): entry [d][mag].  Where a
+ * scaled magnitude falls exactly between two e4m3 subnormals (1.5 units: [9][3],
+ * [10][5], [11][7]) the table holds the lower code, not the even one, so it cannot be
+ * regenerated from the encoder and is kept literally. */
+static const uint8_t kFoldTable[16][8] = {
+    {0x00, 0x30, 0x38, 0x3c, 0x40, 0x44, 0x48, 0x4c}, {0x00, 0x28, 0x30, 0x34, 0x38, 0x3c, 0x40, 0x44},
+    {0x00, 0x20, 0x28, 0x2c, 0x30, 0x34, 0x38, 0x3c}, {0x00, 0x18, 0x20, 0x24, 0x28, 0x2c, 0x30, 0x34},
+    {0x00, 0x10, 0x18, 0x1c, 0x20, 0x24, 0x28, 0x2c}, {0x00, 0x08, 0x10, 0x14, 0x18, 0x1c, 0x20, 0x24},
+    {0x00, 0x04, 0x08, 0x0c, 0x10, 0x14, 0x18, 0x1c}, {0x00, 0x02, 0x04, 0x06, 0x08, 0x0c, 0x10, 0x14},
+    {0x00, 0x01, 0x02, 0x03, 0x04, 0x06, 0x08, 0x0c}, {0x00, 0x00, 0x01, 0x01, 0x02, 0x03, 0x04, 0x06},
+    {0x00, 0x00, 0x00, 0x01, 0x01, 0x01, 0x02, 0x03}, {0x00, 0x00, 0x00, 0x00, 0x00, 0x01, 0x01, 0x01},
+    {0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x01}, {0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00},
+    {0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00}, {0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00, 0x00},
+};
+
+uint8_t orc_fold_entry(unsigned d, unsigned mag) { return kFoldTable[d & 15u][mag & 7u]; }
+
+/* ---- MXFP4 -> e4m3 bytes relative to the per-row max exponent
+ *      (quant.cpp:865-898) ---- */
+int orc_fold_mxfp4_to_fp8(const uint8_t* w, const uint8_t* s, uint8_t* out, uint8_t* wref,
+                          size_t rows, size_t cols) {
+  if (rows == 0 || cols == 0 || cols % MX_BLOCK != 0) return ORC_INVALID_ARGUMENT;
+  const size_t nb = cols / MX_BLOCK;
+  for (size_t r = 0; r < rows; ++r) {
+    uint8_t ref = 0;
+    for (size_t b = 0; b < nb; ++b) ref = s[r * nb + b] > ref ? s[r * nb + b] : ref;
+    wref[r] = ref;
+    for (size_t c = 0; c < cols; ++c) {
+      const uint8_t byte = w[(r * cols + c) / 2];
+      const uint8_t nib = (c % 2 == 0) ? (byte & 15u) : (byte >> 4);
+      int d = (int)ref - (int)s[r * nb + c / MX_BLOCK];
+      d = d < 0 ? 0 : (d > 15 ? 15 : d);
+      out[r * cols + c] = (uint8_t)(orc_fold_entry((unsigned)d, nib & 7u) | ((nib & 8u) ? 0x80u : 0u));
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- folded W4A8 GEMM: (sum fma(a8, w8)) * As[m] * 2^(wref-127)
+ *      (quant.cpp:900-924) ---- */
+int orc_gemm_mxfp4_fp8_ref(const uint8_t* a8, const float* as, const uint8_t* w8,
+                           const uint8_t* wref, float* c, size_t m, size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0) return ORC_INVALID_ARGUMENT;
+  for (size_t i = 0; i < m; ++i) {
+    for (size_t j = 0; j < n; ++j) {
+      const float ws = exp2f((float)wref[j] - 127.0f);
+      float acc = 0.0f;
+      for (size_t t = 0; t < k; ++t) {
+        acc = fmaf(orc_fp8_e4m3_to_float(a8[i * k + t]), orc_fp8_e4m3_to_float(w8[j * k + t]), acc);
+      }
+      c[i * n + j] = acc * as[i] * ws;
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- W4A8 with the lossless weight side: per-token E4M3 QDQ of the activation
+ *      (QuantizeFp8Ref) followed by GemmMxFp4Ref, computed from the packed codes:
+ *      a = e4m3(code) * As[i].  Equals orc_quantize_fp8_ref + orc_gemm_mxfp4_ref
+ *      bit for bit because the QDQ value is exactly that product. ---- */
+int orc_gemm_mxfp4_w4a8_ref(const uint8_t* a8, const float* as, const uint8_t* w,
+                            const uint8_t* s, float* c, size_t m, size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0 || k % MX_BLOCK != 0) return ORC_INVALID_ARGUMENT;
+  float* a = (float*)malloc(m * k * sizeof(float));
+  if (!a) return ORC_OOM;
+  for (size_t i = 0; i < m; ++i) {
+    for (size_t t = 0; t < k; ++t) a[i * k + t] = orc_fp8_e4m3_to_float(a8[i * k + t]) * as[i];
+  }
+  const int st = orc_gemm_mxfp4_ref(a, w, s, c, m, n, k);
+  free(a);
+  return st;
+}
+
+/* ---- router weights: softmax over the selected top-k logits
+ *      (src/backends/rocm/rocm_kernels_basic.cpp:1915-1926) ---- */
+void orc_moe_gate(const float* vals, float* wts, size_t top_k) {
+  float mx = -3.402823466e+38f;
+  for (size_t p = 0; p < top_k; ++p) mx = fmaxf(mx, vals[p]);
+  float sum = 0.0f;
+  for (size_t p = 0; p < top_k; ++p) sum += expf(vals[p] - mx);
+  for (size_t p = 0; p < top_k; ++p) wts[p] = expf(vals[p] - mx) / sum;
+}
+
+/* ---- top-k of one row by descending value; on equal values the lower column
+ *      wins (the reference kernel's exact tie order differs and depends on its
+ *      thread layout, src/backends/rocm/rocm_kernels_basic.cpp:3173-3243; the
+ *      generators assert tie-free inputs) ---- */
+void orc_top_k_row(const float* logits, size_t n, size_t top_k, uint32_t* ids, float* vals) {
+  for (size_t p = 0; p < top_k; ++p) {
+    size_t best = (size_t)-1;
+    for (size_t c = 0; c < n; ++c) {
+      int taken = 0;
+      for (size_t q = 0; q < p; ++q) taken |= (ids[q] == c);
+      if (taken) continue;
+      if (best == (size_t)-1 || logits[c] > logits[best]) best = c;
+    }
+    ids[p] = (uint32_t)best;
+    vals[p] = logits[best];
+  }
+}
+
+/* ---- one Q4_K expert on one token: down(silu(gate x) * (up x))
+ *      (moe_cpu.cpp:39-64) ---- */
+int orc_moe_expert_forward_q4k(const float* x, const uint8_t* gate, const uint8_t* up,
+                               const uint8_t* down, size_t hidden, size_t inter, float* out) {
+  if (hidden == 0 || inter == 0) return ORC_INVALID_ARGUMENT;
+  float* g = (float*)malloc(3 * inter * sizeof(float));
+  if (!g) return ORC_OOM;
+  float* u = g + inter;
+  float* phi = u + inter;
+  int st = orc_gemm_q4k_ref(x, gate, g, 1, inter, hidden);
+  if (st == ORC_OK) st = orc_gemm_q4k_ref(x, up, u, 1, inter, hidden);
+  if (st == ORC_OK) {
+    for (size_t j = 0; j < inter; ++j) phi[j] = (g[j] / (1.0f + expf(-g[j]))) * u[j];
+    st = orc_gemm_q4k_ref(phi, down, out, 1, hidden, inter);
+  }
+  free(g);
+  return st;
+}
+
+/* ---- routed sum over the selected experts of one token, slots in order:
+ *      acc[j] += sum_slot wts[slot] * expert(ids[slot])(x)[j]
+ *      (moe_cpu.cpp:66-129 with one partial per slot, which is what its thread
+ *      pool produces when it has at least top_k threads; the device kernel
+ *      src/backends/rocm/rocm_kernels_moe.cpp:51-79 sums slots the same way) ---- */
+int orc_moe_experts_forward_q4k(const float* x, const uint32_t* ids, const float* wts,
+                                size_t top_k, const uint8_t* gate, size_t gate_stride,
+                                const uint8_t* up, size_t up_stride, const uint8_t* down,
+                                size_t down_stride, size_t hidden, size_t inter, float* acc) {
+  float* out = (float*)malloc(hidden * sizeof(float));
+  float* sum = (float*)calloc(hidden, sizeof(float));
+  if (!out || !sum) {
+    free(out);
+    free(sum);
+    return ORC_OOM;
+  }
+  int st = ORC_OK;
+  for (size_t c = 0; c < top_k && st == ORC_OK; ++c) {
+    const size_t e = ids[c];
+    st = orc_moe_expert_forward_q4k(x, gate + e * gate_stride, up + e * up_stride,
+                                    down + e * down_stride, hidden, inter, out);
+    if (st != ORC_OK) break;
+    for (size_t j = 0; j < hidden; ++j) sum[j] += wts[c] * out[j];
+  }
+  if (st == ORC_OK) {
+    for (size_t j = 0; j < hidden; ++j) acc[j] += sum[j];
+  }
+  free(out);
+  free(sum);
+  return st;
+}
+
+/* Tokens of a batch spread over OpenMP threads; each token is the sequential
+ * routine above, so results do not depend on the thread count. */
+int orc_moe_batch_forward_q4k(const float* x, const uint32_t* ids, const float* wts, size_t rows,
+                              size_t top_k, const uint8_t* gate, size_t gate_stride,
+                              const uint8_t* up, size_t up_stride, const uint8_t* down,
+                              size_t down_stride, size_t hidden, size_t inter, float* out) {
+  int bad = 0;
+#pragma omp parallel for schedule(dynamic)
+  for (long long r = 0; r < (long long)rows; ++r) {
+    memset(out + (size_t)r * hidden, 0, hidden * sizeof(float));
+    const int st = orc_moe_experts_forward_q4k(
+        x + (size_t)r * hidden, ids + (size_t)r * top_k, wts + (size_t)r * top_k, top_k, gate,
+        gate_stride, up, up_stride, down, down_stride, hidden, inter, out + (size_t)r * hidden);
+    if (st != ORC_OK) {
+#pragma omp atomic write
+      bad = st;
+    }
+  }
+  return bad;
+}

@@ -1,0 +1,266 @@
+// Small kernels around the matmul path: split-K reduce, per-token E4M3 activation
+// quantization, MXFP4 row reference exponents, and fp32 dumps of the block decodes
+// (the bit-exact level of the parity tests).
+
+#include "qmm_device.hpp"
+#include "qmm_kernels.hpp"
+
+namespace qmm {
+namespace {
+
+constexpr float kE4M3Max = 448.0f;
+constexpr float kE4M3MinScale = 1.0f / (448.0f * 512.0f);
+
+// c[i] = sum_s part[s * total + i], s ascending ("gemm_vec_reduce",
+// src/backends/rocm/rocm_kernels_gemv.cpp:53-66; "gemm_mxfp4_wmma_reduce",
+// src/backends/rocm/rocm_kernels_basic.cpp:1497-1510).
+__global__ __launch_bounds__(256) void vec_reduce_kernel(const float* __restrict__ part,
+                                                         float* __restrict__ c, uint64_t total,
+                                                         uint64_t split) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float acc = 0.0f;
+  for (uint64_t s = 0; s < split; ++s) acc += part[s * total + i];
+  c[i] = acc;
+}
+
+__global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ dst, float value,
+                                                       uint64_t count) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) dst[i] = value;
+}
+
+// Workgroup-wide max of non-negative values; every thread returns it.
+__device__ __forceinline__ float block_max_256(float v, float* lds) {
+  v = wave_max(v);
+  if ((threadIdx.x & 63u) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float r = fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
+  __syncthreads();
+  return r;
+}
+
+__device__ __forceinline__ float e4m3_clamp_quotient(float x, float s) {
+  const float q = x / s;  // correctly rounded fp32 division, as on the host
+  return fminf(fmaxf(q, -kE4M3Max), kE4M3Max);
+}
+
+// Per-row dynamic E4M3 quantize-dequantize in place ("quantize_fp8",
+// include/tessera/backend.hpp:296-302; src/core/numerics/quant.cpp:180-205).
+// One workgroup per row.
+__global__ __launch_bounds__(256) void quantize_fp8_kernel(float* __restrict__ data,
+                                                           float* __restrict__ scale,
+                                                           uint64_t cols) {
+  __shared__ float lds[4];
+  float* row = data + static_cast<uint64_t>(blockIdx.x) * cols;
+  float amax = 0.0f;
+  for (uint64_t c = threadIdx.x; c < cols; c += 256) amax = fmaxf(amax, fabsf(row[c]));
+  amax = block_max_256(amax, lds);
+  const float s = fmaxf(amax / kE4M3Max, kE4M3MinScale);
+  if (threadIdx.x == 0) scale[blockIdx.x] = s;
+  for (uint64_t c = threadIdx.x; c < cols; c += 256) {
+    const uint32_t code = float_to_e4m3(e4m3_clamp_quotient(row[c], s));
+    row[c] = e4m3_to_float(code) * s;
+  }
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return bit_cast<float>(b << 16); }
+
+// Per-row dynamic E4M3 quantize to packed codes + scale ("quantize_fp8_pack",
+// "quantize_fp8_pack_rows"; include/tessera/backend.hpp:303-307;
+// src/core/numerics/quant.cpp:207-229).  cols is a multiple of 4; one workgroup per
+// row.  kBf16 = true reads bf16 activations instead of fp32 (same values, half the
+// bytes).
+template <bool kBf16>
+__global__ __launch_bounds__(256) void quantize_fp8_pack_kernel(const void* __restrict__ in,
+                                                                uint8_t* __restrict__ out,
+                                                                float* __restrict__ scale,
+                                                                uint64_t cols) {
+  __shared__ float lds[4];
+  const uint64_t quads = cols / 4;
+  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * cols;
+  auto load4 = [&](uint64_t q, float (&v)[4]) {
+    if constexpr (kBf16) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(in) + base + q * 4);
+      v[0] = bf16_bits_to_float(raw.x & 0xFFFFu);
+      v[1] = bf16_bits_to_float(raw.x >> 16);
+      v[2] = bf16_bits_to_float(raw.y & 0xFFFFu);
+      v[3] = bf16_bits_to_float(raw.y >> 16);
+    } else {
+      const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(in) + base + q * 4);
+      v[0] = raw.x, v[1] = raw.y, v[2] = raw.z, v[3] = raw.w;
+    }
+  };
+  float amax = 0.0f;
+  for (uint64_t q = threadIdx.x; q < quads; q += 256) {
+    float v[4];
+    load4(q, v);
+    amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v[0]), fabsf(v[1]))), fmaxf(fabsf(v[2]), fabsf(v[3])));
+  }
+  amax = block_max_256(amax, lds);
+  const float s = fmaxf(amax / kE4M3Max, kE4M3MinScale);
+  if (threadIdx.x == 0) scale[blockIdx.x] = s;
+  uint32_t* dst = reinterpret_cast<uint32_t*>(out + base);
+  for (uint64_t q = threadIdx.x; q < quads; q += 256) {
+    float v[4];
+    load4(q, v);
+    uint32_t word = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      word |= float_to_e4m3(e4m3_clamp_quotient(v[b], s)) << (8 * b);
+    }
+    dst[q] = word;
+  }
+}
+
+// wref[r] = max over the row's E8M0 block exponents ("mxfp4_row_ref",
+// src/backends/rocm/rocm_kernels_basic.cpp:1284-1303).  One wavefront per row.
+__global__ __launch_bounds__(256) void mxfp4_row_ref_kernel(const uint8_t* __restrict__ w,
+                                                            uint8_t* __restrict__ wref, uint64_t n,
+                                                            uint64_t k) {
+  const uint64_t r = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (r >= n) return;
+  const uint64_t blocks = k / 32;
+  const uint8_t* s = w + n * k / 2 + r * blocks;
+  uint32_t ref = 0;
+  for (uint64_t b = threadIdx.x & 63u; b < blocks; b += 64) ref = max(ref, static_cast<uint32_t>(s[b]));
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ref = max(ref, static_cast<uint32_t>(__shfl_xor(static_cast<int>(ref), off, kWave)));
+  if ((threadIdx.x & 63u) == 0) wref[r] = static_cast<uint8_t>(ref);
+}
+
+// fp32 dump of Q4_K blocks, one thread per 16-byte quant chunk (32 values).  Same
+// arithmetic as the reference decode (src/core/numerics/quant.cpp:656-675):
+// (d*sc)*q - dmin*mn with exact products and one rounding.
+__global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t* __restrict__ w,
+                                                          float* __restrict__ out,
+                                                          uint64_t nchunks) {
+  const uint64_t c = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (c >= nchunks) return;
+  const uint64_t blk = c >> 3;
+  const uint32_t j = static_cast<uint32_t>(c & 7u), g = j >> 1, h = j & 1u;
+  const uint8_t* base = w + blk * kQ4KBlockBytes;
+  const uint4 hd = load_u4(base);
+  const uint4 q = load_u4(base + 16 + j * 16);
+  const uint8_t* p = reinterpret_cast<const uint8_t*>(&hd) + 4;
+  auto scale_min = [&](uint32_t sb, uint32_t& sc, uint32_t& mn) {
+    if (sb < 4) {
+      sc = p[sb] & 63u;
+      mn = p[sb + 4] & 63u;
+    } else {
+      sc = (p[sb + 4] & 15u) | ((p[sb - 4] >> 6) << 4);
+      mn = (p[sb + 4] >> 4) | ((p[sb] >> 6) << 4);
+    }
+  };
+  uint32_t sca, mna, scb, mnb;
+  scale_min(2 * g, sca, mna);
+  scale_min(2 * g + 1, scb, mnb);
+  const float d = half_bits_to_float(hd.x & 0xFFFFu), dmin = half_bits_to_float(hd.x >> 16);
+  const float s0 = d * static_cast<float>(sca), o0 = dmin * static_cast<float>(mna);
+  const float s1 = d * static_cast<float>(scb), o1 = dmin * static_cast<float>(mnb);
+  float* dst = out + blk * kQ4KBlockElems + g * 64 + h * 16;
+  const uint8_t* qb = reinterpret_cast<const uint8_t*>(&q);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    dst[i] = s0 * static_cast<float>(qb[i] & 15u) - o0;
+    dst[32 + i] = s1 * static_cast<float>(qb[i] >> 4) - o1;
+  }
+}
+
+// fp32 dump of packed MXFP4 weights, one thread per 32-element block.
+__global__ __launch_bounds__(256) void dequant_mxfp4_kernel(const uint8_t* __restrict__ w,
+                                                            float* __restrict__ out,
+                                                            uint64_t nblocks, uint64_t blob_bytes) {
+  const uint64_t b = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (b >= nblocks) return;
+  const uint4 q = load_u4(w + b * 16);
+  const float scale = e8m0_to_float(w[blob_bytes + b]);
+  const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+  float* dst = out + b * 32;
+#pragma unroll
+  for (int wi = 0; wi < 4; ++wi) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      dst[wi * 8 + j] = scale * e2m1_to_float((qw[wi] >> (4 * j)) & 15u);
+    }
+  }
+}
+
+// o = a + f[idx] * b ("moe_scale_add", src/backends/rocm/rocm_kernels_basic.cpp:1932-1942).
+__global__ __launch_bounds__(256) void moe_scale_add_kernel(const float* __restrict__ a,
+                                                            const float* __restrict__ b,
+                                                            const float* __restrict__ f,
+                                                            float* __restrict__ o, uint64_t n,
+                                                            uint64_t idx) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) o[i] = a[i] + f[idx] * b[i];
+}
+
+inline dim3 grid_for(uint64_t count, uint32_t per_block) {
+  return dim3(static_cast<uint32_t>((count + per_block - 1) / per_block));
+}
+
+}  // namespace
+
+hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64_t split,
+                             hipStream_t stream) {
+  hipLaunchKernelGGL(vec_reduce_kernel, grid_for(total, 256), dim3(256), 0, stream, part, c, total,
+                     split);
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream) {
+  if (count == 0) return hipSuccess;
+  hipLaunchKernelGGL(fill_f32_kernel, grid_for(count, 256), dim3(256), 0, stream, dst, value, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_quantize_fp8(float* data, float* scale, uint64_t rows, uint64_t cols,
+                               hipStream_t stream) {
+  hipLaunchKernelGGL(quantize_fp8_kernel, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream,
+                     data, scale, cols);
+  return hipGetLastError();
+}
+
+hipError_t launch_quantize_fp8_pack(const float* in, uint8_t* out, float* scale, uint64_t rows,
+                                    uint64_t cols, hipStream_t stream) {
+  hipLaunchKernelGGL(quantize_fp8_pack_kernel<false>, dim3(static_cast<uint32_t>(rows)), dim3(256),
+                     0, stream, static_cast<const void*>(in), out, scale, cols);
+  return hipGetLastError();
+}
+
+hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float* scale,
+                                         uint64_t rows, uint64_t cols, hipStream_t stream) {
+  hipLaunchKernelGGL(quantize_fp8_pack_kernel<true>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0,
+                     stream, static_cast<const void*>(in), out, scale, cols);
+  return hipGetLastError();
+}
+
+hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uint64_t k,
+                                hipStream_t stream) {
+  hipLaunchKernelGGL(mxfp4_row_ref_kernel, grid_for(n, 4), dim3(256), 0, stream, w, wref, n, k);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant_q4k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream) {
+  hipLaunchKernelGGL(dequant_q4k_kernel, grid_for(nblocks * 8, 256), dim3(256), 0, stream, w, out,
+                     nblocks * 8);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant_mxfp4(const uint8_t* w, float* out, uint64_t n, uint64_t k,
+                                hipStream_t stream) {
+  const uint64_t nblocks = n * k / 32;
+  hipLaunchKernelGGL(dequant_mxfp4_kernel, grid_for(nblocks, 256), dim3(256), 0, stream, w, out,
+                     nblocks, n * k / 2);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_scale_add(const float* a, const float* b, const float* f, float* o,
+                                uint64_t n, uint64_t idx, hipStream_t stream) {
+  hipLaunchKernelGGL(moe_scale_add_kernel, grid_for(n, 256), dim3(256), 0, stream, a, b, f, o, n,
+                     idx);
+  return hipGetLastError();
+}
+
+}  // namespace qmm

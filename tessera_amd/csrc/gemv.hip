@@ -1,0 +1,708 @@
+// Decode-regime GEMV for block-quantized weights on gfx950 (wave64, no MFMA).
+//
+// C[r, j] = sum_t A[r, t] * deq(W)[j, t] for a handful of activation rows r.
+//
+// The weight stream is the cost (HBM-bound), so the mapping is built around it:
+//   * a row of W is cut into 16-byte "chunks"; thread t of a workgroup owns chunk
+//     (t mod chunks_per_row) of every weight row the workgroup visits, so one
+//     workgroup reads whole rows as contiguous 128-bit loads, row after row;
+//   * because a thread's position along K never changes, its slice of the
+//     activations is loaded once and lives in registers for the whole kernel (an
+//     LDS- or cache-fed activation would cost 8 bytes of on-chip traffic per weight
+//     byte and cap the kernel below the HBM rate);
+//   * each thread's partial dot products are reduced across the wavefront with
+//     cross-lane shuffles and across the wavefronts of the workgroup through a
+//     few floats of LDS, one barrier per U weight rows, in a fixed order
+//     (deterministic, no atomics).
+// Codecs plug the block format into this skeleton.
+
+#include "qmm_device.hpp"
+#include "qmm_kernels.hpp"
+
+namespace qmm {
+namespace {
+
+// ----------------------------------------------------------------------------
+// Q4_K: 144-byte super-block = fp16 d, fp16 dmin, 12 bytes of 6-bit scales/mins,
+// 128 quant bytes (reference layout: src/core/numerics/quant.hpp:11-15, decode
+// src/core/numerics/quant.cpp:58-70,656-675).  A chunk is 16 quant bytes: chunk j
+// of a block covers elements g*64 + h*16 + [0,16) in its low nibbles and the same
+// + 32 in its high nibbles (g = j / 2, h = j % 2), i.e. half of sub-blocks 2g and
+// 2g+1.
+//
+// sum_i x_i * (d*sc*q_i - dmin*mn) = (d*sc) * sum_i x_i q_i - (dmin*mn) * sum_i x_i,
+// and sum_i x_i is a per-thread constant, so the inner loop is one fma per nibble.
+// Nibbles are turned into floats without integer->float converts: a nibble masked in
+// place inside a 16-bit lane is the fp16 subnormal q * 2^-24 (or q * 2^-20 for a
+// nibble at bits 4..7), which v_fma_mix_f32 consumes directly; the power of two is
+// folded into d*sc, so the arithmetic stays exact where the reference's is.
+// ----------------------------------------------------------------------------
+struct Q4KCodec {
+  struct Args {
+    const float* a;
+    const uint8_t* w;
+    uint32_t k;
+  };
+  template <int R>
+  struct X {
+    float lo[R][16];
+    float hi[R][16];
+    float slo[R];
+    float shi[R];
+    uint32_t g;
+  };
+  struct Frag {
+    uint4 q;
+    uint4 h;
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
+
+  template <int R>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+    const uint32_t blk = chunk >> 3, j = chunk & 7u;
+    x.g = j >> 1;
+    const uint32_t k0 = blk * 256u + (j >> 1) * 64u + (j & 1u) * 16u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float* src = p.a + static_cast<size_t>(r) * p.k + k0;
+      float sl = 0.0f, sh = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 16; i += 4) {
+        const float4 lo = *reinterpret_cast<const float4*>(src + i);
+        const float4 hi = *reinterpret_cast<const float4*>(src + 32 + i);
+        x.lo[r][i] = lo.x, x.lo[r][i + 1] = lo.y, x.lo[r][i + 2] = lo.z, x.lo[r][i + 3] = lo.w;
+        x.hi[r][i] = hi.x, x.hi[r][i + 1] = hi.y, x.hi[r][i + 2] = hi.z, x.hi[r][i + 3] = hi.w;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sl += x.lo[r][i];
+        sh += x.hi[r][i];
+      }
+      x.slo[r] = sl;
+      x.shi[r] = sh;
+    }
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
+                                              uint32_t chunk, Frag& f) {
+    const uint8_t* blk = p.w + (static_cast<size_t>(row) * (cpr >> 3) + (chunk >> 3)) * 144u;
+    f.h = load_u4(blk);
+    f.q = load_u4(blk + 16u + (chunk & 7u) * 16u);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    // 6-bit scale/min of sub-blocks 2g and 2g+1 from the 12 packed bytes.
+    const uint32_t s0 = f.h.y, s1 = f.h.z, s2 = f.h.w;
+    const uint32_t sh = (x.g & 1u) * 16u;
+    uint32_t sca, scb, mna, mnb;
+    if (x.g < 2u) {
+      sca = (s0 >> sh) & 63u;
+      scb = (s0 >> (sh + 8u)) & 63u;
+      mna = (s1 >> sh) & 63u;
+      mnb = (s1 >> (sh + 8u)) & 63u;
+    } else {
+      sca = ((s2 >> sh) & 15u) | (((s0 >> (sh + 6u)) & 3u) << 4);
+      scb = ((s2 >> (sh + 8u)) & 15u) | (((s0 >> (sh + 14u)) & 3u) << 4);
+      mna = ((s2 >> (sh + 4u)) & 15u) | (((s1 >> (sh + 6u)) & 3u) << 4);
+      mnb = ((s2 >> (sh + 12u)) & 15u) | (((s1 >> (sh + 14u)) & 3u) << 4);
+    }
+    const float d = half_bits_to_float(f.h.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(f.h.x >> 16);
+    // 2^24 and 2^20 undo the fp16-subnormal encoding of the nibbles (exact).
+    const float dsa = d * static_cast<float>(sca) * 0x1p24f;
+    const float dsb = d * static_cast<float>(scb) * 0x1p20f;
+    const float dma = dmin * static_cast<float>(mna);
+    const float dmb = dmin * static_cast<float>(mnb);
+    const uint32_t qw[4] = {f.q.x, f.q.y, f.q.z, f.q.w};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float al0 = 0.0f, al1 = 0.0f, ah0 = 0.0f, ah1 = 0.0f;
+#pragma unroll
+      for (int wi = 0; wi < 4; ++wi) {
+        const uint32_t w = qw[wi], w8 = w >> 8;
+        const half2_t l02 = bit_cast<half2_t>(w & 0x000F000Fu);   // bytes 0,2 low nibbles
+        const half2_t h02 = bit_cast<half2_t>(w & 0x00F000F0u);   // bytes 0,2 high nibbles * 16
+        const half2_t l13 = bit_cast<half2_t>(w8 & 0x000F000Fu);  // bytes 1,3 low nibbles
+        const half2_t h13 = bit_cast<half2_t>(w8 & 0x00F000F0u);  // bytes 1,3 high nibbles * 16
+        al0 = fmaf(x.lo[r][4 * wi + 0], static_cast<float>(l02[0]), al0);
+        al1 = fmaf(x.lo[r][4 * wi + 1], static_cast<float>(l13[0]), al1);
+        al0 = fmaf(x.lo[r][4 * wi + 2], static_cast<float>(l02[1]), al0);
+        al1 = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al1);
+        ah0 = fmaf(x.hi[r][4 * wi + 0], static_cast<float>(h02[0]), ah0);
+        ah1 = fmaf(x.hi[r][4 * wi + 1], static_cast<float>(h13[0]), ah1);
+        ah0 = fmaf(x.hi[r][4 * wi + 2], static_cast<float>(h02[1]), ah0);
+        ah1 = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah1);
+      }
+      float v = dsa * (al0 + al1) - dma * x.slo[r];
+      v += dsb * (ah0 + ah1) - dmb * x.shi[r];
+      out[r] = v;
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+
+// ----------------------------------------------------------------------------
+// MXFP4 with fp32 activations: packed buffer = n*k/2 nibble bytes (low nibble =
+// even element) then n*k/32 E8M0 bytes (include/tessera/backend.hpp:195-201;
+// src/core/numerics/gemm.cpp:311-344).  A 16-byte chunk is exactly one 32-element
+// block, so the E8M0 scale multiplies the chunk's partial sum once.
+// ----------------------------------------------------------------------------
+struct MxFp4Codec {
+  struct Args {
+    const float* a;
+    const uint8_t* w;
+    const uint8_t* s;  // w + n*k/2
+    uint32_t k;
+  };
+  template <int R>
+  struct X {
+    float v[R][32];
+  };
+  struct Frag {
+    uint4 q;
+    uint32_t s;
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
+
+  template <int R>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float* src = p.a + static_cast<size_t>(r) * p.k + chunk * 32u;
+#pragma unroll
+      for (int i = 0; i < 32; i += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(src + i);
+        x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
+      }
+    }
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
+                                              uint32_t chunk, Frag& f) {
+    const size_t c = static_cast<size_t>(row) * cpr + chunk;
+    f.q = load_u4(p.w + c * 16u);
+    f.s = p.s[c];
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const uint32_t qw[4] = {f.q.x, f.q.y, f.q.z, f.q.w};
+    float2_t wv[16];
+#pragma unroll
+    for (int wi = 0; wi < 4; ++wi) {
+      wv[4 * wi + 0] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[wi], 1.0f, 0);
+      wv[4 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[wi], 1.0f, 1);
+      wv[4 * wi + 2] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[wi], 1.0f, 2);
+      wv[4 * wi + 3] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[wi], 1.0f, 3);
+    }
+    const float scale = e8m0_to_float(f.s);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int b = 0; b < 16; ++b) {
+        a0 = fmaf(x.v[r][2 * b], wv[b][0], a0);
+        a1 = fmaf(x.v[r][2 * b + 1], wv[b][1], a1);
+      }
+      out[r] = (a0 + a1) * scale;
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+
+// ----------------------------------------------------------------------------
+// W4A8: MXFP4 weights, activations already quantized per token to E4M3 codes with
+// one fp32 scale per row (quantize_fp8_pack).  The weight side is lossless:
+// C[r, j] = As[r] * sum_b 2^(s_b - 127) * sum_{t in b} e4m3(a_t) * e2m1(w_t), which is
+// the reference's QuantizeFp8Ref followed by GemmMxFp4Ref
+// (src/core/numerics/quant.cpp:180-205, src/core/numerics/gemm.cpp:311-344) up to
+// summation order.  Both operands convert exactly to fp16 and v_dot2_f32_f16 takes
+// two products per instruction with fp32 accumulation.
+// ----------------------------------------------------------------------------
+struct MxFp4A8Codec {
+  struct Args {
+    const uint8_t* a;   // m x k e4m3 codes
+    const float* as;    // m per-row scales
+    const uint8_t* w;
+    const uint8_t* s;
+    uint32_t k;
+  };
+  template <int R>
+  struct X {
+    half2_t v[R][16];
+  };
+  struct Frag {
+    uint4 q;
+    uint32_t s;
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
+
+  template <int R>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint8_t* src = p.a + static_cast<size_t>(r) * p.k + chunk * 32u;
+      const uint4 c0 = load_u4(src), c1 = load_u4(src + 16);
+      const uint32_t cw[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x.v[r][2 * i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cw[i], 1.0f, false);
+        x.v[r][2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cw[i], 1.0f, true);
+      }
+    }
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
+                                              uint32_t chunk, Frag& f) {
+    const size_t c = static_cast<size_t>(row) * cpr + chunk;
+    f.q = load_u4(p.w + c * 16u);
+    f.s = p.s[c];
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const uint32_t qw[4] = {f.q.x, f.q.y, f.q.z, f.q.w};
+    half2_t wv[16];
+#pragma unroll
+    for (int wi = 0; wi < 4; ++wi) {
+      wv[4 * wi + 0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw[wi], 1.0f, 0);
+      wv[4 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw[wi], 1.0f, 1);
+      wv[4 * wi + 2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw[wi], 1.0f, 2);
+      wv[4 * wi + 3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw[wi], 1.0f, 3);
+    }
+    const float scale = e8m0_to_float(f.s);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int b = 0; b < 16; b += 2) {
+        a0 = __builtin_amdgcn_fdot2(wv[b], x.v[r][b], a0, false);
+        a1 = __builtin_amdgcn_fdot2(wv[b + 1], x.v[r][b + 1], a1, false);
+      }
+      out[r] = (a0 + a1) * scale;
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args& p, uint32_t, int r, float v) {
+    return v * p.as[r];
+  }
+};
+
+// ----------------------------------------------------------------------------
+// FP8 E4M3 weights (n x k bytes) with one fp32 scale per weight row
+// (include/tessera/backend.hpp:191-194; src/core/numerics/gemm.cpp:253-277).
+// A chunk is 16 weights; the row scale multiplies the finished dot product.
+// ----------------------------------------------------------------------------
+struct Fp8Codec {
+  struct Args {
+    const float* a;
+    const uint8_t* w;
+    const float* s;
+    uint32_t k;
+  };
+  template <int R>
+  struct X {
+    float v[R][16];
+  };
+  struct Frag {
+    uint4 q;
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 16u; }
+
+  template <int R>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float* src = p.a + static_cast<size_t>(r) * p.k + chunk * 16u;
+#pragma unroll
+      for (int i = 0; i < 16; i += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(src + i);
+        x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
+      }
+    }
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
+                                              uint32_t chunk, Frag& f) {
+    f.q = load_u4(p.w + (static_cast<size_t>(row) * cpr + chunk) * 16u);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const uint32_t qw[4] = {f.q.x, f.q.y, f.q.z, f.q.w};
+    float2_t wv[8];
+#pragma unroll
+    for (int wi = 0; wi < 4; ++wi) {
+      wv[2 * wi] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, false);
+      wv[2 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, true);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        a0 = fmaf(x.v[r][2 * b], wv[b][0], a0);
+        a1 = fmaf(x.v[r][2 * b + 1], wv[b][1], a1);
+      }
+      out[r] = a0 + a1;
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args& p, uint32_t row, int, float v) {
+    return v * p.s[row];
+  }
+};
+
+// ----------------------------------------------------------------------------
+// The skeleton.  P weight rows share one pass of the workgroup (P = 2 fills the
+// lanes when a row's chunk count is not a multiple of 64); U passes are in flight
+// between barriers.
+// ----------------------------------------------------------------------------
+template <class Codec, int R, int P, int U, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, float* __restrict__ c,
+                                                    uint32_t n, uint32_t cpr, uint32_t ldc) {
+  constexpr int kMaxWaves = MAXT / kWave;
+  __shared__ float red[2][U][P][R][kMaxWaves];
+
+  const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+  const uint32_t slots = P * cpr;
+  const bool valid = t < slots;
+  const uint32_t prow = (P > 1 && valid && t >= cpr) ? 1u : 0u;
+  const uint32_t chunk = valid ? t - prow * cpr : 0u;
+
+  typename Codec::template X<R> x;
+  Codec::template load_x<R>(args, chunk, x);
+
+  // Which of the P rows this wavefront's lanes belong to (at most two when cpr >= 64).
+  const uint32_t first_slot = wave * 64u;
+  const uint32_t last_slot = first_slot + 63u < slots ? first_slot + 63u : slots - 1u;
+  const uint32_t row_a = (P > 1 && first_slot >= cpr) ? 1u : 0u;
+  const uint32_t row_b = (P > 1 && last_slot >= cpr) ? 1u : 0u;
+  const bool two = row_a != row_b;
+
+  const uint32_t groups = (n + P - 1) / P;
+  const uint32_t per_iter = gridDim.x * U;
+  const uint32_t iters = (groups + per_iter - 1) / per_iter;
+
+  for (uint32_t it = 0; it < iters; ++it) {
+    const uint32_t buf = it & 1u;
+    typename Codec::Frag frag[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t grp = (it * U + u) * gridDim.x + blockIdx.x;
+      const uint32_t row = grp * P + prow;
+      ok[u] = valid && row < n;
+      if (ok[u]) {
+        Codec::load(args, row, cpr, chunk, frag[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float v[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) v[r] = 0.0f;
+      if (ok[u]) {
+        Codec::template dot<R>(frag[u], x, v);
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (P > 1 && two) {
+          const float sa = wave_sum(prow == row_a ? v[r] : 0.0f);
+          const float sb = wave_sum(prow == row_a ? 0.0f : v[r]);
+          if (lane == 0) {
+            red[buf][u][0][r][wave] = sa;
+            red[buf][u][P - 1][r][wave] = sb;
+          }
+        } else {
+          const float s = wave_sum(v[r]);
+          if (lane == 0) {
+            red[buf][u][row_a][r][wave] = s;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (t < U * P * R) {
+      const uint32_t u = t / (P * R), p = (t / R) % P, r = t % R;
+      const uint32_t grp = (it * U + u) * gridDim.x + blockIdx.x;
+      const uint32_t row = grp * P + p;
+      if (row < n) {
+        const uint32_t w_lo = (p * cpr) >> 6, w_hi = ((p + 1u) * cpr - 1u) >> 6;
+        float s = 0.0f;
+        for (uint32_t w = w_lo; w <= w_hi; ++w) {
+          s += red[buf][u][p][r][w];
+        }
+        c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, s);
+      }
+    }
+  }
+}
+
+// Small-K variant (a row has 8, 16 or 32 chunks): each wavefront owns 64 / cpr whole
+// rows per pass and reduces inside aligned lane groups, no LDS and no barrier.
+template <class Codec, int R, int U>
+__global__ __launch_bounds__(256) void gemv_smallk_kernel(typename Codec::Args args,
+                                                          float* __restrict__ c, uint32_t n,
+                                                          uint32_t cpr, uint32_t ldc) {
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t rows_per_wave = 64u / cpr;
+  const uint32_t chunk = lane % cpr, sub = lane / cpr;
+  typename Codec::template X<R> x;
+  Codec::template load_x<R>(args, chunk, x);
+  const uint32_t wave_global = blockIdx.x * (blockDim.x >> 6) + (t >> 6);
+  const uint32_t waves_total = gridDim.x * (blockDim.x >> 6);
+  const uint32_t groups = (n + rows_per_wave - 1) / rows_per_wave;
+  for (uint32_t g0 = wave_global; g0 < groups; g0 += waves_total * U) {
+    typename Codec::Frag frag[U];
+    bool ok[U];
+    uint32_t rows[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t grp = g0 + u * waves_total;
+      rows[u] = grp * rows_per_wave + sub;
+      ok[u] = grp < groups && rows[u] < n;
+      if (ok[u]) Codec::load(args, rows[u], cpr, chunk, frag[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float v[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) v[r] = 0.0f;
+      if (ok[u]) Codec::template dot<R>(frag[u], x, v);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float s = v[r];
+        for (uint32_t off = cpr >> 1; off > 0; off >>= 1) {
+          s += __shfl_xor(s, off, kWave);
+        }
+        if (ok[u] && chunk == 0) {
+          c[static_cast<size_t>(r) * ldc + rows[u]] = Codec::template finish<R>(args, rows[u], r, s);
+        }
+      }
+    }
+  }
+}
+
+struct GemvPlan {
+  uint32_t cpr;
+  uint32_t threads;  // workgroup size, multiple of 64
+  int p;             // weight rows per pass
+  bool smallk;
+};
+
+// Workgroup shape: the thread count that wastes the fewest lanes, preferring one
+// row per pass; two rows per pass when that fills the lanes better.
+GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads) {
+  GemvPlan g{cpr, 0, 1, false};
+  if (cpr == 8 || cpr == 16 || cpr == 32) {
+    g.smallk = true;
+    g.threads = 256;
+    return g;
+  }
+  const uint32_t t1 = (cpr + 63u) / 64u * 64u;
+  const uint32_t t2 = (2u * cpr + 63u) / 64u * 64u;
+  g.threads = t1;
+  if (cpr >= 64 && t2 <= max_threads && (t2 - 2u * cpr) * t1 < (t1 - cpr) * t2) {
+    g.p = 2;
+    g.threads = t2;
+  }
+  return g;
+}
+
+int g_num_cus = 256;
+
+template <class Codec, int R, int MAXT, int U>
+hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n, uint32_t k,
+                         uint32_t ldc, hipStream_t stream) {
+  const uint32_t cpr = Codec::chunks_per_row(k);
+  const GemvPlan g = plan_gemv(cpr, MAXT);
+  if (g.smallk) {
+    const uint32_t rows_per_wave = 64u / cpr;
+    const uint32_t groups = (n + rows_per_wave - 1) / rows_per_wave;
+    uint32_t grid = (groups + 4u * U - 1) / (4u * U);
+    const uint32_t cap = static_cast<uint32_t>(g_num_cus) * 8u;
+    grid = grid > cap ? cap : (grid == 0 ? 1 : grid);
+    hipLaunchKernelGGL((gemv_smallk_kernel<Codec, R, U>), dim3(grid), dim3(256), 0, stream, args, c,
+                       n, cpr, ldc);
+    return hipGetLastError();
+  }
+  if (g.threads > MAXT) {
+    return hipErrorInvalidValue;
+  }
+  // Resident workgroups per CU: 16 wavefronts (1024 threads) when the register
+  // budget of __launch_bounds__(MAXT) holds.
+  const uint32_t waves = g.threads / 64u;
+  const uint32_t waves_per_simd = 4u / ((MAXT / 64u + 3u) / 4u);  // 512 VGPRs / budget
+  uint32_t per_cu = (4u * (waves_per_simd == 0 ? 1u : waves_per_simd)) / waves;
+  if (per_cu == 0) per_cu = 1;
+  const uint32_t groups = (n + g.p - 1) / g.p;
+  uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu;
+  const uint32_t need = (groups + U - 1) / U;
+  if (grid > need) grid = need;
+  if (grid == 0) grid = 1;
+  if (g.p == 2) {
+    hipLaunchKernelGGL((gemv_kernel<Codec, R, 2, U, MAXT>), dim3(grid), dim3(g.threads), 0, stream,
+                       args, c, n, cpr, ldc);
+  } else {
+    hipLaunchKernelGGL((gemv_kernel<Codec, R, 1, U, MAXT>), dim3(grid), dim3(g.threads), 0, stream,
+                       args, c, n, cpr, ldc);
+  }
+  return hipGetLastError();
+}
+
+// Fallback for shapes the register-resident mapping does not cover (a row longer
+// than 1024 chunks): one wavefront per weight row, lanes stride over the chunks and
+// fetch their activations from memory each time.  Correct for any K the codec
+// accepts; not tuned.
+template <class Codec>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args args,
+                                                           float* __restrict__ c, uint32_t n,
+                                                           uint32_t cpr, uint32_t ldc) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= n) return;  // whole wavefront leaves together
+  float acc = 0.0f;
+  for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
+    typename Codec::template X<1> x;
+    typename Codec::Frag f;
+    Codec::template load_x<1>(args, chunk, x);
+    Codec::load(args, row, cpr, chunk, f);
+    float v[1];
+    Codec::template dot<1>(f, x, v);
+    acc += v[0];
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) c[row] = Codec::template finish<1>(args, row, 0, acc);
+  (void)ldc;
+}
+
+template <class Codec>
+hipError_t launch_gemv_generic(const typename Codec::Args& args, float* c, uint32_t n, uint32_t k,
+                               hipStream_t stream) {
+  const uint32_t cpr = Codec::chunks_per_row(k);
+  hipLaunchKernelGGL((gemv_generic_kernel<Codec>), dim3((n + 3u) / 4u), dim3(256), 0, stream, args,
+                     c, n, cpr, n);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+void set_num_cus(int cus) { g_num_cus = cus > 0 ? cus : 256; }
+
+// K limits of the register-resident mapping: one 16-byte chunk per thread, at most
+// 1024 threads per row.
+bool gemv_q4k_supported(uint64_t k) { return k % 256 == 0 && k / 32 <= 1024; }
+bool gemv_mxfp4_supported(uint64_t k) { return k % 32 == 0 && k / 32 <= 1024; }
+bool gemv_fp8_supported(uint64_t k) { return k % 16 == 0 && k / 16 <= 1024; }
+
+hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                           uint32_t k, hipStream_t stream) {
+  // Three or four activation rows per pass need 96-128 registers for the activations
+  // alone, which only fits workgroups of up to 576 threads (k <= 18432).
+  const bool wide = (k / 32u + 63u) / 64u * 64u <= 576u;
+  for (uint32_t r0 = 0; r0 < m;) {
+    const uint32_t left = m - r0;
+    Q4KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
+    float* out = c + static_cast<size_t>(r0) * n;
+    hipError_t e;
+    uint32_t took;
+    if (left >= 4 && wide) {
+      e = launch_gemv_r<Q4KCodec, 4, 576, 2>(args, out, n, k, n, stream), took = 4;
+    } else if (left == 3 && wide) {
+      e = launch_gemv_r<Q4KCodec, 3, 576, 2>(args, out, n, k, n, stream), took = 3;
+    } else if (left >= 2) {
+      e = launch_gemv_r<Q4KCodec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
+    } else {
+      e = launch_gemv_r<Q4KCodec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
+    }
+    if (e != hipSuccess) return e;
+    r0 += took;
+  }
+  return hipSuccess;
+}
+
+hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                             uint32_t k, hipStream_t stream) {
+  const uint8_t* s = w + static_cast<size_t>(n) * k / 2;
+  const bool wide = (k / 32u + 63u) / 64u * 64u <= 576u;
+  for (uint32_t r0 = 0; r0 < m;) {
+    const uint32_t left = m - r0;
+    MxFp4Codec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
+    float* out = c + static_cast<size_t>(r0) * n;
+    hipError_t e;
+    uint32_t took;
+    if (left >= 4 && wide) {
+      e = launch_gemv_r<MxFp4Codec, 4, 576, 2>(args, out, n, k, n, stream), took = 4;
+    } else if (left == 3 && wide) {
+      e = launch_gemv_r<MxFp4Codec, 3, 576, 2>(args, out, n, k, n, stream), took = 3;
+    } else if (left >= 2) {
+      e = launch_gemv_r<MxFp4Codec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
+    } else {
+      e = launch_gemv_r<MxFp4Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
+    }
+    if (e != hipSuccess) return e;
+    r0 += took;
+  }
+  return hipSuccess;
+}
+
+hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
+                                uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
+  const uint8_t* s = w + static_cast<size_t>(n) * k / 2;
+  for (uint32_t r0 = 0; r0 < m;) {
+    const uint32_t left = m - r0;
+    MxFp4A8Codec::Args args{a8 + static_cast<size_t>(r0) * k, as + r0, w, s, k};
+    float* out = c + static_cast<size_t>(r0) * n;
+    hipError_t e;
+    uint32_t took;
+    if (left >= 4) {
+      e = launch_gemv_r<MxFp4A8Codec, 4, 1024, 2>(args, out, n, k, n, stream), took = 4;
+    } else if (left >= 2) {
+      e = launch_gemv_r<MxFp4A8Codec, 2, 1024, 4>(args, out, n, k, n, stream), took = 2;
+    } else {
+      e = launch_gemv_r<MxFp4A8Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
+    }
+    if (e != hipSuccess) return e;
+    r0 += took;
+  }
+  return hipSuccess;
+}
+
+hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
+                           uint32_t n, uint32_t k, hipStream_t stream) {
+  for (uint32_t r0 = 0; r0 < m;) {
+    const uint32_t left = m - r0;
+    Fp8Codec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
+    float* out = c + static_cast<size_t>(r0) * n;
+    hipError_t e;
+    uint32_t took;
+    if (left >= 4) {
+      e = launch_gemv_r<Fp8Codec, 4, 1024, 2>(args, out, n, k, n, stream), took = 4;
+    } else if (left >= 2) {
+      e = launch_gemv_r<Fp8Codec, 2, 1024, 4>(args, out, n, k, n, stream), took = 2;
+    } else {
+      e = launch_gemv_r<Fp8Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
+    }
+    if (e != hipSuccess) return e;
+    r0 += took;
+  }
+  return hipSuccess;
+}
+
+}  // namespace qmm

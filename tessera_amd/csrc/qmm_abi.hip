@@ -1,0 +1,456 @@
+// C ABI of the kernel library: device bring-up, the built-in kernel table, launch
+// validation and per-id dispatch.  See include/tessera_qmm.h for the contract of each
+// entry point and the reference interface it stands behind.
+
+#include "../../include/tessera_qmm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "qmm_kernels.hpp"
+
+namespace {
+
+struct LaunchCtx {
+  void* const* buf;
+  const size_t* bytes;  // may be null: sizes unknown, skip size checks
+  size_t nbuf;
+  const uint64_t* sc;
+  size_t nsc;
+  hipStream_t stream;
+
+  template <class T>
+  T* ptr(size_t i) const { return static_cast<T*>(buf[i]); }
+  // Buffer i holds at least `need` bytes (or sizes were not given).
+  bool fits(size_t i, unsigned __int128 need) const {
+    return bytes == nullptr || static_cast<unsigned __int128>(bytes[i]) >= need;
+  }
+};
+
+using qmm_fn = qmm_status (*)(const LaunchCtx&);
+
+thread_local std::string g_last_error;
+thread_local int t_device = -1;  // device this thread last made current
+std::mutex g_init_mutex;
+int g_device = -1;
+std::string g_device_name;
+
+qmm_status map_hip(hipError_t e) {
+  if (e == hipSuccess) return QMM_OK;
+  g_last_error = hipGetErrorString(e);
+  // Same mapping as the reference backend (src/backends/rocm/rocm_backend.cpp:38-45).
+  if (e == hipErrorOutOfMemory) return QMM_OUT_OF_MEMORY;
+  if (e == hipErrorInvalidValue) return QMM_INVALID_ARGUMENT;
+  return QMM_DEVICE_ERROR;
+}
+
+qmm_status bad(const char* why) {
+  g_last_error = why;
+  return QMM_INVALID_ARGUMENT;
+}
+
+using u128 = unsigned __int128;
+constexpr uint64_t kMaxDim = 0x7FFFFFFFull;  // kernels index rows/cols with 32 bits
+
+bool counts(const LaunchCtx& c, size_t nbuf, size_t nsc) { return c.nbuf == nbuf && c.nsc == nsc; }
+
+bool dims_ok(uint64_t m, uint64_t n, uint64_t k) {
+  return m != 0 && n != 0 && k != 0 && m <= kMaxDim && n <= kMaxDim && k <= kMaxDim;
+}
+
+u128 q4k_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * (k / 256) * 144; }
+u128 mxfp4_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * k / 2 + static_cast<u128>(n) * k / 32; }
+
+// ---- Q4_K --------------------------------------------------------------------
+// Regime choice inside the Q4_K ids: the caller names an id by the reference's
+// regime table (src/models/qwen3_5/project.cpp:233-366); every Q4_K GEMM id has the
+// same buffers and m, n, k scalars, so each id accepts every m and picks the gfx950
+// kernel that fits it.
+qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
+                      uint64_t k, hipStream_t s) {
+  if (!qmm::gemv_q4k_supported(k)) {
+    g_last_error = "Q4_K: k above 32768 is not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  return map_hip(qmm::launch_q4k_gemv(a, w, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                      static_cast<uint32_t>(k), s));
+}
+
+// "gemm_q4k", "gemm_q4k_row", "gemm_q4k_batched", "gemm_q4k_wmma": buffers A, W, C;
+// scalars m, n, k (include/tessera/backend.hpp:153-161,207-209,397-415;
+// src/core/decode_internal.hpp:1484-1504).
+qmm_status run_gemm_q4k(const LaunchCtx& c) {
+  if (!counts(c, 3, 3)) return bad("gemm_q4k: expects 3 buffers and 3 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
+  if (!dims_ok(m, n, k) || k % 256 != 0) return bad("gemm_q4k: m, n, k must be non-zero and k a multiple of 256");
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, q4k_bytes(n, k)) ||
+      !c.fits(2, static_cast<u128>(m) * n * 4)) {
+    return bad("gemm_q4k: a buffer is smaller than m, n, k require");
+  }
+  return q4k_matmul(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k, c.stream);
+}
+
+// "gemm_q4k_vec" and "gemm_q4k_rows{R}": buffers A, W, C; scalars m, n, k, split
+// (src/backends/rocm/rocm_kernels_gemv.cpp:17-24,103-156).  C has `split` regions of
+// m*n floats whose sum is the result: region 0 receives the whole dot product and
+// regions 1..split-1 are zeroed, so "gemm_vec_reduce" over them yields the result.
+qmm_status run_gemm_q4k_split(const LaunchCtx& c, uint64_t rows_required) {
+  if (!counts(c, 3, 4)) return bad("gemm_q4k_vec/rows: expects 3 buffers and 4 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], split = c.sc[3];
+  if (!dims_ok(m, n, k) || k % 256 != 0) return bad("gemm_q4k_vec/rows: bad m, n, k");
+  if (rows_required != 0 && m != rows_required) return bad("gemm_q4k_rowsR: m must equal R");
+  if (split == 0 || split > 64 || (k / 256) % split != 0) return bad("gemm_q4k_vec/rows: split must divide k/256");
+  const u128 region = static_cast<u128>(m) * n * 4;
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, q4k_bytes(n, k)) || !c.fits(2, region * split)) {
+    return bad("gemm_q4k_vec/rows: a buffer is smaller than m, n, k, split require");
+  }
+  float* out = c.ptr<float>(2);
+  qmm_status st = q4k_matmul(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, m, n, k, c.stream);
+  if (st == QMM_OK && split > 1) {
+    st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
+  }
+  return st;
+}
+qmm_status run_gemm_q4k_vec(const LaunchCtx& c) { return run_gemm_q4k_split(c, 0); }
+qmm_status run_gemm_q4k_rows2(const LaunchCtx& c) { return run_gemm_q4k_split(c, 2); }
+qmm_status run_gemm_q4k_rows3(const LaunchCtx& c) { return run_gemm_q4k_split(c, 3); }
+qmm_status run_gemm_q4k_rows4(const LaunchCtx& c) { return run_gemm_q4k_split(c, 4); }
+qmm_status run_gemm_q4k_rows5(const LaunchCtx& c) { return run_gemm_q4k_split(c, 5); }
+
+// "gemm_vec_reduce" / "gemm_mxfp4_wmma_reduce": buffers part, c; scalars total, split.
+qmm_status run_vec_reduce(const LaunchCtx& c) {
+  if (!counts(c, 2, 2)) return bad("gemm_vec_reduce: expects 2 buffers and 2 scalars");
+  const uint64_t total = c.sc[0], split = c.sc[1];
+  if (total == 0 || split == 0 || total > (1ull << 40) || split > 4096) return bad("gemm_vec_reduce: bad total or split");
+  if (!c.fits(0, static_cast<u128>(total) * split * 4) || !c.fits(1, static_cast<u128>(total) * 4)) {
+    return bad("gemm_vec_reduce: a buffer is smaller than total, split require");
+  }
+  return map_hip(qmm::launch_vec_reduce(c.ptr<const float>(0), c.ptr<float>(1), total, split, c.stream));
+}
+
+// "dequant_q4k" (not a reference id): buffers W, Out (fp32); scalar nblocks.
+qmm_status run_dequant_q4k(const LaunchCtx& c) {
+  if (!counts(c, 2, 1)) return bad("dequant_q4k: expects 2 buffers and 1 scalar");
+  const uint64_t nb = c.sc[0];
+  if (nb == 0 || nb > (1ull << 32)) return bad("dequant_q4k: bad block count");
+  if (!c.fits(0, static_cast<u128>(nb) * 144) || !c.fits(1, static_cast<u128>(nb) * 1024)) {
+    return bad("dequant_q4k: a buffer is smaller than nblocks requires");
+  }
+  return map_hip(qmm::launch_dequant_q4k(c.ptr<const uint8_t>(0), c.ptr<float>(1), nb, c.stream));
+}
+
+// ---- MXFP4 / FP8 ---------------------------------------------------------------
+// "gemm_mxfp4", "gemm_mxfp4_rows", "gemm_mxfp4_batched": buffers A, W, C; scalars
+// m, n, k with k a multiple of 32 (include/tessera/backend.hpp:195-201,513-523;
+// src/backends/rocm/rocm_kernels_basic.cpp:1092-1214).
+qmm_status run_gemm_mxfp4(const LaunchCtx& c) {
+  if (!counts(c, 3, 3)) return bad("gemm_mxfp4: expects 3 buffers and 3 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
+  if (!dims_ok(m, n, k) || k % 32 != 0) return bad("gemm_mxfp4: m, n, k must be non-zero and k a multiple of 32");
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, mxfp4_bytes(n, k)) ||
+      !c.fits(2, static_cast<u128>(m) * n * 4)) {
+    return bad("gemm_mxfp4: a buffer is smaller than m, n, k require");
+  }
+  if (!qmm::gemv_mxfp4_supported(k)) {
+    g_last_error = "MXFP4: k above 32768 is not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  return map_hip(qmm::launch_mxfp4_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2),
+                                        static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                        static_cast<uint32_t>(k), c.stream));
+}
+qmm_status run_gemm_mxfp4_rows(const LaunchCtx& c) {
+  if (c.nsc >= 1 && c.sc[0] > 16) return bad("gemm_mxfp4_rows: m must be 1..16");
+  return run_gemm_mxfp4(c);
+}
+
+// "mxfp4_row_ref": buffers W, Wref (n bytes); scalars n, k
+// (src/backends/rocm/rocm_kernels_basic.cpp:1284-1303).
+qmm_status run_mxfp4_row_ref(const LaunchCtx& c) {
+  if (!counts(c, 2, 2)) return bad("mxfp4_row_ref: expects 2 buffers and 2 scalars");
+  const uint64_t n = c.sc[0], k = c.sc[1];
+  if (!dims_ok(1, n, k) || k % 32 != 0) return bad("mxfp4_row_ref: bad n or k");
+  if (!c.fits(0, mxfp4_bytes(n, k)) || !c.fits(1, n)) return bad("mxfp4_row_ref: buffer too small");
+  return map_hip(qmm::launch_mxfp4_row_ref(c.ptr<const uint8_t>(0), c.ptr<uint8_t>(1), n, k, c.stream));
+}
+
+// "gemm_mxfp4_wmma": buffers A (m x k E4M3 codes), W (packed MXFP4), As (m fp32),
+// Wref (n bytes), C; scalars m, n, k, split, wperm
+// (src/backends/rocm/rocm_kernels_basic.cpp:1310-1493; src/models/qwen3_5/project.cpp:207-215).
+// gfx950 multiplies E2M1 by E4M3 natively, so the weights are not folded to E4M3 and
+// Wref is unused: the result is As[r] * sum_t e4m3(a_t) * 2^(s-127) * e2m1(w_t), which
+// equals the reference's folded result wherever its fold is exact.  Split regions as
+// for "gemm_q4k_vec".  wperm (pre-permuted weights) must be 0, as the reference
+// always passes.
+qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
+  if (!counts(c, 5, 5)) return bad("gemm_mxfp4_wmma: expects 5 buffers and 5 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], split = c.sc[3], wperm = c.sc[4];
+  if (!dims_ok(m, n, k) || k % 32 != 0) return bad("gemm_mxfp4_wmma: bad m, n, k");
+  if (split == 0 || split > 64) return bad("gemm_mxfp4_wmma: bad split");
+  if (wperm != 0) {
+    g_last_error = "gemm_mxfp4_wmma: pre-permuted weights are not supported";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  const u128 region = static_cast<u128>(m) * n * 4;
+  if (!c.fits(0, static_cast<u128>(m) * k) || !c.fits(1, mxfp4_bytes(n, k)) || !c.fits(2, m * 4) ||
+      !c.fits(3, n) || !c.fits(4, region * split)) {
+    return bad("gemm_mxfp4_wmma: a buffer is smaller than m, n, k, split require");
+  }
+  if (!qmm::gemv_mxfp4_supported(k)) {
+    g_last_error = "MXFP4: k above 32768 is not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  float* out = c.ptr<float>(4);
+  qmm_status st = map_hip(qmm::launch_mxfp4_a8_gemv(
+      c.ptr<const uint8_t>(0), c.ptr<const float>(2), c.ptr<const uint8_t>(1), out,
+      static_cast<uint32_t>(m), static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
+  if (st == QMM_OK && split > 1) {
+    st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
+  }
+  return st;
+}
+
+// "dequant_mxfp4" (not a reference id): buffers W (packed), Out (n x k fp32); scalars n, k.
+qmm_status run_dequant_mxfp4(const LaunchCtx& c) {
+  if (!counts(c, 2, 2)) return bad("dequant_mxfp4: expects 2 buffers and 2 scalars");
+  const uint64_t n = c.sc[0], k = c.sc[1];
+  if (!dims_ok(1, n, k) || k % 32 != 0) return bad("dequant_mxfp4: bad n or k");
+  if (!c.fits(0, mxfp4_bytes(n, k)) || !c.fits(1, static_cast<u128>(n) * k * 4)) return bad("dequant_mxfp4: buffer too small");
+  return map_hip(qmm::launch_dequant_mxfp4(c.ptr<const uint8_t>(0), c.ptr<float>(1), n, k, c.stream));
+}
+
+// "quantize_fp8": buffers data (rows x cols fp32, in place), scale; scalars rows, cols
+// (include/tessera/backend.hpp:296-302,715-722).
+qmm_status run_quantize_fp8(const LaunchCtx& c) {
+  if (!counts(c, 2, 2)) return bad("quantize_fp8: expects 2 buffers and 2 scalars");
+  const uint64_t rows = c.sc[0], cols = c.sc[1];
+  if (!dims_ok(rows, 1, cols)) return bad("quantize_fp8: rows and cols must be non-zero");
+  if (!c.fits(0, static_cast<u128>(rows) * cols * 4) || !c.fits(1, static_cast<u128>(rows) * 4)) return bad("quantize_fp8: buffer too small");
+  return map_hip(qmm::launch_quantize_fp8(c.ptr<float>(0), c.ptr<float>(1), rows, cols, c.stream));
+}
+
+// "quantize_fp8_pack" / "quantize_fp8_pack_rows": buffers In (fp32), Out (codes), scale;
+// scalars rows, cols with cols a multiple of 4 (include/tessera/backend.hpp:303-307,723-730).
+qmm_status run_quantize_fp8_pack(const LaunchCtx& c) {
+  if (!counts(c, 3, 2)) return bad("quantize_fp8_pack: expects 3 buffers and 2 scalars");
+  const uint64_t rows = c.sc[0], cols = c.sc[1];
+  if (!dims_ok(rows, 1, cols) || cols % 4 != 0) return bad("quantize_fp8_pack: cols must be a non-zero multiple of 4");
+  if (!c.fits(0, static_cast<u128>(rows) * cols * 4) || !c.fits(1, static_cast<u128>(rows) * cols) ||
+      !c.fits(2, static_cast<u128>(rows) * 4)) {
+    return bad("quantize_fp8_pack: buffer too small");
+  }
+  return map_hip(qmm::launch_quantize_fp8_pack(c.ptr<const float>(0), c.ptr<uint8_t>(1), c.ptr<float>(2), rows, cols, c.stream));
+}
+
+// "quantize_fp8_pack_a16" (not a reference id): as "quantize_fp8_pack" with bf16 input.
+qmm_status run_quantize_fp8_pack_a16(const LaunchCtx& c) {
+  if (!counts(c, 3, 2)) return bad("quantize_fp8_pack_a16: expects 3 buffers and 2 scalars");
+  const uint64_t rows = c.sc[0], cols = c.sc[1];
+  if (!dims_ok(rows, 1, cols) || cols % 4 != 0) return bad("quantize_fp8_pack_a16: cols must be a non-zero multiple of 4");
+  if (!c.fits(0, static_cast<u128>(rows) * cols * 2) || !c.fits(1, static_cast<u128>(rows) * cols) ||
+      !c.fits(2, static_cast<u128>(rows) * 4)) {
+    return bad("quantize_fp8_pack_a16: buffer too small");
+  }
+  return map_hip(qmm::launch_quantize_fp8_pack_bf16(c.ptr<const uint16_t>(0), c.ptr<uint8_t>(1), c.ptr<float>(2), rows, cols, c.stream));
+}
+
+// "gemm_fp8": buffers A, W (n x k E4M3 bytes), S (n fp32), C; scalars m, n, k
+// (include/tessera/backend.hpp:191-194,504-512).
+qmm_status run_gemm_fp8(const LaunchCtx& c) {
+  if (!counts(c, 4, 3)) return bad("gemm_fp8: expects 4 buffers and 3 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
+  if (!dims_ok(m, n, k)) return bad("gemm_fp8: m, n, k must be non-zero");
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, static_cast<u128>(n) * k) ||
+      !c.fits(2, static_cast<u128>(n) * 4) || !c.fits(3, static_cast<u128>(m) * n * 4)) {
+    return bad("gemm_fp8: a buffer is smaller than m, n, k require");
+  }
+  if (!qmm::gemv_fp8_supported(k)) {
+    g_last_error = "gemm_fp8: k must be a multiple of 16 and at most 16384";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  return map_hip(qmm::launch_fp8_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
+                                      c.ptr<float>(3), static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                      static_cast<uint32_t>(k), c.stream));
+}
+
+// "moe_scale_add": buffers a, b, f, o; scalars n, idx
+// (src/backends/rocm/rocm_kernels_basic.cpp:1932-1942).
+qmm_status run_moe_scale_add(const LaunchCtx& c) {
+  if (!counts(c, 4, 2)) return bad("moe_scale_add: expects 4 buffers and 2 scalars");
+  const uint64_t n = c.sc[0], idx = c.sc[1];
+  if (n == 0 || n > (1ull << 40)) return bad("moe_scale_add: bad n");
+  if (!c.fits(0, static_cast<u128>(n) * 4) || !c.fits(1, static_cast<u128>(n) * 4) ||
+      !c.fits(2, (static_cast<u128>(idx) + 1) * 4) || !c.fits(3, static_cast<u128>(n) * 4)) {
+    return bad("moe_scale_add: buffer too small");
+  }
+  return map_hip(qmm::launch_moe_scale_add(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<const float>(2),
+                                           c.ptr<float>(3), n, idx, c.stream));
+}
+
+struct Entry {
+  const char* id;
+  qmm_fn fn;
+};
+
+const Entry kTable[] = {
+    {"gemm_q4k", run_gemm_q4k},
+    {"gemm_q4k_row", run_gemm_q4k},
+    {"gemm_q4k_batched", run_gemm_q4k},
+    {"gemm_q4k_wmma", run_gemm_q4k},
+    {"gemm_q4k_vec", run_gemm_q4k_vec},
+    {"gemm_q4k_rows2", run_gemm_q4k_rows2},
+    {"gemm_q4k_rows3", run_gemm_q4k_rows3},
+    {"gemm_q4k_rows4", run_gemm_q4k_rows4},
+    {"gemm_q4k_rows5", run_gemm_q4k_rows5},
+    {"gemm_vec_reduce", run_vec_reduce},
+    {"gemm_mxfp4", run_gemm_mxfp4},
+    {"gemm_mxfp4_rows", run_gemm_mxfp4_rows},
+    {"gemm_mxfp4_batched", run_gemm_mxfp4},
+    {"mxfp4_row_ref", run_mxfp4_row_ref},
+    {"gemm_mxfp4_wmma", run_gemm_mxfp4_wmma},
+    {"gemm_mxfp4_wmma_reduce", run_vec_reduce},
+    {"quantize_fp8", run_quantize_fp8},
+    {"quantize_fp8_pack", run_quantize_fp8_pack},
+    {"quantize_fp8_pack_rows", run_quantize_fp8_pack},
+    {"gemm_fp8", run_gemm_fp8},
+    {"moe_scale_add", run_moe_scale_add},
+    {"dequant_q4k", run_dequant_q4k},
+    {"dequant_mxfp4", run_dequant_mxfp4},
+    {"quantize_fp8_pack_a16", run_quantize_fp8_pack_a16},
+};
+constexpr size_t kTableSize = sizeof(kTable) / sizeof(kTable[0]);
+
+}  // namespace
+
+extern "C" {
+
+qmm_status qmm_init(int device) {
+  std::lock_guard<std::mutex> lock(g_init_mutex);
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess) return map_hip(e) == QMM_INVALID_ARGUMENT ? QMM_DEVICE_ERROR : map_hip(e);
+  if (device < 0 || device >= count) return bad("qmm_init: device index out of range");
+  if (g_device == device) return QMM_OK;
+  if ((e = hipSetDevice(device)) != hipSuccess) return map_hip(e);
+  hipDeviceProp_t prop;
+  if ((e = hipGetDeviceProperties(&prop, device)) != hipSuccess) return map_hip(e);
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    g_last_error = std::string("qmm_init: device is ") + prop.gcnArchName + ", this library holds gfx950 code only";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  g_device_name = prop.name;
+  qmm::set_num_cus(prop.multiProcessorCount);
+  g_device = device;
+  return QMM_OK;
+}
+
+const char* qmm_device_name(void) { return g_device_name.c_str(); }
+
+qmm_status qmm_memory_info(uint64_t* total_bytes, uint64_t* free_bytes) {
+  if (total_bytes == nullptr || free_bytes == nullptr) return bad("qmm_memory_info: null output");
+  size_t f = 0, t = 0;
+  const hipError_t e = hipMemGetInfo(&f, &t);
+  if (e != hipSuccess) return map_hip(e);
+  *total_bytes = t;
+  *free_bytes = f;
+  return QMM_OK;
+}
+
+qmm_status qmm_alloc(size_t bytes, void** out_device_ptr) {
+  if (bytes == 0 || out_device_ptr == nullptr) return bad("qmm_alloc: zero bytes or null output");
+  void* p = nullptr;
+  const hipError_t e = hipMalloc(&p, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return map_hip(e);
+  }
+  *out_device_ptr = p;
+  return QMM_OK;
+}
+
+qmm_status qmm_free(void* device_ptr) {
+  if (device_ptr == nullptr) return QMM_OK;
+  return map_hip(hipFree(device_ptr));
+}
+
+qmm_status qmm_copy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream) {
+  if (bytes == 0) return QMM_OK;
+  if (dst_device == nullptr || src_host == nullptr) return bad("qmm_copy_h2d: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  return map_hip(e);
+}
+
+qmm_status qmm_copy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream) {
+  if (bytes == 0) return QMM_OK;
+  if (dst_host == nullptr || src_device == nullptr) return bad("qmm_copy_d2h: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  return map_hip(e);
+}
+
+qmm_status qmm_copy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream) {
+  if (bytes == 0) return QMM_OK;
+  if (dst_device == nullptr || src_device == nullptr) return bad("qmm_copy_d2d: null pointer");
+  return map_hip(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice,
+                                static_cast<hipStream_t>(stream)));
+}
+
+qmm_status qmm_load(const char* id, qmm_kernel* out) {
+  if (id == nullptr || out == nullptr) return bad("qmm_load: null argument");
+  for (size_t i = 0; i < kTableSize; ++i) {
+    if (std::strcmp(kTable[i].id, id) == 0) {
+      *out = static_cast<qmm_kernel>(i + 1);
+      return QMM_OK;
+    }
+  }
+  *out = 0;
+  g_last_error = std::string("qmm_load: no built-in named ") + id;
+  return QMM_UNSUPPORTED_FEATURE;
+}
+
+const char* qmm_kernel_id(qmm_kernel kernel) {
+  return (kernel == 0 || kernel > kTableSize) ? nullptr : kTable[kernel - 1].id;
+}
+
+size_t qmm_kernel_count(void) { return kTableSize; }
+
+const char* qmm_kernel_name(size_t index) { return index < kTableSize ? kTable[index].id : nullptr; }
+
+qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                      void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
+                      const uint64_t* scalars, size_t nscalars, void* stream) {
+  if (kernel == 0 || kernel > kTableSize) return bad("qmm_launch: bad kernel handle");
+  if (grid == nullptr || block == nullptr) return bad("qmm_launch: null grid or block");
+  for (int i = 0; i < 3; ++i) {
+    if (grid[i] == 0 || block[i] == 0) return bad("qmm_launch: zero grid or block dimension");
+  }
+  if (nbuffers > QMM_MAX_BOUND_BUFFERS || nscalars > QMM_MAX_SCALARS) return bad("qmm_launch: too many buffers or scalars");
+  if ((nbuffers != 0 && buffers == nullptr) || (nscalars != 0 && scalars == nullptr)) return bad("qmm_launch: null argument array");
+  for (size_t i = 0; i < nbuffers; ++i) {
+    if (buffers[i] == nullptr) return bad("qmm_launch: null buffer");
+  }
+  if (g_device < 0) {
+    g_last_error = "qmm_launch: qmm_init has not succeeded";
+    return QMM_DEVICE_ERROR;
+  }
+  if (t_device != g_device) {  // callers may hop threads; HIP's current device is per thread
+    const hipError_t e = hipSetDevice(g_device);
+    if (e != hipSuccess) return map_hip(e);
+    t_device = g_device;
+  }
+  const LaunchCtx ctx{buffers, buf_bytes, nbuffers, scalars, nscalars, static_cast<hipStream_t>(stream)};
+  return kTable[kernel - 1].fn(ctx);
+}
+
+qmm_status qmm_sync(void* stream) { return map_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
+
+const char* qmm_last_error(void) { return g_last_error.c_str(); }
+
+}  // extern "C"

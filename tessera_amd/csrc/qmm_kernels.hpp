@@ -1,0 +1,51 @@
+// Host-callable launchers of the gfx950 kernels.  Every launcher enqueues on
+// `stream` and returns the HIP launch status; none allocates or synchronises.
+// Shapes are validated by the caller (qmm_abi.hip) before any of these runs.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace qmm {
+
+void set_num_cus(int cus);
+
+// ---- decode GEMV family (gemv.hip) -----------------------------------------
+bool gemv_q4k_supported(uint64_t k);
+bool gemv_mxfp4_supported(uint64_t k);
+bool gemv_fp8_supported(uint64_t k);
+
+// C (m x n fp32) = A (m x k fp32) . deq(W)^T, W = n rows of k/256 Q4_K blocks.
+hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                           uint32_t k, hipStream_t stream);
+// W = packed MXFP4 (n*k/2 nibble bytes, then n*k/32 E8M0 bytes).
+hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                             uint32_t k, hipStream_t stream);
+// A = m x k E4M3 codes with per-row scales `as`; W packed MXFP4; lossless weight side.
+hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
+                                uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
+// W = n x k E4M3 bytes, s = one fp32 scale per weight row.
+hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
+                           uint32_t n, uint32_t k, hipStream_t stream);
+
+// ---- element-wise helpers (elementwise.hip) ---------------------------------
+hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64_t split,
+                             hipStream_t stream);
+hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream);
+hipError_t launch_quantize_fp8(float* data, float* scale, uint64_t rows, uint64_t cols,
+                               hipStream_t stream);
+hipError_t launch_quantize_fp8_pack(const float* in, uint8_t* out, float* scale, uint64_t rows,
+                                    uint64_t cols, hipStream_t stream);
+hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float* scale,
+                                         uint64_t rows, uint64_t cols, hipStream_t stream);
+hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uint64_t k,
+                                hipStream_t stream);
+hipError_t launch_dequant_q4k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream);
+hipError_t launch_dequant_mxfp4(const uint8_t* w, float* out, uint64_t n, uint64_t k,
+                                hipStream_t stream);
+hipError_t launch_moe_scale_add(const float* a, const float* b, const float* f, float* o,
+                                uint64_t n, uint64_t idx, hipStream_t stream);
+
+}  // namespace qmm

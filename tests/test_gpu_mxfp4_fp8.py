@@ -1,0 +1,225 @@
+"""GPU parity of the MXFP4, W4A8 and FP8 paths against the CPU oracle, through the C ABI.
+
+Bit-exact: MXFP4 dequant (every E2M1 code under every E8M0 exponent), E4M3 codes and scales
+of the per-token activation quantizer.  Tolerance: GEMV outputs vs the oracle's sequential
+fp32 fma, max relative error 1e-3 (tests/util.py:rel_err); the W4A8 kernels multiply exact
+E4M3 x E2M1 products, so their error is summation order only and the same bound holds."""
+import numpy as np
+import pytest
+
+import oracle
+from tessera_amd import StatusCode, StatusError, synth
+from util import rel_err, run, same_bits, same_bits_zero_sign_free
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def mx_gemm(backend, name, a, w, m, n, k):
+    da, dw = backend.Upload(a), backend.Upload(w)
+    dc = backend.AllocateBuffer(4 * m * n)
+    run(backend, name, [da, dw, dc], [m, n, k], grid=((m * n + 7) // 8, 1, 1))
+    backend.Synchronize()
+    return backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
+
+
+def test_mxfp4_dequant_every_code_every_exponent(backend):
+    n, k = 256, 32 * 8
+    blob = np.tile(np.arange(256, dtype=np.uint8), n * k // 2 // 256 + 1)[: n * k // 2]
+    scales = np.repeat(np.arange(255, dtype=np.uint8), 9)[: n * k // 32]   # 0..254, no 0xFF
+    w = np.concatenate([blob, scales])
+    dw = backend.Upload(w)
+    out = backend.AllocateBuffer(4 * n * k)
+    run(backend, "dequant_mxfp4", [dw, out], [n, k])
+    backend.Synchronize()
+    got = backend.CopyD2H(out, dtype=np.float32).reshape(n, k)
+    assert same_bits(got, oracle.dequantize_mxfp4(w, n, k))
+
+
+@pytest.mark.parametrize("k", [256, 1024, 5120])
+def test_mxfp4_gemv_one_hot_reproduces_dequant(backend, k):
+    g = synth.rng(300 + k)
+    n = 80
+    w = synth.mxfp4_weights(g, n, k, -20, 20)
+    w[n * k // 2] = 0            # 2^-127, an fp32 subnormal
+    deq = oracle.dequantize_mxfp4(w, n, k)
+    pos = list(range(64)) + [int(t) for t in g.integers(0, k, 32)]
+    for r0 in range(0, len(pos), 4):
+        sel = pos[r0:r0 + 4]
+        c = mx_gemm(backend, "gemm_mxfp4_rows", synth.one_hot_rows(k, sel), w, len(sel), n, k)
+        for r, t in enumerate(sel):
+            assert same_bits_zero_sign_free(c[r], deq[:, t]), (k, t)
+
+
+MX_SHAPES = [(64, 256), (33, 512), (17, 96), (100, 1024), (129, 1280), (130, 5120), (67, 17408), (3, 32768)]
+
+
+@pytest.mark.parametrize("n,k", MX_SHAPES)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 16])
+def test_gemm_mxfp4_matches_oracle(backend, n, k, m):
+    if m > 4 and k > 8192:
+        pytest.skip("large-k multi-row cases are covered at m <= 4")
+    g = synth.rng(2000 * m + n + k)
+    w = synth.mxfp4_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_mxfp4(a, w, m, n, k)
+    name = "gemm_mxfp4" if m == 1 else "gemm_mxfp4_rows"
+    got = mx_gemm(backend, name, a, w, m, n, k)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
+def quant_inputs(g, rows, cols):
+    x = synth.activations_bf16_outliers(g, rows, cols)
+    if rows > 2:
+        x[1] = 0.0
+        x[2] *= 1e-9
+    return x
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 5120), (4, 5120), (16, 5120), (3, 100), (5, 17408), (2, 4)])
+def test_quantize_fp8_pack_bit_exact(backend, rows, cols):
+    g = synth.rng(rows * 131 + cols)
+    x = quant_inputs(g, rows, cols)
+    codes, scale = oracle.quantize_fp8_pack(x, rows, cols)
+    for name in ("quantize_fp8_pack", "quantize_fp8_pack_rows"):
+        dx = backend.Upload(x)
+        dq = backend.AllocateBuffer(rows * cols)
+        ds = backend.AllocateBuffer(4 * rows)
+        run(backend, name, [dx, dq, ds], [rows, cols], grid=(rows, 1, 1), block=(1024, 1, 1))
+        backend.Synchronize()
+        assert np.array_equal(backend.CopyD2H(dq).reshape(rows, cols), codes)
+        assert same_bits(backend.CopyD2H(ds, dtype=np.float32), scale)
+    # bf16 input carries the same values
+    dx16 = backend.Upload(synth.bf16_bits(x))
+    dq = backend.AllocateBuffer(rows * cols)
+    ds = backend.AllocateBuffer(4 * rows)
+    run(backend, "quantize_fp8_pack_a16", [dx16, dq, ds], [rows, cols])
+    backend.Synchronize()
+    assert np.array_equal(backend.CopyD2H(dq).reshape(rows, cols), codes)
+    assert same_bits(backend.CopyD2H(ds, dtype=np.float32), scale)
+
+
+def test_quantize_fp8_encoder_sweep_bit_exact(backend):
+    """The device E4M3 encoder against the oracle's on a dense sweep of fp32 inputs: every
+    rounding boundary of every binade from 2^-12 to 448, scaled so the row scale is exactly 1
+    (the row holds one 448)."""
+    vals = [oracle.fp8_e4m3_to_float(c) for c in range(0x7F)]
+    pts = []
+    for lo, hi in zip(vals[:-1], vals[1:]):
+        mid = np.float32((lo + hi) / 2)
+        pts += [lo, mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9)),
+                np.nextafter(np.float32(hi), np.float32(0))]
+    g = synth.rng(5)
+    pts = np.array(pts + list(g.uniform(0, 448, 20000)) + list(g.uniform(0, 2.0 ** -5, 20000)) +
+                   [448.0], dtype=np.float32)
+    x = np.concatenate([pts, -pts])
+    x = np.pad(x, (0, (-x.size) % 4)).reshape(1, -1)
+    cols = x.shape[1]
+    codes, scale = oracle.quantize_fp8_pack(x, 1, cols)
+    assert scale[0] == 1.0
+    dx = backend.Upload(x)
+    dq, ds = backend.AllocateBuffer(cols), backend.AllocateBuffer(4)
+    run(backend, "quantize_fp8_pack", [dx, dq, ds], [1, cols])
+    backend.Synchronize()
+    assert np.array_equal(backend.CopyD2H(dq).reshape(1, cols), codes)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 5120), (16, 5120), (3, 100), (4, 17408)])
+def test_quantize_fp8_qdq_bit_exact(backend, rows, cols):
+    g = synth.rng(rows * 17 + cols)
+    x = quant_inputs(g, rows, cols)
+    qdq, scale = oracle.quantize_fp8(x, rows, cols)
+    dx = backend.Upload(x)
+    ds = backend.AllocateBuffer(4 * rows)
+    run(backend, "quantize_fp8", [dx, ds], [rows, cols], grid=(rows, 1, 1))
+    backend.Synchronize()
+    assert same_bits(backend.CopyD2H(dx, dtype=np.float32).reshape(rows, cols), qdq)
+    assert same_bits(backend.CopyD2H(ds, dtype=np.float32), scale)
+
+
+@pytest.mark.parametrize("n,k", [(64, 256), (100, 1024), (130, 5120), (33, 17408)])
+@pytest.mark.parametrize("m,split", [(1, 1), (2, 1), (4, 2), (7, 1), (16, 4)])
+def test_w4a8_wmma_contract(backend, n, k, m, split):
+    """quantize_fp8_pack_rows -> mxfp4_row_ref -> gemm_mxfp4_wmma (-> reduce), the reference's
+    verify pipeline (src/models/qwen3_5/project.cpp:92-231), against QuantizeFp8Ref +
+    GemmMxFp4Ref."""
+    if m > 4 and k > 8192:
+        pytest.skip("large-k multi-row cases are covered at m <= 4")
+    g = synth.rng(3000 * m + n + k)
+    w = synth.mxfp4_weights(g, n, k, -8, -4)
+    x = synth.activations_bf16_outliers(g, m, k)
+    codes, scale = oracle.quantize_fp8_pack(x, m, k)
+    ref = oracle.gemm_mxfp4_w4a8(codes, scale, w, m, n, k)
+    dx, dw = backend.Upload(x), backend.Upload(w)
+    da8, das = backend.AllocateBuffer(m * k), backend.AllocateBuffer(4 * m)
+    dref = backend.AllocateBuffer(n)
+    part = backend.AllocateBuffer(4 * m * n * split)
+    out = backend.AllocateBuffer(4 * m * n)
+    run(backend, "quantize_fp8_pack_rows", [dx, da8, das], [m, k], grid=(m, 1, 1), block=(1024, 1, 1))
+    run(backend, "mxfp4_row_ref", [dw, dref], [n, k], grid=((n + 255) // 256, 1, 1))
+    run(backend, "gemm_mxfp4_wmma", [da8, dw, das, dref, part], [m, n, k, split, 0],
+        grid=((n + 63) // 64, split, 1), block=(128, 1, 1))
+    run(backend, "gemm_mxfp4_wmma_reduce", [part, out], [m * n, split], grid=((m * n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(out, dtype=np.float32).reshape(m, n)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    want_ref = w[n * k // 2:].reshape(n, -1).max(axis=1)
+    assert np.array_equal(backend.CopyD2H(dref), want_ref)
+    # and against the reference's folded arithmetic, which is exact at this exponent spread
+    w8, wref = oracle.fold_mxfp4_to_fp8(w, n, k)
+    folded = oracle.gemm_mxfp4_fp8(codes, scale, w8, wref, m, n, k)
+    assert rel_err(got, folded) <= TOL
+    with pytest.raises(StatusError) as e:   # pre-permuted weights are not part of this build
+        run(backend, "gemm_mxfp4_wmma", [da8, dw, das, dref, part], [m, n, k, split, 1])
+    assert e.value.code == StatusCode.UnsupportedFeature
+
+
+@pytest.mark.parametrize("n,k", [(64, 256), (100, 1008), (130, 5120), (40, 16384)])
+@pytest.mark.parametrize("m", [1, 2, 5])
+def test_gemm_fp8_matches_oracle(backend, n, k, m):
+    g = synth.rng(4000 * m + n + k)
+    codes, scales = synth.fp8_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_fp8(a, codes, scales, m, n, k)
+    da, dw, ds = backend.Upload(a), backend.Upload(codes), backend.Upload(scales)
+    dc = backend.AllocateBuffer(4 * m * n)
+    run(backend, "gemm_fp8", [da, dw, ds, dc], [m, n, k], grid=((m * n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
+def test_gemm_fp8_one_hot_bit_exact(backend):
+    g = synth.rng(77)
+    n, k = 50, 512
+    codes, scales = synth.fp8_weights(g, n, k)
+    pos = [0, 1, 15, 16, 17, 255, 511]
+    ref = oracle.gemm_fp8(synth.one_hot_rows(k, pos), codes, scales, len(pos), n, k)
+    da, dw, ds = backend.Upload(synth.one_hot_rows(k, pos)), backend.Upload(codes), backend.Upload(scales)
+    dc = backend.AllocateBuffer(4 * len(pos) * n)
+    run(backend, "gemm_fp8", [da, dw, ds, dc], [len(pos), n, k])
+    backend.Synchronize()
+    assert same_bits_zero_sign_free(backend.CopyD2H(dc, dtype=np.float32).reshape(len(pos), n), ref)
+
+
+def test_full_size_config2(backend):
+    """BASELINE config 2 at full size: N=17408, K=5120, M in {1, 4, 16}."""
+    g = synth.rng(9090)
+    n, k = 17408, 5120
+    w = synth.mxfp4_weights(g, n, k, -8, -4)
+    dw = backend.Upload(w)
+    dref = backend.AllocateBuffer(n)
+    for m in (1, 4, 16):
+        x = synth.activations_bf16_outliers(g, m, k)
+        codes, scale = oracle.quantize_fp8_pack(x, m, k)
+        dx = backend.Upload(x)
+        da8, das = backend.AllocateBuffer(m * k), backend.AllocateBuffer(4 * m)
+        out = backend.AllocateBuffer(4 * m * n)
+        run(backend, "quantize_fp8_pack_rows", [dx, da8, das], [m, k], grid=(m, 1, 1))
+        run(backend, "gemm_mxfp4_wmma", [da8, dw, das, dref, out], [m, n, k, 1, 0], grid=((n + 63) // 64, 1, 1))
+        backend.Synchronize()
+        assert np.array_equal(backend.CopyD2H(da8).reshape(m, k), codes)
+        got = backend.CopyD2H(out, dtype=np.float32).reshape(m, n)
+        rows = [0, m - 1] if m > 1 else [0]
+        ref = oracle.gemm_mxfp4_w4a8(codes[rows], scale[rows], w, len(rows), n, k)
+        assert rel_err(got[rows], ref) <= TOL, (m, rel_err(got[rows], ref))

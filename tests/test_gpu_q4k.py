@@ -1,0 +1,138 @@
+"""GPU parity of the Q4_K decode path against the CPU oracle, through the C ABI.
+
+Two levels (as the path's contract states): dequantized weights bit-exact against the
+reference block decode; GEMV outputs within max relative error 1e-3 of the reference's
+fp32 sequential-fma result (tests/util.py:rel_err is the metric; the kernels actually land
+near 1e-6, the bound is the contract's)."""
+import numpy as np
+import pytest
+
+import oracle
+from tessera_amd import StatusCode, StatusError, synth
+from util import ref_grid_vec, rel_err, run, same_bits, same_bits_zero_sign_free
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def gemm(backend, name, a, w, m, n, k, extra=()):
+    da, dw = backend.Upload(a), backend.Upload(w)
+    split = extra[0] if extra else 1
+    dc = backend.AllocateBuffer(4 * m * n * split)
+    run(backend, name, [da, dw, dc], [m, n, k, *extra], grid=ref_grid_vec(m, n))
+    backend.Synchronize()
+    return backend.CopyD2H(dc, dtype=np.float32).reshape(split, m, n)
+
+
+def test_dequant_dump_bit_exact_all_blocks(backend):
+    g = synth.rng(100)
+    n, k = 1024, 5120
+    w = synth.q4k_weights(g, n, k)
+    # edge blocks: all-zero, all-ones quants with extreme scales, negative d, fp16 subnormal d
+    blocks = w.reshape(-1, 144)
+    blocks[0] = 0
+    blocks[1, 4:16] = 0xFF
+    blocks[1, 16:] = 0xFF
+    blocks[2, 0:2] = np.array([-0.013], np.float16).view(np.uint8)
+    blocks[3, 0:2] = np.array([3e-6], np.float16).view(np.uint8)
+    nb = blocks.shape[0]
+    dw = backend.Upload(w)
+    out = backend.AllocateBuffer(nb * 1024)
+    run(backend, "dequant_q4k", [dw, out], [nb])
+    backend.Synchronize()
+    got = backend.CopyD2H(out, dtype=np.float32)
+    assert same_bits(got, oracle.dequantize_q4k(w))
+
+
+@pytest.mark.parametrize("k", [256, 512, 1024, 768, 2048, 5120])
+def test_gemv_one_hot_reproduces_dequant_bit_exact(backend, k):
+    """A one-hot activation makes the production GEMV return one column of deq(W): the
+    kernel's own decode (nibble extraction, scale unpack, d*sc*q - dmin*mn) is bit-exact."""
+    g = synth.rng(200 + k)
+    n = 96
+    w = synth.q4k_weights(g, n, k)
+    deq = oracle.dequantize_q4k(w).reshape(n, k)
+    # every position of the first block, then a spread over the rest of the row
+    pos = list(range(256)) + [int(t) for t in g.integers(0, k, 64)]
+    for r0 in range(0, len(pos), 4):
+        sel = pos[r0:r0 + 4]
+        c = gemm(backend, "gemm_q4k", synth.one_hot_rows(k, sel), w, len(sel), n, k)[0]
+        for r, t in enumerate(sel):
+            assert same_bits_zero_sign_free(c[r], deq[:, t]), (k, t)
+
+
+SHAPES = [(64, 256), (33, 512), (100, 1024), (17, 768), (129, 1280), (256, 2048), (130, 5120),
+          (67, 17408), (40, 4352), (1, 256), (5, 32768)]
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 7, 16])
+def test_gemm_q4k_matches_oracle(backend, n, k, m):
+    if m > 4 and k > 8192:
+        pytest.skip("large-k multi-row cases are covered at m <= 4")
+    g = synth.rng(1000 * m + n + k)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
+    for name in ("gemm_q4k", "gemm_q4k_batched") if m != 1 else ("gemm_q4k", "gemm_q4k_row"):
+        got = gemm(backend, name, a, w, m, n, k)[0]
+        assert rel_err(got, ref) <= TOL, (name, rel_err(got, ref))
+
+
+@pytest.mark.parametrize("n,k,split", [(640, 5120, 4), (5120, 5120, 4), (333, 2048, 2), (64, 17408, 4), (64, 256, 1)])
+def test_vec_split_contract_and_reduce(backend, n, k, split):
+    """gemm_q4k_vec writes `split` regions whose ordered sum gemm_vec_reduce returns
+    (src/models/qwen3_5/internal.hpp:104-145)."""
+    g = synth.rng(n + k + split)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, 1, k)
+    ref = oracle.gemm_q4k(a, w, 1, n, k, threads=True)
+    da, dw = backend.Upload(a), backend.Upload(w)
+    part = backend.AllocateBuffer(4 * n * split)
+    backend.CopyH2D(part, np.full(n * split, np.nan, np.float32))   # stale partials must not leak
+    out = backend.AllocateBuffer(4 * n)
+    run(backend, "gemm_q4k_vec", [da, dw, part], [1, n, k, split], grid=((n + 7) // 8, split, 1))
+    run(backend, "gemm_vec_reduce", [part, out], [n, split], grid=((n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(out, dtype=np.float32)
+    assert rel_err(got, ref) <= TOL
+    parts = backend.CopyD2H(part, dtype=np.float32).reshape(split, n)
+    assert np.array_equal(parts.sum(axis=0, dtype=np.float32), got)
+
+
+@pytest.mark.parametrize("rows", [2, 3, 4, 5])
+def test_rows_kernels(backend, rows):
+    g = synth.rng(rows)
+    n, k, split = 200, 2048, 2
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, rows, k)
+    ref = oracle.gemm_q4k(a, w, rows, n, k)
+    got = gemm(backend, f"gemm_q4k_rows{rows}", a, w, rows, n, k, extra=(split,))
+    assert rel_err(got.sum(axis=0), ref) <= TOL
+    with pytest.raises(StatusError) as e:          # the id fixes the row count
+        gemm(backend, f"gemm_q4k_rows{rows}", a[:1], w, 1, n, k, extra=(1,))
+    assert e.value.code == StatusCode.InvalidArgument
+
+
+def test_special_inputs(backend):
+    g = synth.rng(7)
+    n, k = 77, 1024
+    w = synth.q4k_weights(g, n, k)
+    assert np.all(gemm(backend, "gemm_q4k", np.zeros((1, k), np.float32), w, 1, n, k) == 0.0)
+    zero_w = np.zeros_like(w)
+    a = synth.activations_f32(g, 2, k)
+    assert np.all(gemm(backend, "gemm_q4k", a, zero_w, 2, n, k) == 0.0)
+
+
+def test_full_size_configs(backend):
+    """BASELINE configs 0 and 1 at full size: 5120x5120, 17408x5120 (gate/up), 5120x17408 (down)."""
+    for seed, (n, k) in enumerate([(5120, 5120), (17408, 5120), (5120, 17408)]):
+        g = synth.rng(4242 + seed)
+        w = synth.q4k_weights(g, n, k)
+        a = synth.activations_f32(g, 1, k)
+        ref = oracle.gemm_q4k(a, w, 1, n, k, threads=True)
+        got = gemm(backend, "gemm_q4k_vec", a, w, 1, n, k, extra=(1,))[0]
+        assert rel_err(got, ref) <= TOL, (n, k, rel_err(got, ref))
+        # linearity, a size-independent property: W(2a) == 2 W a exactly (power-of-two scaling)
+        got2 = gemm(backend, "gemm_q4k_vec", 2 * a, w, 1, n, k, extra=(1,))[0]
+        assert np.array_equal(got2, 2 * got)

@@ -1,0 +1,41 @@
+"""Shared helpers of the GPU parity tests."""
+import numpy as np
+
+from tessera_amd import KernelLaunch
+
+
+def rel_err(got: np.ndarray, ref: np.ndarray) -> float:
+    """max |got - ref| / max(|ref|, eps) with eps = 1e-3 * rms(ref), so that outputs that
+    cancel to (nearly) zero do not dominate the figure."""
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    eps = 1e-3 * np.sqrt(np.mean(ref * ref)) + 1e-30
+    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps)))
+
+
+def norm_err(got: np.ndarray, ref: np.ndarray) -> float:
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    return float(np.linalg.norm(got - ref) / (np.linalg.norm(ref) + 1e-30))
+
+
+def same_bits(a: np.ndarray, b: np.ndarray) -> bool:
+    return np.array_equal(np.ascontiguousarray(a, np.float32).view(np.uint32),
+                          np.ascontiguousarray(b, np.float32).view(np.uint32))
+
+
+def same_bits_zero_sign_free(a: np.ndarray, b: np.ndarray) -> bool:
+    """Bit equality except that -0 and +0 compare equal (a dot product starts from +0)."""
+    return same_bits(np.asarray(a, np.float32) + np.float32(0), np.asarray(b, np.float32) + np.float32(0))
+
+
+def run(backend, name, buffers, scalars, grid=(1, 1, 1), block=(256, 1, 1)):
+    k = backend.LoadKernel(name)
+    backend.LaunchKernel(k, KernelLaunch(grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                         list(buffers), list(scalars)))
+
+
+def ref_grid_vec(m, n):
+    """The reference's launch shape for the warp-per-output family
+    (src/core/decode_internal.hpp:896-901): ceil(m*n/8) workgroups of 256."""
+    return ((m * n + 7) // 8, 1, 1)

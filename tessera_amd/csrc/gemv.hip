@@ -22,6 +22,14 @@
 namespace qmm {
 namespace {
 
+// Per-thread byte offsets of a chunk relative to the (wavefront-uniform) start of a
+// row group; the uniform part goes through scalar registers, so a load is one
+// global_load with an SGPR base and a 32-bit VGPR offset.
+struct Lane {
+  uint32_t off0;
+  uint32_t off1;
+};
+
 // ----------------------------------------------------------------------------
 // Q4_K: 144-byte super-block = fp16 d, fp16 dmin, 12 bytes of 6-bit scales/mins,
 // 128 quant bytes (reference layout: src/core/numerics/quant.hpp:11-15, decode
@@ -30,12 +38,14 @@ namespace {
 // + 32 in its high nibbles (g = j / 2, h = j % 2), i.e. half of sub-blocks 2g and
 // 2g+1.
 //
-// sum_i x_i * (d*sc*q_i - dmin*mn) = (d*sc) * sum_i x_i q_i - (dmin*mn) * sum_i x_i,
+// sum_i x_i * (d*sc*q_i - dmin*mn) = d * sc * sum_i x_i q_i - dmin * mn * sum_i x_i,
 // and sum_i x_i is a per-thread constant, so the inner loop is one fma per nibble.
-// Nibbles are turned into floats without integer->float converts: a nibble masked in
-// place inside a 16-bit lane is the fp16 subnormal q * 2^-24 (or q * 2^-20 for a
-// nibble at bits 4..7), which v_fma_mix_f32 consumes directly; the power of two is
-// folded into d*sc, so the arithmetic stays exact where the reference's is.
+// Nibbles become floats without integer->float converts: a nibble masked in place
+// inside a 16-bit lane is the fp16 subnormal q * 2^-24 (q * 2^-20 for a nibble at
+// bits 4..7, for which the activation is pre-divided by 16), which v_fma_mix_f32
+// consumes directly; 2^24 is folded into d.  Every product that is exact in the
+// reference decode stays exact here, so a one-hot activation returns the reference's
+// dequantized weight bit for bit.
 // ----------------------------------------------------------------------------
 struct Q4KCodec {
   struct Args {
@@ -46,10 +56,12 @@ struct Q4KCodec {
   template <int R>
   struct X {
     float lo[R][16];
-    float hi[R][16];
+    float hi[R][16];  // activation / 16
     float slo[R];
     float shi[R];
-    uint32_t g;
+    uint32_t sh;      // 0 or 16: bit offset of the sub-block pair inside a scale word
+    uint32_t lm, hm;  // byte-pair masks: 0x3F3F / 0 for groups 0,1; 0x0F0F / 0x3030 for 2,3
+    bool upper;       // groups 2,3
   };
   struct Frag {
     uint4 q;
@@ -59,18 +71,22 @@ struct Q4KCodec {
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
 
   template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
-    const uint32_t blk = chunk >> 3, j = chunk & 7u;
-    x.g = j >> 1;
-    const uint32_t k0 = blk * 256u + (j >> 1) * 64u + (j & 1u) * 16u;
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
+    const uint32_t blk = chunk >> 3, j = chunk & 7u, g = j >> 1;
+    x.sh = (g & 1u) * 16u;
+    x.upper = g >= 2u;
+    x.lm = x.upper ? 0x0F0Fu : 0x3F3Fu;
+    x.hm = x.upper ? 0x3030u : 0u;
+    const uint32_t k0 = blk * 256u + g * 64u + (j & 1u) * 16u;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float* src = p.a + static_cast<size_t>(r) * p.k + k0;
       float sl = 0.0f, sh = 0.0f;
 #pragma unroll
       for (int i = 0; i < 16; i += 4) {
-        const float4 lo = *reinterpret_cast<const float4*>(src + i);
-        const float4 hi = *reinterpret_cast<const float4*>(src + 32 + i);
+        float4 lo = *reinterpret_cast<const float4*>(src + i);
+        float4 hi = *reinterpret_cast<const float4*>(src + 32 + i);
+        if (!valid) lo = hi = make_float4(0.f, 0.f, 0.f, 0.f);
         x.lo[r][i] = lo.x, x.lo[r][i + 1] = lo.y, x.lo[r][i + 2] = lo.z, x.lo[r][i + 3] = lo.w;
         x.hi[r][i] = hi.x, x.hi[r][i + 1] = hi.y, x.hi[r][i + 2] = hi.z, x.hi[r][i + 3] = hi.w;
       }
@@ -78,47 +94,45 @@ struct Q4KCodec {
       for (int i = 0; i < 16; ++i) {
         sl += x.lo[r][i];
         sh += x.hi[r][i];
+        x.hi[r][i] *= 0.0625f;
       }
       x.slo[r] = sl;
       x.shi[r] = sh;
     }
   }
 
-  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
-                                              uint32_t chunk, Frag& f) {
-    const uint8_t* blk = p.w + (static_cast<size_t>(row) * (cpr >> 3) + (chunk >> 3)) * 144u;
-    f.h = load_u4(blk);
-    f.q = load_u4(blk + 16u + (chunk & 7u) * 16u);
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t hdr = prow * (cpr >> 3) * 144u + (chunk >> 3) * 144u;
+    return Lane{hdr, hdr + 16u + (chunk & 7u) * 16u};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const uint8_t* base = p.w + static_cast<size_t>(row) * ((cpr >> 3) * 144u);
+    f.h = load_u4(base + ln.off0);
+    f.q = load_u4(base + ln.off1);
   }
 
   template <int R>
   static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
-    // 6-bit scale/min of sub-blocks 2g and 2g+1 from the 12 packed bytes.
+    // 6-bit scale/min of sub-blocks 2g and 2g+1, kept as byte pairs (2g in byte 0,
+    // 2g+1 in byte 1).  Groups 0,1 read six bits straight from bytes 2g, 2g+1 (+4 for
+    // the mins); groups 2,3 join a nibble of bytes 8.. with the top two bits of the
+    // bytes that groups 0,1 use.
     const uint32_t s0 = f.h.y, s1 = f.h.z, s2 = f.h.w;
-    const uint32_t sh = (x.g & 1u) * 16u;
-    uint32_t sca, scb, mna, mnb;
-    if (x.g < 2u) {
-      sca = (s0 >> sh) & 63u;
-      scb = (s0 >> (sh + 8u)) & 63u;
-      mna = (s1 >> sh) & 63u;
-      mnb = (s1 >> (sh + 8u)) & 63u;
-    } else {
-      sca = ((s2 >> sh) & 15u) | (((s0 >> (sh + 6u)) & 3u) << 4);
-      scb = ((s2 >> (sh + 8u)) & 15u) | (((s0 >> (sh + 14u)) & 3u) << 4);
-      mna = ((s2 >> (sh + 4u)) & 15u) | (((s1 >> (sh + 6u)) & 3u) << 4);
-      mnb = ((s2 >> (sh + 12u)) & 15u) | (((s1 >> (sh + 14u)) & 3u) << 4);
-    }
-    const float d = half_bits_to_float(f.h.x & 0xFFFFu);
+    const uint32_t ls = x.upper ? s2 : s0;
+    const uint32_t lmn = x.upper ? (s2 >> 4) : s1;
+    const uint32_t sc2 = ((ls >> x.sh) & x.lm) | ((s0 >> (x.sh + 2u)) & x.hm);
+    const uint32_t mn2 = ((lmn >> x.sh) & x.lm) | ((s1 >> (x.sh + 2u)) & x.hm);
+    const float sca = static_cast<float>(sc2 & 0xFFu), scb = static_cast<float>((sc2 >> 8) & 0xFFu);
+    const float mna = static_cast<float>(mn2 & 0xFFu), mnb = static_cast<float>((mn2 >> 8) & 0xFFu);
+    const float d24 = half_bits_to_float(f.h.x & 0xFFFFu) * 0x1p24f;  // undoes the 2^-24 below
     const float dmin = half_bits_to_float(f.h.x >> 16);
-    // 2^24 and 2^20 undo the fp16-subnormal encoding of the nibbles (exact).
-    const float dsa = d * static_cast<float>(sca) * 0x1p24f;
-    const float dsb = d * static_cast<float>(scb) * 0x1p20f;
-    const float dma = dmin * static_cast<float>(mna);
-    const float dmb = dmin * static_cast<float>(mnb);
     const uint32_t qw[4] = {f.q.x, f.q.y, f.q.z, f.q.w};
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      float al0 = 0.0f, al1 = 0.0f, ah0 = 0.0f, ah1 = 0.0f;
+      float al = 0.0f, ah = 0.0f;
 #pragma unroll
       for (int wi = 0; wi < 4; ++wi) {
         const uint32_t w = qw[wi], w8 = w >> 8;
@@ -126,18 +140,18 @@ struct Q4KCodec {
         const half2_t h02 = bit_cast<half2_t>(w & 0x00F000F0u);   // bytes 0,2 high nibbles * 16
         const half2_t l13 = bit_cast<half2_t>(w8 & 0x000F000Fu);  // bytes 1,3 low nibbles
         const half2_t h13 = bit_cast<half2_t>(w8 & 0x00F000F0u);  // bytes 1,3 high nibbles * 16
-        al0 = fmaf(x.lo[r][4 * wi + 0], static_cast<float>(l02[0]), al0);
-        al1 = fmaf(x.lo[r][4 * wi + 1], static_cast<float>(l13[0]), al1);
-        al0 = fmaf(x.lo[r][4 * wi + 2], static_cast<float>(l02[1]), al0);
-        al1 = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al1);
-        ah0 = fmaf(x.hi[r][4 * wi + 0], static_cast<float>(h02[0]), ah0);
-        ah1 = fmaf(x.hi[r][4 * wi + 1], static_cast<float>(h13[0]), ah1);
-        ah0 = fmaf(x.hi[r][4 * wi + 2], static_cast<float>(h02[1]), ah0);
-        ah1 = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah1);
+        al = fmaf(x.lo[r][4 * wi + 0], static_cast<float>(l02[0]), al);
+        ah = fmaf(x.hi[r][4 * wi + 0], static_cast<float>(h02[0]), ah);
+        al = fmaf(x.lo[r][4 * wi + 1], static_cast<float>(l13[0]), al);
+        ah = fmaf(x.hi[r][4 * wi + 1], static_cast<float>(h13[0]), ah);
+        al = fmaf(x.lo[r][4 * wi + 2], static_cast<float>(l02[1]), al);
+        ah = fmaf(x.hi[r][4 * wi + 2], static_cast<float>(h02[1]), ah);
+        al = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al);
+        ah = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah);
       }
-      float v = dsa * (al0 + al1) - dma * x.slo[r];
-      v += dsb * (ah0 + ah1) - dmb * x.shi[r];
-      out[r] = v;
+      const float t1 = fmaf(scb, ah, sca * al);
+      const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
+      out[r] = fmaf(d24, t1, -(dmin * t2));
     }
   }
 
@@ -172,23 +186,30 @@ struct MxFp4Codec {
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
 
   template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float* src = p.a + static_cast<size_t>(r) * p.k + chunk * 32u;
 #pragma unroll
       for (int i = 0; i < 32; i += 4) {
-        const float4 v = *reinterpret_cast<const float4*>(src + i);
+        float4 v = *reinterpret_cast<const float4*>(src + i);
+        if (!valid) v = make_float4(0.f, 0.f, 0.f, 0.f);
         x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
       }
     }
   }
 
-  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
-                                              uint32_t chunk, Frag& f) {
-    const size_t c = static_cast<size_t>(row) * cpr + chunk;
-    f.q = load_u4(p.w + c * 16u);
-    f.s = p.s[c];
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t c = prow * cpr + chunk;
+    return Lane{c * 16u, c};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const size_t c = static_cast<size_t>(row) * cpr;
+    f.q = load_u4(p.w + c * 16u + ln.off0);
+    f.s = (p.s + c)[ln.off1];
   }
 
   template <int R>
@@ -250,11 +271,12 @@ struct MxFp4A8Codec {
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
 
   template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const uint8_t* src = p.a + static_cast<size_t>(r) * p.k + chunk * 32u;
-      const uint4 c0 = load_u4(src), c1 = load_u4(src + 16);
+      uint4 c0 = load_u4(src), c1 = load_u4(src + 16);
+      if (!valid) c0 = c1 = make_uint4(0, 0, 0, 0);
       const uint32_t cw[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -264,11 +286,17 @@ struct MxFp4A8Codec {
     }
   }
 
-  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
-                                              uint32_t chunk, Frag& f) {
-    const size_t c = static_cast<size_t>(row) * cpr + chunk;
-    f.q = load_u4(p.w + c * 16u);
-    f.s = p.s[c];
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t c = prow * cpr + chunk;
+    return Lane{c * 16u, c};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const size_t c = static_cast<size_t>(row) * cpr;
+    f.q = load_u4(p.w + c * 16u + ln.off0);
+    f.s = (p.s + c)[ln.off1];
   }
 
   template <int R>
@@ -324,21 +352,27 @@ struct Fp8Codec {
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 16u; }
 
   template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, X<R>& x) {
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float* src = p.a + static_cast<size_t>(r) * p.k + chunk * 16u;
 #pragma unroll
       for (int i = 0; i < 16; i += 4) {
-        const float4 v = *reinterpret_cast<const float4*>(src + i);
+        float4 v = *reinterpret_cast<const float4*>(src + i);
+        if (!valid) v = make_float4(0.f, 0.f, 0.f, 0.f);
         x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
       }
     }
   }
 
-  static __device__ __forceinline__ void load(const Args& p, uint32_t row, uint32_t cpr,
-                                              uint32_t chunk, Frag& f) {
-    f.q = load_u4(p.w + (static_cast<size_t>(row) * cpr + chunk) * 16u);
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    return Lane{(prow * cpr + chunk) * 16u, 0u};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    f.q = load_u4(p.w + static_cast<size_t>(row) * cpr * 16u + ln.off0);
   }
 
   template <int R>
@@ -370,87 +404,94 @@ struct Fp8Codec {
 
 // ----------------------------------------------------------------------------
 // The skeleton.  P weight rows share one pass of the workgroup (P = 2 fills the
-// lanes when a row's chunk count is not a multiple of 64); U passes are in flight
-// between barriers.
+// lanes when a row's chunk count is not a multiple of 64).  Each thread keeps D row
+// fragments in registers as a software pipeline: fragment d is consumed and at once
+// refilled with the row D passes ahead, so D loads per thread stay in flight while the
+// arithmetic runs (about 100 KB outstanding per CU, what the HBM latency asks for).
+// One barrier per D passes publishes the per-wavefront partial sums.
 // ----------------------------------------------------------------------------
-template <class Codec, int R, int P, int U, int MAXT>
+template <class Codec, int R, int P, int D, int MAXT>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, float* __restrict__ c,
                                                     uint32_t n, uint32_t cpr, uint32_t ldc) {
   constexpr int kMaxWaves = MAXT / kWave;
-  __shared__ float red[2][U][P][R][kMaxWaves];
+  __shared__ float red[2][D][P][R][kMaxWaves];
 
-  const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t slots = P * cpr;
   const bool valid = t < slots;
   const uint32_t prow = (P > 1 && valid && t >= cpr) ? 1u : 0u;
   const uint32_t chunk = valid ? t - prow * cpr : 0u;
 
+  // Invalid lanes (past the last chunk) carry zero activations, so they add nothing.
   typename Codec::template X<R> x;
-  Codec::template load_x<R>(args, chunk, x);
+  Codec::template load_x<R>(args, chunk, valid, x);
 
   // Which of the P rows this wavefront's lanes belong to (at most two when cpr >= 64).
   const uint32_t first_slot = wave * 64u;
   const uint32_t last_slot = first_slot + 63u < slots ? first_slot + 63u : slots - 1u;
   const uint32_t row_a = (P > 1 && first_slot >= cpr) ? 1u : 0u;
   const uint32_t row_b = (P > 1 && last_slot >= cpr) ? 1u : 0u;
-  const bool two = row_a != row_b;
+  const bool two = row_a != row_b;  // wavefront-uniform
+  const float in_a = (prow == row_a) ? 1.0f : 0.0f, in_b = 1.0f - in_a;
 
+  // Work unit: a block of D consecutive row groups (D*P weight rows).  Groups past the
+  // end are clamped for the loads and dropped at the store; when n is odd and P = 2 the
+  // last group has no second row, so its lanes re-read the first one.
   const uint32_t groups = (n + P - 1) / P;
-  const uint32_t per_iter = gridDim.x * U;
-  const uint32_t iters = (groups + per_iter - 1) / per_iter;
+  const uint32_t nblocks = (groups + D - 1) / D;
+  const Lane ln = Codec::make_lane(args, cpr, chunk, prow);
+  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, 0u);
+  const bool ragged = (P > 1) && (n % P != 0);
+  auto fetch = [&](uint32_t blk, int d, typename Codec::Frag& f) {
+    uint32_t grp = blk * D + d;
+    grp = grp < groups ? grp : groups - 1u;
+    const bool tail = ragged && grp == groups - 1u;
+    Codec::load(args, tail ? ln_tail : ln, grp * P, cpr, f);
+  };
 
-  for (uint32_t it = 0; it < iters; ++it) {
-    const uint32_t buf = it & 1u;
-    typename Codec::Frag frag[U];
-    bool ok[U];
+  typename Codec::Frag frag[D];
+  uint32_t blk = blockIdx.x;
+  if (blk < nblocks) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t grp = (it * U + u) * gridDim.x + blockIdx.x;
-      const uint32_t row = grp * P + prow;
-      ok[u] = valid && row < n;
-      if (ok[u]) {
-        Codec::load(args, row, cpr, chunk, frag[u]);
-      }
-    }
+    for (int d = 0; d < D; ++d) fetch(blk, d, frag[d]);
+  }
+  uint32_t buf = 0;
+  for (; blk < nblocks; blk += gridDim.x) {
+    uint32_t nxt = blk + gridDim.x;
+    nxt = nxt < nblocks ? nxt : nblocks - 1u;  // the last refill re-reads, unused
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+    for (int d = 0; d < D; ++d) {
       float v[R];
-#pragma unroll
-      for (int r = 0; r < R; ++r) v[r] = 0.0f;
-      if (ok[u]) {
-        Codec::template dot<R>(frag[u], x, v);
-      }
+      Codec::template dot<R>(frag[d], x, v);
+      fetch(nxt, d, frag[d]);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (P > 1 && two) {
-          const float sa = wave_sum(prow == row_a ? v[r] : 0.0f);
-          const float sb = wave_sum(prow == row_a ? 0.0f : v[r]);
-          if (lane == 0) {
-            red[buf][u][0][r][wave] = sa;
-            red[buf][u][P - 1][r][wave] = sb;
+          const float sa = wave_sum_last(v[r] * in_a);
+          const float sb = wave_sum_last(v[r] * in_b);
+          if (lane == 63u) {
+            red[buf][d][0][r][wave] = sa;
+            red[buf][d][P - 1][r][wave] = sb;
           }
         } else {
-          const float s = wave_sum(v[r]);
-          if (lane == 0) {
-            red[buf][u][row_a][r][wave] = s;
-          }
+          const float sa = wave_sum_last(v[r]);
+          if (lane == 63u) red[buf][d][row_a][r][wave] = sa;
         }
       }
     }
     __syncthreads();
-    if (t < U * P * R) {
-      const uint32_t u = t / (P * R), p = (t / R) % P, r = t % R;
-      const uint32_t grp = (it * U + u) * gridDim.x + blockIdx.x;
-      const uint32_t row = grp * P + p;
+    if (t < D * P * R) {
+      const uint32_t d = t / (P * R), p = (t / R) % P, r = t % R;
+      const uint32_t row = (blk * D + d) * P + p;
       if (row < n) {
         const uint32_t w_lo = (p * cpr) >> 6, w_hi = ((p + 1u) * cpr - 1u) >> 6;
-        float s = 0.0f;
-        for (uint32_t w = w_lo; w <= w_hi; ++w) {
-          s += red[buf][u][p][r][w];
-        }
-        c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, s);
+        float sum = 0.0f;
+        for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][d][p][r][w];
+        c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, sum);
       }
     }
+    buf ^= 1u;
   }
 }
 
@@ -464,7 +505,8 @@ __global__ __launch_bounds__(256) void gemv_smallk_kernel(typename Codec::Args a
   const uint32_t rows_per_wave = 64u / cpr;
   const uint32_t chunk = lane % cpr, sub = lane / cpr;
   typename Codec::template X<R> x;
-  Codec::template load_x<R>(args, chunk, x);
+  Codec::template load_x<R>(args, chunk, true, x);
+  const Lane ln = Codec::make_lane(args, cpr, chunk, 0u);
   const uint32_t wave_global = blockIdx.x * (blockDim.x >> 6) + (t >> 6);
   const uint32_t waves_total = gridDim.x * (blockDim.x >> 6);
   const uint32_t groups = (n + rows_per_wave - 1) / rows_per_wave;
@@ -477,7 +519,7 @@ __global__ __launch_bounds__(256) void gemv_smallk_kernel(typename Codec::Args a
       const uint32_t grp = g0 + u * waves_total;
       rows[u] = grp * rows_per_wave + sub;
       ok[u] = grp < groups && rows[u] < n;
-      if (ok[u]) Codec::load(args, rows[u], cpr, chunk, frag[u]);
+      Codec::load(args, ln, ok[u] ? rows[u] : 0u, cpr, frag[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -548,12 +590,14 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
   // Resident workgroups per CU: 16 wavefronts (1024 threads) when the register
   // budget of __launch_bounds__(MAXT) holds.
   const uint32_t waves = g.threads / 64u;
-  const uint32_t waves_per_simd = 4u / ((MAXT / 64u + 3u) / 4u);  // 512 VGPRs / budget
-  uint32_t per_cu = (4u * (waves_per_simd == 0 ? 1u : waves_per_simd)) / waves;
+  // __launch_bounds__(MAXT) caps registers so that MAXT/64 wavefronts fit one CU, i.e.
+  // ceil(MAXT/256) per SIMD; that many wavefronts per SIMD are resident for any block size.
+  const uint32_t waves_per_simd = (MAXT / 64u + 3u) / 4u;
+  uint32_t per_cu = (4u * waves_per_simd) / waves;
   if (per_cu == 0) per_cu = 1;
   const uint32_t groups = (n + g.p - 1) / g.p;
   uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu;
-  const uint32_t need = (groups + U - 1) / U;
+  const uint32_t need = (groups + U - 1) / U;  // U = pipeline depth D of gemv_kernel
   if (grid > need) grid = need;
   if (grid == 0) grid = 1;
   if (g.p == 2) {
@@ -581,8 +625,8 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args 
   for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
     typename Codec::template X<1> x;
     typename Codec::Frag f;
-    Codec::template load_x<1>(args, chunk, x);
-    Codec::load(args, row, cpr, chunk, f);
+    Codec::template load_x<1>(args, chunk, true, x);
+    Codec::load(args, Codec::make_lane(args, cpr, chunk, 0u), row, cpr, f);
     float v[1];
     Codec::template dot<1>(f, x, v);
     acc += v[0];
@@ -629,7 +673,7 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     } else if (left >= 2) {
       e = launch_gemv_r<Q4KCodec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<Q4KCodec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
+      e = launch_gemv_r<Q4KCodec, 1, 1024, 8>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;

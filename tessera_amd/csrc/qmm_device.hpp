@@ -92,6 +92,25 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// DPP add: v + (v moved across lanes by `ctrl`); lanes the move does not reach add 0.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, bit_cast<int>(v), kCtrl, kRowMask, 0xF, false);
+  return v + bit_cast<float>(moved);
+}
+
+// Sum over the 64 lanes using DPP only (no LDS crossbar): xor-butterflies inside each
+// row of 16 lanes, then row broadcasts.  The total is valid in lane 63.
+__device__ __forceinline__ float wave_sum_last(float v) {
+  v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane holds its row's sum
+  v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {

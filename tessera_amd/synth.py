@@ -69,12 +69,27 @@ def mxfp4_column_shard(packed: np.ndarray, n: int, k: int, row0: int, rows: int)
     return np.concatenate([blob[row0:row0 + rows].reshape(-1), sc[row0:row0 + rows].reshape(-1)])
 
 
+def encode_e4m3(x: np.ndarray) -> np.ndarray:
+    """fp32 -> OCP E4M3 codes, round to nearest even, |x| clamped to 448 (numpy, for
+    generating weights; the kernels and the oracle have their own encoders)."""
+    x = np.clip(np.ascontiguousarray(x, dtype=np.float32), -448.0, 448.0)
+    bits = x.view(np.uint32)
+    sign = ((bits >> 24) & 0x80).astype(np.uint32)
+    mag = bits & 0x7FFFFFFF
+    sub = np.rint(np.abs(x) * np.float32(512.0)).astype(np.uint32)          # below 2^-6
+    r = mag + 0x7FFFF + ((mag >> 20) & 1)
+    norm = (r >> 20) - (120 << 3)
+    code = np.where(mag < 0x3C800000, sub, norm)
+    return (sign | code).astype(np.uint8)
+
+
 def fp8_weights(g: np.random.Generator, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:
-    """E4M3 codes (NaN codes 0x7F/0xFF excluded) and per-row scales ~ U[1e-3, 2e-2]."""
-    codes = g.integers(0, 256, size=n * k, dtype=np.uint8)
-    codes[(codes & 0x7F) == 0x7F] = 0x38  # 1.0
-    scales = g.uniform(1e-3, 2e-2, size=n).astype(np.float32)
-    return codes, scales
+    """A per-row-scaled E4M3 weight matrix as a real checkpoint holds it: W ~ N(0, 0.02^2),
+    scale[r] = amax(W[r]) / 448, codes = e4m3(W / scale).  Returns (codes n*k, scales n)."""
+    w = (g.standard_normal(size=(n, k)) * 0.02).astype(np.float32)
+    scales = (np.abs(w).max(axis=1) / np.float32(448.0)).astype(np.float32)
+    codes = encode_e4m3(w / scales[:, None])
+    return codes.reshape(-1), scales
 
 
 def activations_f32(g: np.random.Generator, m: int, k: int) -> np.ndarray:

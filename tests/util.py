@@ -5,11 +5,15 @@ from tessera_amd import KernelLaunch
 
 
 def rel_err(got: np.ndarray, ref: np.ndarray) -> float:
-    """max |got - ref| / max(|ref|, eps) with eps = 1e-3 * rms(ref), so that outputs that
-    cancel to (nearly) zero do not dominate the figure."""
+    """max |got - ref| / max(|ref|, eps) with eps = 0.05 * rms(ref).
+
+    The floor is there because the reference result is itself an fp32 sequential sum: its own
+    rounding noise is about sqrt(k) * 2^-24 * rms(ref) (1e-5 * rms at k = 17408), so an output
+    that cancels to less than a few percent of the rms cannot be reproduced to 1e-3 of its own
+    size by any other summation order.  Such outputs are held to 1e-3 * 0.05 * rms instead."""
     got = np.asarray(got, dtype=np.float64).reshape(-1)
     ref = np.asarray(ref, dtype=np.float64).reshape(-1)
-    eps = 1e-3 * np.sqrt(np.mean(ref * ref)) + 1e-30
+    eps = 0.05 * np.sqrt(np.mean(ref * ref)) + 1e-30
     return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps)))
 
 

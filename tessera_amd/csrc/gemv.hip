@@ -16,6 +16,12 @@
 //     (deterministic, no atomics).
 // Codecs plug the block format into this skeleton.
 
+#include <cstdlib>
+#ifndef QMM_EXP_D
+#define QMM_EXP_D 2
+#endif
+#include <type_traits>
+
 #include "qmm_device.hpp"
 #include "qmm_kernels.hpp"
 
@@ -120,6 +126,10 @@ struct Q4KCodec {
     // 2g+1 in byte 1).  Groups 0,1 read six bits straight from bytes 2g, 2g+1 (+4 for
     // the mins); groups 2,3 join a nibble of bytes 8.. with the top two bits of the
     // bytes that groups 0,1 use.
+#ifdef QMM_EXP_NODOT
+    for (int r = 0; r < R; ++r) out[r] = bit_cast<float>((f.h.x ^ f.q.x ^ f.q.y ^ f.q.z ^ f.q.w ^ f.h.y) & 0x3fffffffu);
+    return;
+#endif
     const uint32_t s0 = f.h.y, s1 = f.h.z, s2 = f.h.w;
     const uint32_t ls = x.upper ? s2 : s0;
     const uint32_t lmn = x.upper ? (s2 >> 4) : s1;
@@ -134,6 +144,17 @@ struct Q4KCodec {
     for (int r = 0; r < R; ++r) {
       float al = 0.0f, ah = 0.0f;
 #pragma unroll
+#ifdef QMM_EXP_CVT
+      for (int wi = 0; wi < 4; ++wi) {
+        const uint32_t lo = qw[wi] & 0x0F0F0F0Fu, hi = (qw[wi] >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          al = fmaf(x.lo[r][4 * wi + b], static_cast<float>((lo >> (8 * b)) & 0xFFu), al);
+          ah = fmaf(x.hi[r][4 * wi + b], static_cast<float>((hi >> (8 * b)) & 0xFFu), ah);
+        }
+      }
+      al *= 0x1p-24f; ah *= 0x1p-20f;
+#else
       for (int wi = 0; wi < 4; ++wi) {
         const uint32_t w = qw[wi], w8 = w >> 8;
         const half2_t l02 = bit_cast<half2_t>(w & 0x000F000Fu);   // bytes 0,2 low nibbles
@@ -149,6 +170,7 @@ struct Q4KCodec {
         al = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al);
         ah = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah);
       }
+#endif
       const float t1 = fmaf(scb, ah, sca * al);
       const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
       out[r] = fmaf(d24, t1, -(dmin * t2));
@@ -403,76 +425,86 @@ struct Fp8Codec {
 };
 
 // ----------------------------------------------------------------------------
-// The skeleton.  P weight rows share one pass of the workgroup (P = 2 fills the
-// lanes when a row's chunk count is not a multiple of 64).  Each thread keeps D row
-// fragments in registers as a software pipeline: fragment d is consumed and at once
-// refilled with the row D passes ahead, so D loads per thread stay in flight while the
-// arithmetic runs (about 100 KB outstanding per CU, what the HBM latency asks for).
-// One barrier per D passes publishes the per-wavefront partial sums.
+// The skeleton.  A workgroup owns a contiguous range of row groups; a group is P
+// weight rows laid side by side over the threads (P * chunks_per_row slots, so the
+// lanes stay full when a row's chunk count is not a multiple of 64).  Each thread
+// keeps D row fragments in registers as a software pipeline: fragment d is consumed
+// and at once refilled with the group D steps ahead, so D loads per thread stay in
+// flight while the arithmetic runs.  One barrier per D groups publishes the
+// per-wavefront partial sums; a few threads then add them in wavefront order and
+// store (deterministic, no atomics).
 // ----------------------------------------------------------------------------
 template <class Codec, int R, int P, int D, int MAXT>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, float* __restrict__ c,
-                                                    uint32_t n, uint32_t cpr, uint32_t ldc) {
+                                                    uint32_t n, uint32_t cpr, uint32_t ldc,
+                                                    uint32_t groups_per_wg) {
   constexpr int kMaxWaves = MAXT / kWave;
   __shared__ float red[2][D][P][R][kMaxWaves];
+#ifdef QMM_EXP_NULL0
+  if (n != 0xFFFFFFFFu) return;
+#endif
 
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t slots = P * cpr;
   const bool valid = t < slots;
-  const uint32_t prow = (P > 1 && valid && t >= cpr) ? 1u : 0u;
+  const uint32_t prow = valid ? t / cpr : 0u;
   const uint32_t chunk = valid ? t - prow * cpr : 0u;
 
-  // Invalid lanes (past the last chunk) carry zero activations, so they add nothing.
-  typename Codec::template X<R> x;
-  Codec::template load_x<R>(args, chunk, valid, x);
-
-  // Which of the P rows this wavefront's lanes belong to (at most two when cpr >= 64).
+  // Which of the P rows this wavefront's lanes belong to: at most two, because the
+  // launcher only uses this kernel when a row has at least 64 chunks.
   const uint32_t first_slot = wave * 64u;
   const uint32_t last_slot = first_slot + 63u < slots ? first_slot + 63u : slots - 1u;
-  const uint32_t row_a = (P > 1 && first_slot >= cpr) ? 1u : 0u;
-  const uint32_t row_b = (P > 1 && last_slot >= cpr) ? 1u : 0u;
+  const uint32_t row_a = first_slot / cpr, row_b = last_slot / cpr;
   const bool two = row_a != row_b;  // wavefront-uniform
   const float in_a = (prow == row_a) ? 1.0f : 0.0f, in_b = 1.0f - in_a;
 
-  // Work unit: a block of D consecutive row groups (D*P weight rows).  Groups past the
-  // end are clamped for the loads and dropped at the store; when n is odd and P = 2 the
-  // last group has no second row, so its lanes re-read the first one.
+  // Groups [g0, g1) belong to this workgroup.  A group index past the end is clamped
+  // for the loads and dropped at the store; rows past n inside the last group re-read
+  // the group's first row.
   const uint32_t groups = (n + P - 1) / P;
-  const uint32_t nblocks = (groups + D - 1) / D;
+  const uint32_t g0 = blockIdx.x * groups_per_wg;
+  const uint32_t g1 = g0 + groups_per_wg < groups ? g0 + groups_per_wg : groups;
   const Lane ln = Codec::make_lane(args, cpr, chunk, prow);
-  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, 0u);
-  const bool ragged = (P > 1) && (n % P != 0);
-  auto fetch = [&](uint32_t blk, int d, typename Codec::Frag& f) {
-    uint32_t grp = blk * D + d;
+  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, (groups - 1u) * P + prow < n ? prow : 0u);
+  const bool ragged = n % P != 0;
+  auto fetch = [&](uint32_t grp, typename Codec::Frag& f) {
     grp = grp < groups ? grp : groups - 1u;
     const bool tail = ragged && grp == groups - 1u;
     Codec::load(args, tail ? ln_tail : ln, grp * P, cpr, f);
   };
 
+  // Weight loads first, activations second: both are in flight before anything waits.
   typename Codec::Frag frag[D];
-  uint32_t blk = blockIdx.x;
-  if (blk < nblocks) {
 #pragma unroll
-    for (int d = 0; d < D; ++d) fetch(blk, d, frag[d]);
-  }
+  for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
+
+  // Invalid lanes (past the last chunk) carry zero activations, so they add nothing.
+  typename Codec::template X<R> x;
+  Codec::template load_x<R>(args, chunk, valid, x);
+
   uint32_t buf = 0;
-  for (; blk < nblocks; blk += gridDim.x) {
-    uint32_t nxt = blk + gridDim.x;
-    nxt = nxt < nblocks ? nxt : nblocks - 1u;  // the last refill re-reads, unused
+  // One round = D pipeline stages, one barrier.  `refill` rounds reload every
+  // fragment they consume (unconditionally, so the compiler can count outstanding loads
+  // exactly and never waits for more than the one fragment it needs); the last round
+  // loads nothing and skips stages past the range.
+  auto round = [&](uint32_t g, auto refill) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
+      if (!decltype(refill)::value && g + d >= g1) break;
       float v[R];
       Codec::template dot<R>(frag[d], x, v);
-      fetch(nxt, d, frag[d]);
+#ifndef QMM_EXP_NOLOAD
+      if constexpr (decltype(refill)::value) fetch(g + D + d, frag[d]);
+#endif
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        if (P > 1 && two) {
+        if (two) {
           const float sa = wave_sum_last(v[r] * in_a);
           const float sb = wave_sum_last(v[r] * in_b);
           if (lane == 63u) {
-            red[buf][d][0][r][wave] = sa;
-            red[buf][d][P - 1][r][wave] = sb;
+            red[buf][d][row_a][r][wave] = sa;
+            red[buf][d][row_b][r][wave] = sb;
           }
         } else {
           const float sa = wave_sum_last(v[r]);
@@ -480,11 +512,11 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
         }
       }
     }
-    __syncthreads();
+    lds_barrier();  // LDS only: the prefetched global loads stay in flight across it
     if (t < D * P * R) {
       const uint32_t d = t / (P * R), p = (t / R) % P, r = t % R;
-      const uint32_t row = (blk * D + d) * P + p;
-      if (row < n) {
+      const uint32_t row = (g + d) * P + p;
+      if (g + d < g1 && row < n) {
         const uint32_t w_lo = (p * cpr) >> 6, w_hi = ((p + 1u) * cpr - 1u) >> 6;
         float sum = 0.0f;
         for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][d][p][r][w];
@@ -492,7 +524,14 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       }
     }
     buf ^= 1u;
-  }
+  };
+
+#ifdef QMM_EXP_NULL
+  if (n != 0xFFFFFFFFu) return;
+#endif
+  uint32_t g = g0;
+  for (; g + D < g1; g += D) round(g, std::true_type{});
+  if (g < g1) round(g, std::false_type{});
 }
 
 // Small-K variant (a row has 8, 16 or 32 chunks): each wavefront owns 64 / cpr whole
@@ -544,12 +583,17 @@ __global__ __launch_bounds__(256) void gemv_smallk_kernel(typename Codec::Args a
 struct GemvPlan {
   uint32_t cpr;
   uint32_t threads;  // workgroup size, multiple of 64
-  int p;             // weight rows per pass
+  uint32_t p;        // weight rows per group
   bool smallk;
 };
 
-// Workgroup shape: the thread count that wastes the fewest lanes, preferring one
-// row per pass; two rows per pass when that fills the lanes better.
+int g_num_cus = 256;
+int g_tune_p = 0;  // QMM_GEMV_P: force rows per group (experiments only)
+
+// Workgroup shape: rows per group P in 1..kMaxP and the thread count P*cpr rounded up
+// to whole wavefronts; picks the P that idles the fewest lanes, larger P on ties
+// (fewer, fuller workgroups share one copy of the activations).
+template <uint32_t kMaxP>
 GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads) {
   GemvPlan g{cpr, 0, 1, false};
   if (cpr == 8 || cpr == 16 || cpr == 32) {
@@ -557,24 +601,49 @@ GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads) {
     g.threads = 256;
     return g;
   }
-  const uint32_t t1 = (cpr + 63u) / 64u * 64u;
-  const uint32_t t2 = (2u * cpr + 63u) / 64u * 64u;
-  g.threads = t1;
-  if (cpr >= 64 && t2 <= max_threads && (t2 - 2u * cpr) * t1 < (t1 - cpr) * t2) {
-    g.p = 2;
-    g.threads = t2;
+  g.threads = (cpr + 63u) / 64u * 64u;
+  if (cpr < 64) return g;  // a wavefront may span at most two rows
+  double best = static_cast<double>(cpr) / g.threads;
+  for (uint32_t p = 2; p <= kMaxP; ++p) {
+    const uint32_t t = (p * cpr + 63u) / 64u * 64u;
+    if (t > max_threads) break;
+    const double fill = static_cast<double>(p * cpr) / t;
+    if (fill >= best || (g_tune_p != 0 && static_cast<int>(p) == g_tune_p)) {
+      best = fill;
+      g.p = p;
+      g.threads = t;
+      if (g_tune_p != 0 && static_cast<int>(p) == g_tune_p) break;
+    }
   }
   return g;
 }
 
-int g_num_cus = 256;
+template <class Codec, int R, int MAXT, int D, uint32_t P>
+hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n, uint32_t cpr,
+                         uint32_t ldc, uint32_t threads, hipStream_t stream) {
+  // Resident workgroups per CU under __launch_bounds__(MAXT): the register budget
+  // admits ceil(MAXT/256) wavefronts per SIMD whatever the block size.
+  const uint32_t waves = threads / 64u;
+  const uint32_t waves_per_simd = (MAXT / 64u + 3u) / 4u;
+  uint32_t per_cu = (4u * waves_per_simd) / waves;
+  if (per_cu == 0) per_cu = 1;
+  const uint32_t groups = (n + P - 1) / P;
+  uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu;
+  if (grid > groups) grid = groups;
+  uint32_t per_wg = (groups + grid - 1) / grid;
+  grid = (groups + per_wg - 1) / per_wg;
+  hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT>), dim3(grid), dim3(threads), 0, stream, args,
+                     c, n, cpr, ldc, per_wg);
+  return hipGetLastError();
+}
 
-template <class Codec, int R, int MAXT, int U>
+template <class Codec, int R, int MAXT, int D, uint32_t kMaxP = 2>
 hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n, uint32_t k,
                          uint32_t ldc, hipStream_t stream) {
   const uint32_t cpr = Codec::chunks_per_row(k);
-  const GemvPlan g = plan_gemv(cpr, MAXT);
+  const GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT);
   if (g.smallk) {
+    constexpr int U = D > 4 ? 4 : D;
     const uint32_t rows_per_wave = 64u / cpr;
     const uint32_t groups = (n + rows_per_wave - 1) / rows_per_wave;
     uint32_t grid = (groups + 4u * U - 1) / (4u * U);
@@ -584,30 +653,17 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
                        n, cpr, ldc);
     return hipGetLastError();
   }
-  if (g.threads > MAXT) {
-    return hipErrorInvalidValue;
+  if (g.threads > MAXT) return hipErrorInvalidValue;
+  switch (g.p) {
+    case 1: return launch_gemv_p<Codec, R, MAXT, D, 1>(args, c, n, cpr, ldc, g.threads, stream);
+    case 2: return launch_gemv_p<Codec, R, MAXT, D, 2>(args, c, n, cpr, ldc, g.threads, stream);
+    case 3: if constexpr (kMaxP >= 3) return launch_gemv_p<Codec, R, MAXT, D, 3>(args, c, n, cpr, ldc, g.threads, stream); break;
+    case 4: if constexpr (kMaxP >= 4) return launch_gemv_p<Codec, R, MAXT, D, 4>(args, c, n, cpr, ldc, g.threads, stream); break;
+    case 5: if constexpr (kMaxP >= 5) return launch_gemv_p<Codec, R, MAXT, D, 5>(args, c, n, cpr, ldc, g.threads, stream); break;
+    case 6: if constexpr (kMaxP >= 6) return launch_gemv_p<Codec, R, MAXT, D, 6>(args, c, n, cpr, ldc, g.threads, stream); break;
+    default: break;
   }
-  // Resident workgroups per CU: 16 wavefronts (1024 threads) when the register
-  // budget of __launch_bounds__(MAXT) holds.
-  const uint32_t waves = g.threads / 64u;
-  // __launch_bounds__(MAXT) caps registers so that MAXT/64 wavefronts fit one CU, i.e.
-  // ceil(MAXT/256) per SIMD; that many wavefronts per SIMD are resident for any block size.
-  const uint32_t waves_per_simd = (MAXT / 64u + 3u) / 4u;
-  uint32_t per_cu = (4u * waves_per_simd) / waves;
-  if (per_cu == 0) per_cu = 1;
-  const uint32_t groups = (n + g.p - 1) / g.p;
-  uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu;
-  const uint32_t need = (groups + U - 1) / U;  // U = pipeline depth D of gemv_kernel
-  if (grid > need) grid = need;
-  if (grid == 0) grid = 1;
-  if (g.p == 2) {
-    hipLaunchKernelGGL((gemv_kernel<Codec, R, 2, U, MAXT>), dim3(grid), dim3(g.threads), 0, stream,
-                       args, c, n, cpr, ldc);
-  } else {
-    hipLaunchKernelGGL((gemv_kernel<Codec, R, 1, U, MAXT>), dim3(grid), dim3(g.threads), 0, stream,
-                       args, c, n, cpr, ldc);
-  }
-  return hipGetLastError();
+  return hipErrorInvalidValue;
 }
 
 // Fallback for shapes the register-resident mapping does not cover (a row longer
@@ -647,7 +703,10 @@ hipError_t launch_gemv_generic(const typename Codec::Args& args, float* c, uint3
 
 }  // namespace
 
-void set_num_cus(int cus) { g_num_cus = cus > 0 ? cus : 256; }
+void set_num_cus(int cus) {
+  g_num_cus = cus > 0 ? cus : 256;
+  if (const char* e = std::getenv("QMM_GEMV_P")) g_tune_p = std::atoi(e);
+}
 
 // K limits of the register-resident mapping: one 16-byte chunk per thread, at most
 // 1024 threads per row.
@@ -673,7 +732,7 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     } else if (left >= 2) {
       e = launch_gemv_r<Q4KCodec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<Q4KCodec, 1, 1024, 8>(args, out, n, k, n, stream), took = 1;
+      e = launch_gemv_r<Q4KCodec, 1, 1024, QMM_EXP_D, 6>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;

@@ -17,8 +17,9 @@
 // Codecs plug the block format into this skeleton.
 
 #include <cstdlib>
-#ifndef QMM_EXP_D
-#define QMM_EXP_D 2
+#ifndef QMM_D1
+#define QMM_D1 2
+#define QMM_T1 1024
 #endif
 #include <type_traits>
 
@@ -27,6 +28,28 @@
 
 namespace qmm {
 namespace {
+
+// Where a codec reads fp32 activations from: straight from global memory ...
+struct GlobalX {
+  const float* a;
+  uint32_t k;
+  __device__ __forceinline__ float4 operator()(int r, uint32_t elem) const {
+    return *reinterpret_cast<const float4*>(a + static_cast<size_t>(r) * k + elem);
+  }
+};
+// ... or from a piece of the activation rows staged in LDS.  A thread's slice is a
+// few hundred contiguous bytes, so reading it straight from global memory makes every
+// lane of a load touch its own cache line; the staged copy is filled with coalesced
+// loads and padded by 4 floats per 64 so the strided reads spread over the banks.
+struct StagedX {
+  const float* lds;
+  uint32_t base;    // first element of the staged piece
+  uint32_t stride;  // padded floats per staged row
+  static __device__ __forceinline__ uint32_t pad(uint32_t e) { return e + (e >> 6) * 4u; }
+  __device__ __forceinline__ float4 operator()(int r, uint32_t elem) const {
+    return *reinterpret_cast<const float4*>(lds + r * stride + pad(elem - base));
+  }
+};
 
 // Per-thread byte offsets of a chunk relative to the (wavefront-uniform) start of a
 // row group; the uniform part goes through scalar registers, so a load is one
@@ -75,9 +98,15 @@ struct Q4KCodec {
   };
 
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
+  // Whether the skeleton stages fp32 activations through LDS for this codec, and the
+  // first activation element a chunk needs (its slice stays inside that 64-aligned group
+  // or starts there).
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return (chunk >> 1) * 64u; }
 
-  template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
     const uint32_t blk = chunk >> 3, j = chunk & 7u, g = j >> 1;
     x.sh = (g & 1u) * 16u;
     x.upper = g >= 2u;
@@ -86,12 +115,11 @@ struct Q4KCodec {
     const uint32_t k0 = blk * 256u + g * 64u + (j & 1u) * 16u;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float* src = p.a + static_cast<size_t>(r) * p.k + k0;
       float sl = 0.0f, sh = 0.0f;
 #pragma unroll
       for (int i = 0; i < 16; i += 4) {
-        float4 lo = *reinterpret_cast<const float4*>(src + i);
-        float4 hi = *reinterpret_cast<const float4*>(src + 32 + i);
+        float4 lo = src(r, k0 + i);
+        float4 hi = src(r, k0 + 32 + i);
         if (!valid) lo = hi = make_float4(0.f, 0.f, 0.f, 0.f);
         x.lo[r][i] = lo.x, x.lo[r][i + 1] = lo.y, x.lo[r][i + 2] = lo.z, x.lo[r][i + 3] = lo.w;
         x.hi[r][i] = hi.x, x.hi[r][i + 1] = hi.y, x.hi[r][i + 2] = hi.z, x.hi[r][i + 3] = hi.w;
@@ -126,10 +154,6 @@ struct Q4KCodec {
     // 2g+1 in byte 1).  Groups 0,1 read six bits straight from bytes 2g, 2g+1 (+4 for
     // the mins); groups 2,3 join a nibble of bytes 8.. with the top two bits of the
     // bytes that groups 0,1 use.
-#ifdef QMM_EXP_NODOT
-    for (int r = 0; r < R; ++r) out[r] = bit_cast<float>((f.h.x ^ f.q.x ^ f.q.y ^ f.q.z ^ f.q.w ^ f.h.y) & 0x3fffffffu);
-    return;
-#endif
     const uint32_t s0 = f.h.y, s1 = f.h.z, s2 = f.h.w;
     const uint32_t ls = x.upper ? s2 : s0;
     const uint32_t lmn = x.upper ? (s2 >> 4) : s1;
@@ -144,17 +168,6 @@ struct Q4KCodec {
     for (int r = 0; r < R; ++r) {
       float al = 0.0f, ah = 0.0f;
 #pragma unroll
-#ifdef QMM_EXP_CVT
-      for (int wi = 0; wi < 4; ++wi) {
-        const uint32_t lo = qw[wi] & 0x0F0F0F0Fu, hi = (qw[wi] >> 4) & 0x0F0F0F0Fu;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          al = fmaf(x.lo[r][4 * wi + b], static_cast<float>((lo >> (8 * b)) & 0xFFu), al);
-          ah = fmaf(x.hi[r][4 * wi + b], static_cast<float>((hi >> (8 * b)) & 0xFFu), ah);
-        }
-      }
-      al *= 0x1p-24f; ah *= 0x1p-20f;
-#else
       for (int wi = 0; wi < 4; ++wi) {
         const uint32_t w = qw[wi], w8 = w >> 8;
         const half2_t l02 = bit_cast<half2_t>(w & 0x000F000Fu);   // bytes 0,2 low nibbles
@@ -170,7 +183,127 @@ struct Q4KCodec {
         al = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al);
         ah = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah);
       }
-#endif
+      const float t1 = fmaf(scb, ah, sca * al);
+      const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
+      out[r] = fmaf(d24, t1, -(dmin * t2));
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+
+// ----------------------------------------------------------------------------
+// Q4_K, single activation row: the same arithmetic with a 32-byte chunk per thread
+// (one whole group g of a block: sub-block 2g in the low nibbles, 2g+1 in the high
+// nibbles), so the header decode, the cross-lane reduction and the loop overhead are
+// paid once per 64 weights instead of once per 32.
+// ----------------------------------------------------------------------------
+struct Q4KPairCodec {
+  using Args = Q4KCodec::Args;
+  template <int R>
+  struct X {
+    float lo[R][32];
+    float hi[R][32];  // activation / 16
+    float slo[R];
+    float shi[R];
+    uint32_t sh;
+    uint32_t lm, hm;
+    bool upper;
+  };
+  struct Frag {
+    uint4 h;
+    uint4 q0;
+    uint4 q1;
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 64u; }
+  // Whether the skeleton stages fp32 activations through LDS for this codec, and the
+  // first activation element a chunk needs (its slice stays inside that 64-aligned group
+  // or starts there).
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 64u; }
+
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    const uint32_t blk = chunk >> 2, g = chunk & 3u;
+    x.sh = (g & 1u) * 16u;
+    x.upper = g >= 2u;
+    x.lm = x.upper ? 0x0F0Fu : 0x3F3Fu;
+    x.hm = x.upper ? 0x3030u : 0u;
+    const uint32_t k0 = blk * 256u + g * 64u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float sl = 0.0f, sh = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 32; i += 4) {
+        float4 lo = src(r, k0 + i);
+        float4 hi = src(r, k0 + 32 + i);
+        if (!valid) lo = hi = make_float4(0.f, 0.f, 0.f, 0.f);
+        x.lo[r][i] = lo.x, x.lo[r][i + 1] = lo.y, x.lo[r][i + 2] = lo.z, x.lo[r][i + 3] = lo.w;
+        x.hi[r][i] = hi.x, x.hi[r][i + 1] = hi.y, x.hi[r][i + 2] = hi.z, x.hi[r][i + 3] = hi.w;
+      }
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        sl += x.lo[r][i];
+        sh += x.hi[r][i];
+        x.hi[r][i] *= 0.0625f;
+      }
+      x.slo[r] = sl;
+      x.shi[r] = sh;
+    }
+  }
+
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t hdr = prow * (cpr >> 2) * 144u + (chunk >> 2) * 144u;
+    return Lane{hdr, hdr + 16u + (chunk & 3u) * 32u};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const uint8_t* base = p.w + static_cast<size_t>(row) * ((cpr >> 2) * 144u);
+    f.h = load_u4(base + ln.off0);
+    f.q0 = load_u4(base + ln.off1);
+    f.q1 = load_u4(base + ln.off1 + 16u);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const uint32_t s0 = f.h.y, s1 = f.h.z, s2 = f.h.w;
+    const uint32_t ls = x.upper ? s2 : s0;
+    const uint32_t lmn = x.upper ? (s2 >> 4) : s1;
+    const uint32_t sc2 = ((ls >> x.sh) & x.lm) | ((s0 >> (x.sh + 2u)) & x.hm);
+    const uint32_t mn2 = ((lmn >> x.sh) & x.lm) | ((s1 >> (x.sh + 2u)) & x.hm);
+    const float sca = static_cast<float>(sc2 & 0xFFu), scb = static_cast<float>((sc2 >> 8) & 0xFFu);
+    const float mna = static_cast<float>(mn2 & 0xFFu), mnb = static_cast<float>((mn2 >> 8) & 0xFFu);
+    const float d24 = half_bits_to_float(f.h.x & 0xFFFFu) * 0x1p24f;
+    const float dmin = half_bits_to_float(f.h.x >> 16);
+    const uint32_t qw[8] = {f.q0.x, f.q0.y, f.q0.z, f.q0.w, f.q1.x, f.q1.y, f.q1.z, f.q1.w};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float al = 0.0f, ah = 0.0f, bl = 0.0f, bh = 0.0f;  // two chains per half for ILP
+#pragma unroll
+      for (int wi = 0; wi < 8; ++wi) {
+        const uint32_t w = qw[wi], w8 = w >> 8;
+        const half2_t l02 = bit_cast<half2_t>(w & 0x000F000Fu);
+        const half2_t h02 = bit_cast<half2_t>(w & 0x00F000F0u);
+        const half2_t l13 = bit_cast<half2_t>(w8 & 0x000F000Fu);
+        const half2_t h13 = bit_cast<half2_t>(w8 & 0x00F000F0u);
+        al = fmaf(x.lo[r][4 * wi + 0], static_cast<float>(l02[0]), al);
+        ah = fmaf(x.hi[r][4 * wi + 0], static_cast<float>(h02[0]), ah);
+        bl = fmaf(x.lo[r][4 * wi + 1], static_cast<float>(l13[0]), bl);
+        bh = fmaf(x.hi[r][4 * wi + 1], static_cast<float>(h13[0]), bh);
+        al = fmaf(x.lo[r][4 * wi + 2], static_cast<float>(l02[1]), al);
+        ah = fmaf(x.hi[r][4 * wi + 2], static_cast<float>(h02[1]), ah);
+        bl = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), bl);
+        bh = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), bh);
+      }
+      al += bl;
+      ah += bh;
       const float t1 = fmaf(scb, ah, sca * al);
       const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
       out[r] = fmaf(d24, t1, -(dmin * t2));
@@ -206,15 +339,20 @@ struct MxFp4Codec {
   };
 
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
+  // Whether the skeleton stages fp32 activations through LDS for this codec, and the
+  // first activation element a chunk needs (its slice stays inside that 64-aligned group
+  // or starts there).
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 32u; }
 
-  template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float* src = p.a + static_cast<size_t>(r) * p.k + chunk * 32u;
 #pragma unroll
       for (int i = 0; i < 32; i += 4) {
-        float4 v = *reinterpret_cast<const float4*>(src + i);
+        float4 v = src(r, chunk * 32u + i);
         if (!valid) v = make_float4(0.f, 0.f, 0.f, 0.f);
         x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
       }
@@ -291,9 +429,15 @@ struct MxFp4A8Codec {
   };
 
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 32u; }
+  // Whether the skeleton stages fp32 activations through LDS for this codec, and the
+  // first activation element a chunk needs (its slice stays inside that 64-aligned group
+  // or starts there).
+  static constexpr bool kStageX = false;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 32u; }
 
-  template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const uint8_t* src = p.a + static_cast<size_t>(r) * p.k + chunk * 32u;
@@ -372,15 +516,20 @@ struct Fp8Codec {
   };
 
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 16u; }
+  // Whether the skeleton stages fp32 activations through LDS for this codec, and the
+  // first activation element a chunk needs (its slice stays inside that 64-aligned group
+  // or starts there).
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 16u; }
 
-  template <int R>
-  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x) {
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float* src = p.a + static_cast<size_t>(r) * p.k + chunk * 16u;
 #pragma unroll
       for (int i = 0; i < 16; i += 4) {
-        float4 v = *reinterpret_cast<const float4*>(src + i);
+        float4 v = src(r, chunk * 16u + i);
         if (!valid) v = make_float4(0.f, 0.f, 0.f, 0.f);
         x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
       }
@@ -440,9 +589,6 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
                                                     uint32_t groups_per_wg) {
   constexpr int kMaxWaves = MAXT / kWave;
   __shared__ float red[2][D][P][R][kMaxWaves];
-#ifdef QMM_EXP_NULL0
-  if (n != 0xFFFFFFFFu) return;
-#endif
 
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -481,7 +627,30 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
 
   // Invalid lanes (past the last chunk) carry zero activations, so they add nothing.
   typename Codec::template X<R> x;
-  Codec::template load_x<R>(args, chunk, valid, x);
+  if constexpr (Codec::kStageX) {
+    constexpr uint32_t kPiece = R == 1 ? 8192u : (R == 2 ? 4096u : 2048u);  // floats per row
+    constexpr uint32_t kStride = kPiece + kPiece / 16u;
+    __shared__ __attribute__((aligned(16))) float xs[R * kStride];
+    const uint32_t k = args.k;
+    const uint32_t mine = Codec::x_elem0(chunk);
+    for (uint32_t base = 0; base < k; base += kPiece) {
+      const uint32_t len = k - base < kPiece ? k - base : kPiece;
+      if (base != 0) lds_barrier();  // the previous piece has been read
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        for (uint32_t e = t * 4u; e < len; e += blockDim.x * 4u) {
+          *reinterpret_cast<float4*>(&xs[r * kStride + StagedX::pad(e)]) =
+              *reinterpret_cast<const float4*>(args.a + static_cast<size_t>(r) * k + base + e);
+        }
+      }
+      lds_barrier();
+      if (mine >= base && mine < base + len) {
+        Codec::template load_x<R>(args, chunk, valid, x, StagedX{xs, base, kStride});
+      }
+    }
+  } else {
+    Codec::template load_x<R>(args, chunk, valid, x, 0);
+  }
 
   uint32_t buf = 0;
   // One round = D pipeline stages, one barrier.  `refill` rounds reload every
@@ -494,9 +663,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       if (!decltype(refill)::value && g + d >= g1) break;
       float v[R];
       Codec::template dot<R>(frag[d], x, v);
-#ifndef QMM_EXP_NOLOAD
       if constexpr (decltype(refill)::value) fetch(g + D + d, frag[d]);
-#endif
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (two) {
@@ -526,9 +693,6 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
     buf ^= 1u;
   };
 
-#ifdef QMM_EXP_NULL
-  if (n != 0xFFFFFFFFu) return;
-#endif
   uint32_t g = g0;
   for (; g + D < g1; g += D) round(g, std::true_type{});
   if (g < g1) round(g, std::false_type{});
@@ -544,7 +708,11 @@ __global__ __launch_bounds__(256) void gemv_smallk_kernel(typename Codec::Args a
   const uint32_t rows_per_wave = 64u / cpr;
   const uint32_t chunk = lane % cpr, sub = lane / cpr;
   typename Codec::template X<R> x;
-  Codec::template load_x<R>(args, chunk, true, x);
+  if constexpr (Codec::kStageX) {
+    Codec::template load_x<R>(args, chunk, true, x, GlobalX{args.a, args.k});
+  } else {
+    Codec::template load_x<R>(args, chunk, true, x, 0);
+  }
   const Lane ln = Codec::make_lane(args, cpr, chunk, 0u);
   const uint32_t wave_global = blockIdx.x * (blockDim.x >> 6) + (t >> 6);
   const uint32_t waves_total = gridDim.x * (blockDim.x >> 6);
@@ -596,7 +764,7 @@ int g_tune_p = 0;  // QMM_GEMV_P: force rows per group (experiments only)
 template <uint32_t kMaxP>
 GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads) {
   GemvPlan g{cpr, 0, 1, false};
-  if (cpr == 8 || cpr == 16 || cpr == 32) {
+  if (cpr == 4 || cpr == 8 || cpr == 16 || cpr == 32) {
     g.smallk = true;
     g.threads = 256;
     return g;
@@ -655,12 +823,14 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
   }
   if (g.threads > MAXT) return hipErrorInvalidValue;
   switch (g.p) {
-    case 1: return launch_gemv_p<Codec, R, MAXT, D, 1>(args, c, n, cpr, ldc, g.threads, stream);
-    case 2: return launch_gemv_p<Codec, R, MAXT, D, 2>(args, c, n, cpr, ldc, g.threads, stream);
-    case 3: if constexpr (kMaxP >= 3) return launch_gemv_p<Codec, R, MAXT, D, 3>(args, c, n, cpr, ldc, g.threads, stream); break;
-    case 4: if constexpr (kMaxP >= 4) return launch_gemv_p<Codec, R, MAXT, D, 4>(args, c, n, cpr, ldc, g.threads, stream); break;
-    case 5: if constexpr (kMaxP >= 5) return launch_gemv_p<Codec, R, MAXT, D, 5>(args, c, n, cpr, ldc, g.threads, stream); break;
-    case 6: if constexpr (kMaxP >= 6) return launch_gemv_p<Codec, R, MAXT, D, 6>(args, c, n, cpr, ldc, g.threads, stream); break;
+#define QMM_GEMV_CASE(PP)                                                                       \
+  case PP:                                                                                      \
+    if constexpr (kMaxP >= PP)                                                                  \
+      return launch_gemv_p<Codec, R, MAXT, D, PP>(args, c, n, cpr, ldc, g.threads, stream);     \
+    break;
+    QMM_GEMV_CASE(1) QMM_GEMV_CASE(2) QMM_GEMV_CASE(3) QMM_GEMV_CASE(4) QMM_GEMV_CASE(5) QMM_GEMV_CASE(6)
+    QMM_GEMV_CASE(7) QMM_GEMV_CASE(8) QMM_GEMV_CASE(9) QMM_GEMV_CASE(10) QMM_GEMV_CASE(11) QMM_GEMV_CASE(12)
+#undef QMM_GEMV_CASE
     default: break;
   }
   return hipErrorInvalidValue;
@@ -681,7 +851,11 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args 
   for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
     typename Codec::template X<1> x;
     typename Codec::Frag f;
-    Codec::template load_x<1>(args, chunk, true, x);
+    if constexpr (Codec::kStageX) {
+      Codec::template load_x<1>(args, chunk, true, x, GlobalX{args.a, args.k});
+    } else {
+      Codec::template load_x<1>(args, chunk, true, x, 0);
+    }
     Codec::load(args, Codec::make_lane(args, cpr, chunk, 0u), row, cpr, f);
     float v[1];
     Codec::template dot<1>(f, x, v);
@@ -710,7 +884,7 @@ void set_num_cus(int cus) {
 
 // K limits of the register-resident mapping: one 16-byte chunk per thread, at most
 // 1024 threads per row.
-bool gemv_q4k_supported(uint64_t k) { return k % 256 == 0 && k / 32 <= 1024; }
+bool gemv_q4k_supported(uint64_t k) { return k % 256 == 0 && k / 32 <= 1024; }  // multi-row limit
 bool gemv_mxfp4_supported(uint64_t k) { return k % 32 == 0 && k / 32 <= 1024; }
 bool gemv_fp8_supported(uint64_t k) { return k % 16 == 0 && k / 16 <= 1024; }
 
@@ -732,7 +906,7 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     } else if (left >= 2) {
       e = launch_gemv_r<Q4KCodec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<Q4KCodec, 1, 1024, QMM_EXP_D, 6>(args, out, n, k, n, stream), took = 1;
+      e = launch_gemv_r<Q4KPairCodec, 1, QMM_T1, QMM_D1, 12>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;

@@ -161,7 +161,7 @@ def main():
                    "layers_rotated": args.layers, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_kernel<Q4KCodec> N=17408 K=5120",
+                     "kernel": "gemv_kernel<Q4KPairCodec> N=17408 K=5120",
                      "us_per_launch": round(us_per_launch, 3),
                      "algorithmic_bytes_per_launch": gemv_algorithmic_bytes(N_FF, K_HID),
                      "down_us_per_launch": round(us_down, 3),

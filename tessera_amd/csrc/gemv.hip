@@ -17,10 +17,6 @@
 // Codecs plug the block format into this skeleton.
 
 #include <cstdlib>
-#ifndef QMM_D1
-#define QMM_D1 2
-#define QMM_T1 1024
-#endif
 #include <type_traits>
 
 #include "qmm_device.hpp"
@@ -285,7 +281,7 @@ struct Q4KPairCodec {
     const uint32_t qw[8] = {f.q0.x, f.q0.y, f.q0.z, f.q0.w, f.q1.x, f.q1.y, f.q1.z, f.q1.w};
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      float al = 0.0f, ah = 0.0f, bl = 0.0f, bh = 0.0f;  // two chains per half for ILP
+      float al = 0.0f, ah = 0.0f;
 #pragma unroll
       for (int wi = 0; wi < 8; ++wi) {
         const uint32_t w = qw[wi], w8 = w >> 8;
@@ -295,15 +291,13 @@ struct Q4KPairCodec {
         const half2_t h13 = bit_cast<half2_t>(w8 & 0x00F000F0u);
         al = fmaf(x.lo[r][4 * wi + 0], static_cast<float>(l02[0]), al);
         ah = fmaf(x.hi[r][4 * wi + 0], static_cast<float>(h02[0]), ah);
-        bl = fmaf(x.lo[r][4 * wi + 1], static_cast<float>(l13[0]), bl);
-        bh = fmaf(x.hi[r][4 * wi + 1], static_cast<float>(h13[0]), bh);
+        al = fmaf(x.lo[r][4 * wi + 1], static_cast<float>(l13[0]), al);
+        ah = fmaf(x.hi[r][4 * wi + 1], static_cast<float>(h13[0]), ah);
         al = fmaf(x.lo[r][4 * wi + 2], static_cast<float>(l02[1]), al);
         ah = fmaf(x.hi[r][4 * wi + 2], static_cast<float>(h02[1]), ah);
-        bl = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), bl);
-        bh = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), bh);
+        al = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al);
+        ah = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah);
       }
-      al += bl;
-      ah += bh;
       const float t1 = fmaf(scb, ah, sca * al);
       const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
       out[r] = fmaf(d24, t1, -(dmin * t2));
@@ -906,7 +900,7 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     } else if (left >= 2) {
       e = launch_gemv_r<Q4KCodec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<Q4KPairCodec, 1, QMM_T1, QMM_D1, 12>(args, out, n, k, n, stream), took = 1;
+      e = launch_gemv_r<Q4KPairCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;

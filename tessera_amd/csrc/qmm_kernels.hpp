@@ -30,6 +30,12 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream);
 
+// ---- MFMA GEMMs (gemm_mxfp4.hip, gemm_q4k.hip) --------------------------------------
+bool gemm_mxfp4_a8_supported(uint64_t k);
+// W4A8 on the scaled MFMA: A = m x k E4M3 codes + per-row scales, W packed MXFP4.
+hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
+                                uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
+
 // ---- element-wise helpers (elementwise.hip) ---------------------------------
 hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64_t split,
                              hipStream_t stream);

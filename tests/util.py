@@ -17,6 +17,13 @@ def rel_err(got: np.ndarray, ref: np.ndarray) -> float:
     return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps)))
 
 
+def rms_err(got: np.ndarray, ref: np.ndarray) -> float:
+    """max |got - ref| / rms(ref): the absolute error in units of a typical output."""
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    return float(np.max(np.abs(got - ref)) / (np.sqrt(np.mean(ref * ref)) + 1e-30))
+
+
 def norm_err(got: np.ndarray, ref: np.ndarray) -> float:
     got = np.asarray(got, dtype=np.float64).reshape(-1)
     ref = np.asarray(ref, dtype=np.float64).reshape(-1)

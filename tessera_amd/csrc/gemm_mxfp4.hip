@@ -11,13 +11,18 @@
 // fp32 accumulation, so the result equals the reference's QuantizeFp8Ref + GemmMxFp4Ref
 // up to summation order.
 //
-// Tiling: a 256-thread workgroup owns a 128 x 128 tile of C; each of its four
-// wavefronts a 64 x 64 quadrant (2 x 2 MFMA tiles of 32 x 32, 64 accumulator
-// registers).  K advances 256 per step: the activation tile (128 x 256 bytes) goes
-// through LDS, padded so the 16-byte fragment reads spread over all banks; the weight
-// fragments are 16-byte loads straight from global memory into the B operand, one
-// MX block per lane, with the next step's loads issued before the current step's
-// MFMAs.
+// Shape of the kernel.  A workgroup owns a BM x BN tile of C (256 x 256 with eight
+// wavefronts for prefill: 64 x 128 and 128 accumulator registers per wavefront, two
+// wavefronts per SIMD so that one's LDS reads run under the other's MFMAs) and walks K in
+// steps of 128.  Operand tiles travel HBM -> LDS directly (global_load_lds, 16 bytes a
+// lane), never through registers, into a ring of three LDS stages: while step s is
+// multiplied, the loads of steps s+1 and s+2 are in flight, about 96 KB per CU, which is
+// what the memory latency under load (about 2 microseconds) times the consumption rate
+// asks for.  A direct load lands lane p's 16 bytes at position p of a 1 KB block, so rows
+// cannot be padded; instead each lane fetches the chunk whose index is XOR-swizzled with
+// its row, and the fragment reads undo the swizzle.  With that, the 16-byte fragment
+// reads of 16 consecutive rows fall on 16 distinct bank groups.  Workgroups are
+// persistent (one per CU) and the ring runs across tile boundaries.
 
 #include "qmm_device.hpp"
 #include "qmm_kernels.hpp"
@@ -25,147 +30,279 @@
 namespace qmm {
 namespace {
 
-constexpr int kBM = 128, kBN = 128, kKS = 256;      // workgroup tile, K per step
-constexpr int kARow = kKS + 16;                      // padded LDS row of the A tile, bytes
-constexpr int kSteps = kKS / 64;                     // MFMA K-steps per K step
+constexpr int kKS = 128;                    // K per step: one 32-bit word of E8M0 bytes per weight row
+constexpr int kDmaPerStage = 13;            // direct loads a wavefront issues per stage (8 A, 4 B, 1 scales)
 
-struct BFrag {
-  uint4 q[kSteps][2];   // [k-step][n-subtile]: 32 E2M1 values of one MX block
-  uint2 s[2];           // 8 E8M0 bytes per n-subtile: the row's blocks of this K step
-};
+// Direct HBM -> LDS load: lane p's `bytes` at global `base + voff` land at LDS address
+// lds_addr + p * bytes (base and lds_addr wave-uniform).  Issued as inline assembly so
+// that the waits stay under this file's control: the kernel waits for exactly the stage
+// it is about to publish (vmcnt counts direct loads in order) and keeps two younger
+// stages in flight across its LDS reads.
+__device__ __forceinline__ void direct_load16(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+__device__ __forceinline__ void direct_load4(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
 
-__global__ __launch_bounds__(256) void mxfp4_a8_gemm_kernel(
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
     const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
-    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds_a[kBM * kARow];
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end) {
+  constexpr int kWaves = WM * WN;
+  static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BN % 64 == 0, "tile shape");
+  static_assert((BM / 8) % kWaves == 0 && (BN / 16) % kWaves == 0, "direct-load blocks divide among the wavefronts");
+  constexpr int kTI = BM / WM / 32, kTJ = BN / WN / 32;      // MFMA tiles per wavefront
+  constexpr int kABlk = BM / 8 / kWaves, kBBlk = BN / 16 / kWaves;  // 1 KB direct-load blocks per wavefront
+  constexpr int kDma = kABlk + kBBlk + 1;                    // direct loads a wavefront issues per stage
+  constexpr uint32_t kBBase = BM * kKS, kSBase = kBBase + BN * kKS / 2;
+  constexpr uint32_t kStage = kSBase + BN * 4;
+  __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kStage];
 
-  const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-  const uint32_t wm = wave >> 1, wn = wave & 1u;          // quadrant of the tile
-  const uint32_t m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t wm = wave / WN, wn = wave % WN;
   const uint32_t l32 = lane & 31u, kg = lane >> 5;        // MFMA row/column and K half
-  const uint8_t* scales = w + static_cast<size_t>(n) * k / 2;
   const uint32_t row_bytes = k / 2, row_blocks = k / 32;
+  const uint32_t tiles_n = (n_end - n_begin + BN - 1) / BN;
+  const uint32_t tiles = tiles_n * ((m + BM - 1) / BM);
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) uint8_t*)lds));
 
-  // Weight rows of this lane's two n-subtiles (clamped at the matrix edge; the stores
-  // are masked instead).
-  uint32_t wrow[2];
+  // Direct loads of one tile.  Activation block L (1 KB, rows 8L..8L+7, eight 16-byte chunks
+  // a row): lane p fetches row 8L + p/8, chunk (p%8) ^ ((row>>1)&7).  Weight block L (rows
+  // 16L..16L+15, four chunks a row): row 16L + p/4, chunk (p%4) ^ ((row>>2)&3).  Scale block
+  // (64 rows, one word a row): row 64L + p.  A wavefront moves kABlk + kBBlk + 1 blocks per
+  // stage; rows past the matrix edge are clamped to the last row (never stored).
+  struct Source {
+    const uint8_t *a, *b, *s;           // tile origins (wave-uniform)
+    uint32_t a_off[kABlk], b_off[kBBlk], s_off;
+  };
+  auto locate = [&](uint32_t tile, Source& src) {
+    const uint32_t m0 = (tile / tiles_n) * BM, n0 = n_begin + (tile % tiles_n) * BN;
+    src.a = a8 + static_cast<size_t>(m0) * k;
+    src.b = w + static_cast<size_t>(n0) * row_bytes;
+    src.s = w + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(n0) * row_blocks;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const uint32_t r = n0 + wn * 64u + j * 32u + l32;
-    wrow[j] = r < n ? r : n - 1u;
+    for (int i = 0; i < kABlk; ++i) {
+      const uint32_t row = 8u * (wave * kABlk + i) + lane / 8u;
+      const uint32_t chunk = (lane % 8u) ^ ((row >> 1) & 7u);
+      src.a_off[i] = (m0 + row < m ? row : m - 1u - m0) * k + chunk * 16u;
+    }
+#pragma unroll
+    for (int i = 0; i < kBBlk; ++i) {
+      const uint32_t row = 16u * (wave * kBBlk + i) + lane / 4u;
+      const uint32_t chunk = (lane % 4u) ^ ((row >> 2) & 3u);
+      src.b_off[i] = (n0 + row < n ? row : n - 1u - n0) * row_bytes + chunk * 16u;
+    }
+    const uint32_t row = 64u * (wave % (BN / 64)) + lane;
+    src.s_off = (n0 + row < n ? row : n - 1u - n0) * row_blocks;
+  };
+  auto issue_stage = [&](uint32_t stage_off, const Source& src, uint32_t k0) {
+    const uint32_t stage = lds_base + stage_off;
+    const uint8_t* ga = src.a + k0;
+    const uint8_t* gb = src.b + k0 / 2;
+    const uint8_t* gs = src.s + k0 / 32;
+#pragma unroll
+    for (int i = 0; i < kABlk; ++i) direct_load16(ga, src.a_off[i], stage + (wave * kABlk + i) * 1024u);
+#pragma unroll
+    for (int i = 0; i < kBBlk; ++i) direct_load16(gb, src.b_off[i], stage + kBBase + (wave * kBBlk + i) * 1024u);
+    direct_load4(gs, src.s_off, stage + kSBase + (wave % (BN / 64)) * 256u);
+  };
+
+  // Fragments of one 64-wide K slice.  8-bit A operand: a lane of K half `kg` supplies
+  // k = 16*kg + [0,16) in its first four registers and k = 32 + 16*kg + [0,16) in the last
+  // four (the instruction is two K=32 steps back to back), i.e. chunks 4*ks + kg and
+  // 4*ks + 2 + kg of its row; the 4-bit B operand is k = 32*kg + [0,32), chunk 2*ks + kg.
+  struct Frag {
+    int8v_t a[kTI];
+    uint4 b[kTJ];
+  };
+  uint32_t a_fr[2][2], b_fr[2];
+  {
+    const uint32_t row = wm * (BM / WM) + l32, swz = (l32 >> 1) & 7u;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int hi = 0; hi < 2; ++hi) a_fr[ks][hi] = row * 128u + (((ks * 4u + hi * 2u + kg) ^ swz) * 16u);
   }
-
-  auto load_b = [&](uint32_t k0, BFrag& f) {
+  {
+    const uint32_t row = wn * (BN / WN) + l32, swz = (l32 >> 2) & 3u;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const uint8_t* row = w + static_cast<size_t>(wrow[j]) * row_bytes + k0 / 2;
+    for (int ks = 0; ks < 2; ++ks) b_fr[ks] = kBBase + row * 64u + (((ks * 2u + kg) ^ swz) * 16u);
+  }
+  const uint32_t s_fr = kSBase + (wn * (BN / WN) + l32) * 4u;
+  auto read_frags = [&](uint32_t stage_off, int ks, Frag& f) {
+    const uint8_t* stage = lds + stage_off;
 #pragma unroll
-      for (int ks = 0; ks < kSteps; ++ks) {
-        f.q[ks][j] = load_u4(row + ks * 32 + kg * 16);   // block 2*ks + kg of this step
-      }
-      f.s[j] = *reinterpret_cast<const uint2*>(scales + static_cast<size_t>(wrow[j]) * row_blocks + k0 / 32);
+    for (int i = 0; i < kTI; ++i) {
+      const uint4 lo = *reinterpret_cast<const uint4*>(stage + a_fr[ks][0] + i * 32 * 128);
+      const uint4 hi = *reinterpret_cast<const uint4*>(stage + a_fr[ks][1] + i * 32 * 128);
+      f.a[i] = int8v_t{static_cast<int>(lo.x), static_cast<int>(lo.y), static_cast<int>(lo.z),
+                       static_cast<int>(lo.w), static_cast<int>(hi.x), static_cast<int>(hi.y),
+                       static_cast<int>(hi.z), static_cast<int>(hi.w)};
+    }
+#pragma unroll
+    for (int j = 0; j < kTJ; ++j) {
+      f.b[j] = *reinterpret_cast<const uint4*>(stage + b_fr[ks] + j * 32 * 64);
     }
   };
-
-  // Activation tile staging: thread t moves 16 bytes of row (t / 16) + 16 * i, i = 0..7.
-  const uint32_t a_col = (t & 15u) * 16u, a_row = t >> 4;
-  auto load_a = [&](uint32_t k0, uint4 (&r)[8]) {
+  // Scale words of this lane's weight rows; block 2*ks + kg sits at byte 2*ks once lanes of
+  // the upper K half have shifted their four bytes down by one (done at the use).
+  auto read_scales = [&](uint32_t stage_off, uint32_t (&raw)[kTJ]) {
+    const uint8_t* stage = lds + stage_off;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t row = m0 + a_row + 16u * i;
-      r[i] = row < m ? load_u4(a8 + static_cast<size_t>(row) * k + k0 + a_col) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto store_a = [&](const uint4 (&r)[8]) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      *reinterpret_cast<uint4*>(&lds_a[(a_row + 16u * i) * kARow + a_col]) = r[i];
-    }
+    for (int j = 0; j < kTJ; ++j) raw[j] = *reinterpret_cast<const uint32_t*>(stage + s_fr + j * 128);
   };
 
-  float16_t acc[2][2];
+  float16_t acc[kTI][kTJ];
+  auto mfmas = [&](const Frag& f, int ks, const int (&sv)[kTJ]) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < kTJ; ++j) {
+      const int8v_t bf = int8v_t{static_cast<int>(f.b[j].x), static_cast<int>(f.b[j].y),
+                                 static_cast<int>(f.b[j].z), static_cast<int>(f.b[j].w), 0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  BFrag bcur, bnext;
-  uint4 areg[8];
-  load_a(0, areg);
-  load_b(0, bcur);
-
-  for (uint32_t k0 = 0; k0 < k; k0 += kKS) {
-    __syncthreads();        // the previous step's fragment reads are done
-    store_a(areg);
-    __syncthreads();
-    const uint32_t kn = k0 + kKS;
-    if (kn < k) {           // uniform: prefetch the next step while this one computes
-      load_a(kn, areg);
-      load_b(kn, bnext);
-    }
-#pragma unroll
-    for (int ks = 0; ks < kSteps; ++ks) {
-      int8v_t af[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        // 8-bit A operand: a lane of K half `kg` supplies k = 16*kg + [0,16) in its first
-        // four registers and k = 32 + 16*kg + [0,16) in the last four (the instruction is
-        // two K=32 steps back to back); the 4-bit B operand is simply k = 32*kg + [0,32).
-        const uint8_t* p = &lds_a[(wm * 64u + i * 32u + l32) * kARow + ks * 64 + kg * 16u];
-        const uint4 lo = *reinterpret_cast<const uint4*>(p);
-        const uint4 hi = *reinterpret_cast<const uint4*>(p + 32);
-        af[i] = int8v_t{static_cast<int>(lo.x), static_cast<int>(lo.y), static_cast<int>(lo.z),
-                        static_cast<int>(lo.w), static_cast<int>(hi.x), static_cast<int>(hi.y),
-                        static_cast<int>(hi.z), static_cast<int>(hi.w)};
-      }
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const uint4 q = bcur.q[ks][j];
-        const int8v_t bf = int8v_t{static_cast<int>(q.x), static_cast<int>(q.y), static_cast<int>(q.z),
-                                   static_cast<int>(q.w), 0, 0, 0, 0};
-        // Scale byte of block 2*ks + kg: lanes of the upper K half shift their eight
-        // bytes down by one so that every lane finds it at byte 2*ks.
-        const uint64_t s64 = (static_cast<uint64_t>(bcur.s[j].y) << 32 | bcur.s[j].x) >> (kg * 8u);
-        const int sreg = static_cast<int>(ks < 2 ? static_cast<uint32_t>(s64) : static_cast<uint32_t>(s64 >> 32));
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          // A: E4M3 (cbsz 0) with unit scale (E8M0 127); B: E2M1 (blgp 4) with the block scale.
-          if ((ks & 1) == 0) {
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 0, sreg);
-          } else {
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 2, sreg);
-          }
+      for (int i = 0; i < kTI; ++i) {
+        // A: E4M3 (cbsz 0) with unit scale (E8M0 127); B: E2M1 (blgp 4) with the block scale.
+        if (ks == 0) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 0, sv[j]);
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 2, sv[j]);
         }
       }
     }
-    if (kn < k) bcur = bnext;
-  }
+  };
 
-  // Epilogue: lane holds column l32 and rows (e/4)*8 + kg*4 + e%4 of each 32 x 32 tile.
+  // Every wavefront waits for its own direct loads of the stage about to be published (all
+  // but the youngest stage's; loads complete in issue order, and stores issued in between
+  // only make the wait longer), and for its LDS reads of the stage about to be overwritten,
+  // before the barrier.
+  auto publish = [&]() {
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kDma) : "memory");
+  };
+
+  const uint32_t steps = k / kKS;
+  Frag f0, f1;
+  int sv[kTJ];
+  uint32_t sv_raw[kTJ];
+  uint32_t rd = 0, nx = kStage, fill = 2 * kStage;
+
+  // Persistent loop over this workgroup's tiles, flattened into one loop over K steps so
+  // that the ring of stages never drains: the load cursor runs two steps ahead of the
+  // multiply cursor and simply moves on to the next tile when a tile's K is exhausted, so
+  // the first loads and fragment reads of a tile run under the previous tile's epilogue.
+  // Past the last tile the cursor reloads a stage nobody reads rather than branching.
+  uint32_t tile = blockIdx.x;
+  if (tile >= tiles) return;
+  const uint32_t my_tiles = (tiles - tile + gridDim.x - 1) / gridDim.x;
+  Source src;
+  locate(tile, src);
+  uint32_t load_tile = tile, load_step = 0;
+  auto advance_load = [&]() {
+    if (++load_step == steps) {          // uniform
+      asm volatile("" ::: "memory");     // keeps this rare block a branch, not a chain of selects
+      load_step = 0;
+      load_tile += gridDim.x;
+      if (load_tile < tiles) locate(load_tile, src);
+    }
+  };
+  issue_stage(0, src, 0);
+  advance_load();
+  issue_stage(kStage, src, load_step * kKS);
+  advance_load();
+  publish();
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < kTI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const uint32_t col = n0 + wn * 64u + j * 32u + l32;
+    for (int j = 0; j < kTJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  for (uint32_t done_tiles = 0; done_tiles < my_tiles; ++done_tiles) {
+    for (uint32_t cur = 0; cur < steps; ++cur) {
+      // One step of K: `rd` is the stage being multiplied, `nx` the stage of the step after
+      // it and `fill` the one the load cursor's step goes into.  Two wavefronts share each
+      // SIMD, so one's fragment reads run under the other's MFMAs.
+      issue_stage(fill, src, load_step * kKS);
+      read_scales(rd, sv_raw);
+#pragma unroll
+      for (int j = 0; j < kTJ; ++j) sv[j] = static_cast<int>(sv_raw[j] >> (kg * 8u));
+      read_frags(rd, 0, f0);
+      read_frags(rd, 1, f1);
+      mfmas(f0, 0, sv);
+      mfmas(f1, 1, sv);
+      publish();
+      const uint32_t done = rd;
+      rd = nx;
+      nx = fill;
+      fill = done;
+      advance_load();
+    }
+
+    // Epilogue: lane holds column l32 and rows (e/4)*8 + kg*4 + e%4 of each 32 x 32 tile.
+    const uint32_t m0 = (tile / tiles_n) * BM, n0 = n_begin + (tile % tiles_n) * BN;
+    tile += gridDim.x;
+#pragma unroll
+    for (int i = 0; i < kTI; ++i) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const uint32_t row = m0 + wm * 64u + i * 32u + (e >> 2) * 8u + kg * 4u + (e & 3u);
-        if (row < m && col < n) c[static_cast<size_t>(row) * n + col] = acc[i][j][e] * as[row];
+        const uint32_t row = m0 + wm * (BM / WM) + i * 32u + (e >> 2) * 8u + kg * 4u + (e & 3u);
+        const float scale = as[row < m ? row : m - 1u];
+#pragma unroll
+        for (int j = 0; j < kTJ; ++j) {
+          const uint32_t col = n0 + wn * (BN / WN) + j * 32u + l32;
+          if (row < m && col < n_end) c[static_cast<size_t>(row) * n + col] = acc[i][j][e] * scale;
+        }
       }
     }
+#pragma unroll
+    for (int i = 0; i < kTI; ++i)
+#pragma unroll
+      for (int j = 0; j < kTJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
   }
+  // No direct load may still be writing LDS when the workgroup retires.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace
 
-bool gemm_mxfp4_a8_supported(uint64_t k) { return k % 256 == 0; }
+bool gemm_mxfp4_a8_supported(uint64_t k) { return k % 128 == 0; }
 
+namespace {
+
+template <int BM, int BN, int WM, int WN>
+void launch_range(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                  uint32_t k, uint32_t n_begin, uint32_t n_end, uint32_t max_groups, hipStream_t stream) {
+  const uint32_t tiles = ((m + BM - 1) / BM) * ((n_end - n_begin + BN - 1) / BN);
+  const uint32_t grid = tiles < max_groups ? tiles : max_groups;
+  hipLaunchKernelGGL((mxfp4_a8_gemm_kernel<BM, BN, WM, WN>), dim3(grid), dim3(64 * WM * WN), 0, stream,
+                     a8, as, w, c, m, n, k, n_begin, n_end);
+}
+
+}  // namespace
+
+// The bulk of C goes to persistent 256 x 256 tiles, whole rounds of one tile per CU; the
+// columns left over when the tile count is not a multiple of the CU count would keep a
+// few CUs busy for a whole extra round, so they are cut into 128 x 64 tiles that spread
+// over every CU instead (two such workgroups share a CU).
 hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
-  const dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
-  hipLaunchKernelGGL(mxfp4_a8_gemm_kernel, grid, dim3(256), 0, stream, a8, as, w, c, m, n, k);
+  const uint32_t cus = static_cast<uint32_t>(num_cus());
+  const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u;
+  const uint32_t tiles = tiles_m * tiles_n;
+  uint32_t main_tn = tiles_n;
+  if (tiles > cus && tiles % cus != 0 && tiles % cus <= cus / 2) {
+    main_tn = (tiles / cus) * cus / tiles_m;
+  } else if (tiles < cus / 2) {
+    main_tn = 0;                        // too few large tiles to fill the chip: small tiles throughout
+  }
+  const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
+  if (n_split > 0) launch_range<256, 256, 4, 2>(a8, as, w, c, m, n, k, 0u, n_split, cus, stream);
+  if (n_split < n) launch_range<128, 64, 2, 2>(a8, as, w, c, m, n, k, n_split, n, 2u * cus, stream);
   return hipGetLastError();
 }
 

@@ -871,6 +871,8 @@ hipError_t launch_gemv_generic(const typename Codec::Args& args, float* c, uint3
 
 }  // namespace
 
+int num_cus() { return g_num_cus; }
+
 void set_num_cus(int cus) {
   g_num_cus = cus > 0 ? cus : 256;
   if (const char* e = std::getenv("QMM_GEMV_P")) g_tune_p = std::atoi(e);

@@ -11,6 +11,7 @@
 namespace qmm {
 
 void set_num_cus(int cus);
+int num_cus();
 
 // ---- decode GEMV family (gemv.hip) -----------------------------------------
 bool gemv_q4k_supported(uint64_t k);

@@ -70,8 +70,45 @@ u128 mxfp4_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * k / 2 +
 // regime table (src/models/qwen3_5/project.cpp:233-366); every Q4_K GEMM id has the
 // same buffers and m, n, k scalars, so each id accepts every m and picks the gfx950
 // kernel that fits it.
+// Device scratch owned by the library (the fp16 copy of the activations that the Q4_K MFMA
+// GEMM reads).  Grown on demand and kept until the process ends; growing synchronises the
+// device (hipFree), so the first large prefill call must not sit inside a stream capture.
+// Launches that use it are ordered by the caller's stream, as everything else here.
+void* g_workspace = nullptr;
+size_t g_workspace_bytes = 0;
+std::mutex g_workspace_mutex;
+
+qmm_status workspace(size_t bytes, void** out) {
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  if (bytes > g_workspace_bytes) {
+    if (g_workspace != nullptr) (void)hipFree(g_workspace);
+    g_workspace = nullptr;
+    g_workspace_bytes = 0;
+    const size_t want = (bytes + (size_t{1} << 24) - 1) & ~((size_t{1} << 24) - 1);
+    const hipError_t e = hipMalloc(&g_workspace, want);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return map_hip(e);
+    }
+    g_workspace_bytes = want;
+  }
+  *out = g_workspace;
+  return QMM_OK;
+}
+
+// From this many rows on, Q4_K goes to the fp16 MFMA GEMM; below, the bandwidth-bound GEMV
+// reads each weight once per group of up to four rows.
+constexpr uint64_t kQ4KGemmMinRows = 24;
+
 qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
                       uint64_t k, hipStream_t s) {
+  if (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) {
+    void* ws = nullptr;
+    const qmm_status st = workspace(qmm::gemm_q4k_workspace_bytes(m, k), &ws);
+    if (st != QMM_OK) return st;
+    return map_hip(qmm::launch_q4k_gemm(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                        static_cast<uint32_t>(k), s));
+  }
   if (!qmm::gemv_q4k_supported(k)) {
     g_last_error = "Q4_K: k above 32768 is not implemented";
     return QMM_UNSUPPORTED_FEATURE;

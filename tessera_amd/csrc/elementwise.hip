@@ -196,6 +196,89 @@ __global__ __launch_bounds__(256) void moe_scale_add_kernel(const float* __restr
   if (i < n) o[i] = a[i] + f[idx] * b[i];
 }
 
+// "moe_gate" (src/backends/rocm/rocm_kernels_basic.cpp:1896-1929): softmax over the top_k
+// selected router logits, and the shared expert's sigmoid gate sig = sigmoid(x . w).
+// One workgroup; same summation tree as the reference (strided partials, then halving).
+__global__ __launch_bounds__(256) void moe_gate_kernel(const float* __restrict__ vals,
+                                                       const float* __restrict__ x,
+                                                       const float* __restrict__ w,
+                                                       float* __restrict__ wts, float* __restrict__ sig,
+                                                       uint32_t top_k, uint32_t hidden) {
+  __shared__ float red[256];
+  const uint32_t tid = threadIdx.x;
+  float dot = 0.0f;
+  for (uint32_t t = tid; t < hidden; t += 256u) dot += x[t] * w[t];
+  red[tid] = dot;
+  __syncthreads();
+  for (uint32_t s = 128u; s > 0u; s >>= 1) {
+    if (tid < s) red[tid] += red[tid + s];
+    __syncthreads();
+  }
+  if (tid == 0u) {
+    float m = -3.402823466e+38f;
+    for (uint32_t p = 0; p < top_k; ++p) m = fmaxf(m, vals[p]);
+    float sum = 0.0f;
+    for (uint32_t p = 0; p < top_k; ++p) sum += expf(vals[p] - m);
+    for (uint32_t p = 0; p < top_k; ++p) wts[p] = expf(vals[p] - m) / sum;
+    sig[0] = 1.0f / (1.0f + expf(-red[0]));
+  }
+}
+
+// "top_k_rows" (src/backends/rocm/rocm_kernels_basic.cpp:3176-3243): per-row top-k of
+// `vocab` fp32 logits in descending order, one workgroup per row.  Pass p selects the
+// largest value not yet taken; ties go to the earlier column inside a thread's strided
+// share and to the lower thread across threads, as in the reference's strict-greater merge.
+__global__ __launch_bounds__(256) void top_k_rows_kernel(const float* __restrict__ logits,
+                                                         uint32_t* __restrict__ ids,
+                                                         float* __restrict__ vals, uint64_t vocab,
+                                                         uint32_t top_k, uint64_t row_base) {
+  __shared__ float rv[256];
+  __shared__ uint32_t ri[256];
+  __shared__ uint32_t rown[256];
+  const uint32_t tid = threadIdx.x;
+  const float* row = logits + (row_base + blockIdx.x) * vocab;
+  // Columns this thread has already given away: they are the thread's largest, in order, so
+  // "not yet taken" is "smaller than the last one given, or equal to it at a later column".
+  float last_v = 0.0f;
+  uint64_t last_c = 0;
+  bool any = false;
+  for (uint32_t p = 0; p < top_k; ++p) {
+    float best = -INFINITY;
+    uint64_t best_c = ~0ull;
+    for (uint64_t c = tid; c < vocab; c += 256u) {
+      const float v = row[c];
+      const bool open = !any || v < last_v || (v == last_v && c > last_c);
+      if (open && (best_c == ~0ull || v > best)) {
+        best = v;
+        best_c = c;
+      }
+    }
+    rv[tid] = best_c != ~0ull ? best : -INFINITY;
+    ri[tid] = best_c != ~0ull ? static_cast<uint32_t>(best_c) : 0u;
+    rown[tid] = tid;
+    __syncthreads();
+    for (uint32_t s = 128u; s > 0u; s >>= 1) {
+      if (tid < s && rv[tid + s] > rv[tid]) {
+        rv[tid] = rv[tid + s];
+        ri[tid] = ri[tid + s];
+        rown[tid] = rown[tid + s];
+      }
+      __syncthreads();
+    }
+    if (tid == 0u) {
+      vals[static_cast<size_t>(blockIdx.x) * top_k + p] = rv[0];
+      ids[static_cast<size_t>(blockIdx.x) * top_k + p] = ri[0];
+    }
+    const uint32_t owner = rown[0];
+    __syncthreads();
+    if (tid == owner && best_c != ~0ull) {
+      last_v = best;
+      last_c = best_c;
+      any = true;
+    }
+  }
+}
+
 inline dim3 grid_for(uint64_t count, uint32_t per_block) {
   return dim3(static_cast<uint32_t>((count + per_block - 1) / per_block));
 }
@@ -260,6 +343,19 @@ hipError_t launch_moe_scale_add(const float* a, const float* b, const float* f, 
                                 uint64_t n, uint64_t idx, hipStream_t stream) {
   hipLaunchKernelGGL(moe_scale_add_kernel, grid_for(n, 256), dim3(256), 0, stream, a, b, f, o, n,
                      idx);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_gate(const float* vals, const float* x, const float* w, float* wts, float* sig,
+                           uint32_t top_k, uint32_t hidden, hipStream_t stream) {
+  hipLaunchKernelGGL(moe_gate_kernel, dim3(1), dim3(256), 0, stream, vals, x, w, wts, sig, top_k, hidden);
+  return hipGetLastError();
+}
+
+hipError_t launch_top_k_rows(const float* logits, uint32_t* ids, float* vals, uint32_t rows,
+                             uint64_t vocab, uint32_t top_k, uint64_t row_base, hipStream_t stream) {
+  hipLaunchKernelGGL(top_k_rows_kernel, dim3(rows), dim3(256), 0, stream, logits, ids, vals, vocab, top_k,
+                     row_base);
   return hipGetLastError();
 }
 

@@ -192,6 +192,115 @@ struct Q4KCodec {
 };
 
 // ----------------------------------------------------------------------------
+// Routed-expert variants of the Q4_K codec (mixture-of-experts feed-forward; reference
+// kernels src/backends/rocm/rocm_kernels_moe.cpp:15-79, launch protocol
+// src/models/qwen3_5/moe.cpp:396-423).  Expert tensors are expert-major: expert e of a
+// tensor starts `stride` bytes after expert e-1, rows inside it are ordinary Q4_K rows.
+// The selected expert ids live in device memory, so the weight row is looked up in the
+// kernel.  `batch` moves every per-token pointer to token y (grid.y).
+// ----------------------------------------------------------------------------
+
+// Gate or up projection of the `top_k` selected experts: output row slot*inter + j is row j
+// of expert ids[slot].  With `gate_out` set this is the up pass and the stored value is
+// silu(gate_out[row]) * (U x)[row]: the gate pass wrote gate_out, so two launches leave phi.
+struct Q4KExpertUpCodec : Q4KCodec {
+  struct Args {
+    const float* a;
+    const uint8_t* w;
+    uint32_t k;            // hidden
+    const uint32_t* ids;
+    uint64_t stride;
+    uint32_t inter, top_k;
+    uint32_t n_experts;    // ids are clamped below this, so a bad id cannot leave the tensor
+    const float* gate_out;
+  };
+  static __device__ __forceinline__ void batch(Args& p, uint32_t y) {
+    p.a += static_cast<size_t>(y) * p.k;
+    p.ids += static_cast<size_t>(y) * p.top_k;
+    if (p.gate_out != nullptr) p.gate_out += static_cast<size_t>(y) * p.top_k * p.inter;
+  }
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    Q4KCodec::load_x<R>(Q4KCodec::Args{p.a, p.w, p.k}, chunk, valid, x, src);
+  }
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk, uint32_t prow) {
+    return Q4KCodec::make_lane(Q4KCodec::Args{}, cpr, chunk, prow);
+  }
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row, uint32_t cpr,
+                                              Frag& f) {
+    const uint32_t slot = row / p.inter, j = row - slot * p.inter;
+    const uint32_t e = p.ids[slot] < p.n_experts ? p.ids[slot] : p.n_experts - 1u;
+    const uint8_t* base = p.w + e * p.stride + static_cast<size_t>(j) * ((cpr >> 3) * 144u);
+    f.h = load_u4(base + ln.off0);
+    f.q = load_u4(base + ln.off1);
+  }
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args& p, uint32_t row, int, float v) {
+    if (p.gate_out == nullptr) return v;
+    const float g = p.gate_out[row];
+    return (g / (1.0f + expf(-g))) * v;
+  }
+};
+
+// Down projection of the selected experts, summed with the routing weights:
+// out[j] = sum_slot wts[slot] * (D_ids[slot] phi_slot)[j].  One output row is treated as a
+// single dot product over K = top_k * inter whose weight blocks come from top_k experts and
+// whose activations (phi, contiguous slot by slot) are scaled by their slot's weight.
+struct Q4KExpertDownCodec : Q4KCodec {
+  struct Args {
+    const float* a;        // phi, top_k x inter
+    const uint8_t* w;
+    uint32_t k;            // top_k * inter
+    const uint32_t* ids;
+    uint64_t stride;
+    uint32_t inter, top_k, hidden;
+    uint32_t n_experts;    // ids are clamped below this
+    const float* wts;
+    const float* prev;     // the output itself when accumulating, else null
+  };
+  static __device__ __forceinline__ void batch(Args& p, uint32_t y) {
+    p.a += static_cast<size_t>(y) * p.k;
+    p.ids += static_cast<size_t>(y) * p.top_k;
+    p.wts += static_cast<size_t>(y) * p.top_k;
+    if (p.prev != nullptr) p.prev += static_cast<size_t>(y) * p.hidden;
+  }
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    Q4KCodec::load_x<R>(Q4KCodec::Args{p.a, p.w, p.k}, chunk, valid, x, src);
+    const float wt = p.wts[chunk / (p.inter / 32u)];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        x.lo[r][i] *= wt;
+        x.hi[r][i] *= wt;
+      }
+      x.slo[r] *= wt;
+      x.shi[r] *= wt;
+    }
+  }
+  // Offsets are relative to row 0 of expert 0; they stay below 4 GB (checked by the caller).
+  static __device__ __forceinline__ Lane make_lane(const Args& p, uint32_t, uint32_t chunk, uint32_t prow) {
+    const uint32_t per_slot = p.inter / 32u, slot = chunk / per_slot, cin = chunk - slot * per_slot;
+    const uint32_t e = p.ids[slot] < p.n_experts ? p.ids[slot] : p.n_experts - 1u;
+    const uint32_t hdr = static_cast<uint32_t>(e * p.stride) + prow * (p.inter / 256u) * 144u +
+                         (cin >> 3) * 144u;
+    return Lane{hdr, hdr + 16u + (cin & 7u) * 16u};
+  }
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row, uint32_t, Frag& f) {
+    const uint8_t* base = p.w + static_cast<size_t>(row) * ((p.inter / 256u) * 144u);
+    f.h = load_u4(base + ln.off0);
+    f.q = load_u4(base + ln.off1);
+  }
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args& p, uint32_t row, int, float v) {
+    return p.prev != nullptr ? p.prev[row] + v : v;
+  }
+};
+
+// ----------------------------------------------------------------------------
 // Q4_K, single activation row: the same arithmetic with a 32-byte chunk per thread
 // (one whole group g of a block: sub-block 2g in the low nibbles, 2g+1 in the high
 // nibbles), so the header decode, the cross-lane reduction and the loop overhead are
@@ -841,6 +950,10 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args 
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (row >= n) return;  // whole wavefront leaves together
+  if constexpr (requires { Codec::batch(args, 0u); }) {   // one activation row per grid.y
+    Codec::batch(args, blockIdx.y);
+    c += static_cast<size_t>(blockIdx.y) * ldc;
+  }
   float acc = 0.0f;
   for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
     typename Codec::template X<1> x;
@@ -976,6 +1089,33 @@ hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, flo
     r0 += took;
   }
   return hipSuccess;
+}
+
+// ---- mixture-of-experts (Q4_K experts) ------------------------------------------------
+
+hipError_t launch_moe_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up,
+                                  const uint32_t* ids, float* phi, uint32_t hidden, uint32_t inter,
+                                  uint32_t top_k, uint64_t gate_stride, uint64_t up_stride,
+                                  uint32_t n_experts, uint32_t rows, hipStream_t stream) {
+  const uint32_t n = top_k * inter, cpr = Q4KCodec::chunks_per_row(hidden);
+  const dim3 grid((n + 3u) / 4u, rows);
+  Q4KExpertUpCodec::Args g{x, gate, hidden, ids, gate_stride, inter, top_k, n_experts, nullptr};
+  hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertUpCodec>), grid, dim3(256), 0, stream, g, phi, n, cpr, n);
+  Q4KExpertUpCodec::Args u{x, up, hidden, ids, up_stride, inter, top_k, n_experts, phi};
+  hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertUpCodec>), grid, dim3(256), 0, stream, u, phi, n, cpr, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_down_q4k(const float* phi, const uint8_t* down, const uint32_t* ids,
+                               const float* wts, float* out, uint32_t hidden, uint32_t inter,
+                               uint32_t top_k, uint64_t down_stride, bool accumulate, uint32_t n_experts,
+                               uint32_t rows, hipStream_t stream) {
+  const uint32_t k = top_k * inter, cpr = Q4KCodec::chunks_per_row(k);
+  Q4KExpertDownCodec::Args a{phi, down, k, ids, down_stride, inter, top_k, hidden, n_experts, wts,
+                             accumulate ? out : nullptr};
+  hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertDownCodec>), dim3((hidden + 3u) / 4u, rows), dim3(256), 0,
+                     stream, a, out, hidden, cpr, hidden);
+  return hipGetLastError();
 }
 
 }  // namespace qmm

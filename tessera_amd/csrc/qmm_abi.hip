@@ -339,6 +339,105 @@ qmm_status run_moe_scale_add(const LaunchCtx& c) {
                                            c.ptr<float>(3), n, idx, c.stream));
 }
 
+// ---- routed experts ------------------------------------------------------------------
+// "moe_experts_gate_up_q4k": buffers x, gate, up, ids, phi; scalars hidden, inter, top_k,
+// gate_stride, up_stride (src/backends/rocm/rocm_kernels_moe.cpp:15-47;
+// src/models/qwen3_5/moe.cpp:396-404).  "..._rows" (not a reference id) adds a trailing
+// scalar `rows`: x is rows x hidden, ids rows x top_k, phi rows x top_k x inter, one token
+// per row in a single launch.
+qmm_status run_moe_gate_up_n(const LaunchCtx& c, bool batched) {
+  if (!counts(c, 5, batched ? 6 : 5)) return bad("moe_experts_gate_up_q4k: expects 5 buffers and 5 (6) scalars");
+  const uint64_t hidden = c.sc[0], inter = c.sc[1], top_k = c.sc[2], gs = c.sc[3], us = c.sc[4];
+  const uint64_t rows = batched ? c.sc[5] : 1;
+  if (hidden == 0 || inter == 0 || hidden % 256 != 0 || inter % 256 != 0 || hidden > (1u << 20) ||
+      inter > (1u << 20) || top_k == 0 || top_k > 64 || rows == 0 || rows > 65535) {
+    return bad("moe_experts_gate_up_q4k: bad hidden, inter, top_k or rows");
+  }
+  const u128 expert = q4k_bytes(inter, hidden);
+  if (gs < expert || us < expert) return bad("moe_experts_gate_up_q4k: expert stride smaller than one expert");
+  if (!c.fits(0, static_cast<u128>(rows) * hidden * 4) || !c.fits(1, expert) || !c.fits(2, expert) ||
+      !c.fits(3, static_cast<u128>(rows) * top_k * 4) || !c.fits(4, static_cast<u128>(rows) * top_k * inter * 4)) {
+    return bad("moe_experts_gate_up_q4k: a buffer is smaller than the shape requires");
+  }
+  // Experts the smaller of the two tensors holds (all of them when sizes were not given).
+  uint64_t experts = 0xFFFFFFFFull;
+  if (c.bytes != nullptr) {
+    const uint64_t eg = (c.bytes[1] - static_cast<uint64_t>(expert)) / gs + 1, eu = (c.bytes[2] - static_cast<uint64_t>(expert)) / us + 1;
+    experts = eg < eu ? eg : eu;
+    if (experts > 0xFFFFFFFFull) experts = 0xFFFFFFFFull;
+  }
+  return map_hip(qmm::launch_moe_gate_up_q4k(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint8_t>(2),
+                                             c.ptr<const uint32_t>(3), c.ptr<float>(4), static_cast<uint32_t>(hidden),
+                                             static_cast<uint32_t>(inter), static_cast<uint32_t>(top_k), gs, us,
+                                             static_cast<uint32_t>(experts), static_cast<uint32_t>(rows), c.stream));
+}
+qmm_status run_moe_gate_up(const LaunchCtx& c) { return run_moe_gate_up_n(c, false); }
+qmm_status run_moe_gate_up_rows(const LaunchCtx& c) { return run_moe_gate_up_n(c, true); }
+
+// "moe_experts_down_q4k": buffers phi, down, ids, wts, out; scalars hidden, inter, top_k,
+// down_stride, accumulate (src/backends/rocm/rocm_kernels_moe.cpp:49-79;
+// src/models/qwen3_5/moe.cpp:413-423).  "..._rows" adds a trailing `rows` as above.
+qmm_status run_moe_down_n(const LaunchCtx& c, bool batched) {
+  if (!counts(c, 5, batched ? 6 : 5)) return bad("moe_experts_down_q4k: expects 5 buffers and 5 (6) scalars");
+  const uint64_t hidden = c.sc[0], inter = c.sc[1], top_k = c.sc[2], ds = c.sc[3], acc = c.sc[4];
+  const uint64_t rows = batched ? c.sc[5] : 1;
+  if (hidden == 0 || inter == 0 || inter % 256 != 0 || hidden > (1u << 24) || inter > (1u << 20) ||
+      top_k == 0 || top_k > 64 || top_k * inter / 32 > 32768 || rows == 0 || rows > 65535) {
+    return bad("moe_experts_down_q4k: bad hidden, inter, top_k or rows");
+  }
+  if (ds < q4k_bytes(hidden, inter)) return bad("moe_experts_down_q4k: expert stride smaller than one expert");
+  if (!c.fits(0, static_cast<u128>(rows) * top_k * inter * 4) || !c.fits(1, q4k_bytes(hidden, inter)) ||
+      !c.fits(2, static_cast<u128>(rows) * top_k * 4) || !c.fits(3, static_cast<u128>(rows) * top_k * 4) ||
+      !c.fits(4, static_cast<u128>(rows) * hidden * 4)) {
+    return bad("moe_experts_down_q4k: a buffer is smaller than the shape requires");
+  }
+  if (c.bytes != nullptr && c.bytes[1] >= (1ull << 32)) {
+    g_last_error = "moe_experts_down_q4k: expert tensors of 4 GB and more are not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  uint64_t experts = 0xFFFFFFFFull;
+  if (c.bytes != nullptr) experts = (c.bytes[1] - static_cast<uint64_t>(q4k_bytes(hidden, inter))) / ds + 1;
+  return map_hip(qmm::launch_moe_down_q4k(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint32_t>(2),
+                                          c.ptr<const float>(3), c.ptr<float>(4), static_cast<uint32_t>(hidden),
+                                          static_cast<uint32_t>(inter), static_cast<uint32_t>(top_k), ds, acc != 0,
+                                          static_cast<uint32_t>(experts), static_cast<uint32_t>(rows), c.stream));
+}
+qmm_status run_moe_down(const LaunchCtx& c) { return run_moe_down_n(c, false); }
+qmm_status run_moe_down_rows(const LaunchCtx& c) { return run_moe_down_n(c, true); }
+
+// "moe_gate": buffers vals (top_k), x, w (hidden), wts (top_k), sig (1); scalars top_k, hidden
+// (src/backends/rocm/rocm_kernels_basic.cpp:1896-1929).
+qmm_status run_moe_gate(const LaunchCtx& c) {
+  if (!counts(c, 5, 2)) return bad("moe_gate: expects 5 buffers and 2 scalars");
+  const uint64_t top_k = c.sc[0], hidden = c.sc[1];
+  if (top_k == 0 || top_k > 4096 || hidden == 0 || hidden > (1u << 24)) return bad("moe_gate: bad top_k or hidden");
+  if (!c.fits(0, top_k * 4) || !c.fits(1, hidden * 4) || !c.fits(2, hidden * 4) || !c.fits(3, top_k * 4) ||
+      !c.fits(4, 4)) {
+    return bad("moe_gate: buffer too small");
+  }
+  return map_hip(qmm::launch_moe_gate(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<const float>(2),
+                                      c.ptr<float>(3), c.ptr<float>(4), static_cast<uint32_t>(top_k),
+                                      static_cast<uint32_t>(hidden), c.stream));
+}
+
+// "top_k_rows": buffers logits, ids, vals; scalars rows, vocab, top_k, row_base
+// (src/backends/rocm/rocm_kernels_basic.cpp:3170-3243; top_k is at most 32 there).
+qmm_status run_top_k_rows(const LaunchCtx& c) {
+  if (!counts(c, 3, 4)) return bad("top_k_rows: expects 3 buffers and 4 scalars");
+  const uint64_t rows = c.sc[0], vocab = c.sc[1], top_k = c.sc[2], base = c.sc[3];
+  if (rows == 0 || rows > kMaxDim || vocab == 0 || vocab > kMaxDim || top_k == 0 || top_k > 32 || top_k > vocab ||
+      base > kMaxDim) {
+    return bad("top_k_rows: bad rows, vocab, top_k (1..32) or row_base");
+  }
+  if (!c.fits(0, static_cast<u128>(base + rows) * vocab * 4) || !c.fits(1, static_cast<u128>(rows) * top_k * 4) ||
+      !c.fits(2, static_cast<u128>(rows) * top_k * 4)) {
+    return bad("top_k_rows: buffer too small");
+  }
+  return map_hip(qmm::launch_top_k_rows(c.ptr<const float>(0), c.ptr<uint32_t>(1), c.ptr<float>(2),
+                                        static_cast<uint32_t>(rows), vocab, static_cast<uint32_t>(top_k), base,
+                                        c.stream));
+}
+
 struct Entry {
   const char* id;
   qmm_fn fn;
@@ -366,6 +465,12 @@ const Entry kTable[] = {
     {"quantize_fp8_pack_rows", run_quantize_fp8_pack},
     {"gemm_fp8", run_gemm_fp8},
     {"moe_scale_add", run_moe_scale_add},
+    {"moe_experts_gate_up_q4k", run_moe_gate_up},
+    {"moe_experts_down_q4k", run_moe_down},
+    {"moe_experts_gate_up_q4k_rows", run_moe_gate_up_rows},
+    {"moe_experts_down_q4k_rows", run_moe_down_rows},
+    {"moe_gate", run_moe_gate},
+    {"top_k_rows", run_top_k_rows},
     {"dequant_q4k", run_dequant_q4k},
     {"dequant_mxfp4", run_dequant_mxfp4},
     {"quantize_fp8_pack_a16", run_quantize_fp8_pack_a16},

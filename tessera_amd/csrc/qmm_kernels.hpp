@@ -31,6 +31,18 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream);
 
+// ---- routed experts, Q4_K (gemv.hip) ----------------------------------------------
+// phi[t][slot*inter + j] = silu(G_e x_t)[j] * (U_e x_t)[j], e = ids[t][slot]; `rows` tokens.
+hipError_t launch_moe_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up,
+                                  const uint32_t* ids, float* phi, uint32_t hidden, uint32_t inter,
+                                  uint32_t top_k, uint64_t gate_stride, uint64_t up_stride,
+                                  uint32_t n_experts, uint32_t rows, hipStream_t stream);
+// out[t][j] (+)= sum_slot wts[t][slot] * (D_e phi[t][slot])[j].
+hipError_t launch_moe_down_q4k(const float* phi, const uint8_t* down, const uint32_t* ids,
+                               const float* wts, float* out, uint32_t hidden, uint32_t inter,
+                               uint32_t top_k, uint64_t down_stride, bool accumulate, uint32_t n_experts,
+                               uint32_t rows, hipStream_t stream);
+
 // ---- MFMA GEMMs (gemm_mxfp4.hip, gemm_q4k.hip) --------------------------------------
 bool gemm_mxfp4_a8_supported(uint64_t k);
 // W4A8 on the scaled MFMA: A = m x k E4M3 codes + per-row scales, W packed MXFP4.
@@ -58,6 +70,10 @@ hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uin
 hipError_t launch_dequant_q4k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream);
 hipError_t launch_dequant_mxfp4(const uint8_t* w, float* out, uint64_t n, uint64_t k,
                                 hipStream_t stream);
+hipError_t launch_moe_gate(const float* vals, const float* x, const float* w, float* wts, float* sig,
+                           uint32_t top_k, uint32_t hidden, hipStream_t stream);
+hipError_t launch_top_k_rows(const float* logits, uint32_t* ids, float* vals, uint32_t rows,
+                             uint64_t vocab, uint32_t top_k, uint64_t row_base, hipStream_t stream);
 hipError_t launch_moe_scale_add(const float* a, const float* b, const float* f, float* o,
                                 uint64_t n, uint64_t idx, hipStream_t stream);
 

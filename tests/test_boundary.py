@@ -19,7 +19,8 @@ REFERENCE_IDS = [
     "gemm_q4k_rows5", "gemm_q4k_batched", "gemm_q4k_wmma", "gemm_vec_reduce", "gemm_mxfp4",
     "gemm_mxfp4_rows", "gemm_mxfp4_batched", "mxfp4_row_ref", "gemm_mxfp4_wmma",
     "gemm_mxfp4_wmma_reduce", "quantize_fp8", "quantize_fp8_pack", "quantize_fp8_pack_rows",
-    "gemm_fp8", "moe_scale_add",
+    "gemm_fp8", "moe_scale_add", "moe_experts_gate_up_q4k", "moe_experts_down_q4k", "moe_gate",
+    "top_k_rows",
 ]
 
 

@@ -1,0 +1,138 @@
+"""Routed-expert (mixture-of-experts) Q4_K path on the GPU against the CPU oracle, through the
+C ABI: top_k_rows -> moe_gate -> moe_experts_gate_up_q4k -> moe_experts_down_q4k, the ids and
+launch protocol of src/models/qwen3_5/moe.cpp:396-423, plus the *_rows forms that run a whole
+chunk of tokens in one launch.  Routing (ids) must match exactly; routing weights, phi and the
+routed sum are fp32-accumulate paths held to the 1e-3 bound of tests/util.py:rel_err."""
+import numpy as np
+import pytest
+
+import oracle
+from tessera_amd import synth
+from util import rel_err, run
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def expert_tensors(g, experts, hidden, inter):
+    gate = np.concatenate([synth.q4k_weights(g, inter, hidden) for _ in range(experts)])
+    up = np.concatenate([synth.q4k_weights(g, inter, hidden) for _ in range(experts)])
+    down = np.concatenate([synth.q4k_weights(g, hidden, inter) for _ in range(experts)])
+    return gate, up, down
+
+
+def silu(v):
+    v = v.astype(np.float32)
+    with np.errstate(over="ignore"):
+        return (v / (np.float32(1) + np.exp(-v, dtype=np.float32))).astype(np.float32)
+
+
+@pytest.mark.parametrize("experts,hidden,inter,top_k", [(16, 512, 256, 4), (8, 2048, 512, 8), (5, 256, 768, 2)])
+def test_decode_row_matches_oracle(backend, experts, hidden, inter, top_k):
+    g = synth.rng(experts * 100 + hidden + inter)
+    gate, up, down = expert_tensors(g, experts, hidden, inter)
+    x = synth.activations_bf16(g, 1, hidden)
+    logits = g.standard_normal(size=(1, experts)).astype(np.float32)
+    gs, ds = gate.size // experts, down.size // experts
+
+    d_logits = backend.Upload(logits)
+    d_ids, d_vals = backend.AllocateBuffer(4 * top_k), backend.AllocateBuffer(4 * top_k)
+    run(backend, "top_k_rows", [d_logits, d_ids, d_vals], [1, experts, top_k, 0], grid=(1, 1, 1))
+    d_x, d_wsh = backend.Upload(x), backend.Upload(synth.activations_f32(g, 1, hidden))
+    d_wts, d_sig = backend.AllocateBuffer(4 * top_k), backend.AllocateBuffer(4)
+    run(backend, "moe_gate", [d_vals, d_x, d_wsh, d_wts, d_sig], [top_k, hidden], grid=(1, 1, 1))
+    d_gate, d_up, d_down = backend.Upload(gate), backend.Upload(up), backend.Upload(down)
+    d_phi = backend.AllocateBuffer(4 * top_k * inter)
+    run(backend, "moe_experts_gate_up_q4k", [d_x, d_gate, d_up, d_ids, d_phi], [hidden, inter, top_k, gs, gs],
+        grid=((inter * top_k + 7) // 8, 1, 1))
+    d_out = backend.Upload(np.full(hidden, 3.0, dtype=np.float32))
+    run(backend, "moe_experts_down_q4k", [d_phi, d_down, d_ids, d_wts, d_out], [hidden, inter, top_k, ds, 0],
+        grid=((hidden + 7) // 8, 1, 1))
+    backend.Synchronize()
+
+    ids = backend.CopyD2H(d_ids, dtype=np.uint32)
+    vals = backend.CopyD2H(d_vals, dtype=np.float32)
+    want_ids, want_vals = oracle.top_k_row(logits[0], top_k)
+    assert np.array_equal(ids, want_ids) and np.array_equal(vals, want_vals)
+    wts = backend.CopyD2H(d_wts, dtype=np.float32)
+    want_wts = oracle.moe_gate(want_vals)
+    assert np.allclose(wts, want_wts, rtol=1e-5) and abs(float(wts.sum()) - 1.0) < 1e-5
+    sig = backend.CopyD2H(d_sig, dtype=np.float32)[0]
+    wsh = backend.CopyD2H(d_wsh, dtype=np.float32)
+    dot = float(np.dot(x[0].astype(np.float64), wsh.astype(np.float64)))
+    assert abs(sig - 1.0 / (1.0 + np.exp(-dot))) < 1e-5
+
+    phi = backend.CopyD2H(d_phi, dtype=np.float32).reshape(top_k, inter)
+    for s, e in enumerate(want_ids):
+        ge = oracle.gemm_q4k(x, gate[e * gs:(e + 1) * gs], 1, inter, hidden)[0]
+        ue = oracle.gemm_q4k(x, up[e * gs:(e + 1) * gs], 1, inter, hidden)[0]
+        assert rel_err(phi[s], silu(ge) * ue) <= TOL, (s, rel_err(phi[s], silu(ge) * ue))
+    out = backend.CopyD2H(d_out, dtype=np.float32)
+    ref = oracle.moe_batch_forward_q4k(x, want_ids, want_wts, gate, up, down, hidden, inter)[0]
+    assert rel_err(out, ref) <= TOL, rel_err(out, ref)
+
+    # accumulate = 1 adds the routed sum to what the output already holds
+    run(backend, "moe_experts_down_q4k", [d_phi, d_down, d_ids, d_wts, d_out], [hidden, inter, top_k, ds, 1],
+        grid=((hidden + 7) // 8, 1, 1))
+    backend.Synchronize()
+    twice = backend.CopyD2H(d_out, dtype=np.float32)
+    assert rel_err(twice, 2 * ref) <= TOL
+
+
+def forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts):
+    rows, top_k = ids.shape
+    gs, ds = gate.size // experts, down.size // experts
+    d_x, d_ids, d_wts = backend.Upload(x), backend.Upload(ids), backend.Upload(wts)
+    d_gate, d_up, d_down = backend.Upload(gate), backend.Upload(up), backend.Upload(down)
+    d_phi = backend.AllocateBuffer(4 * rows * top_k * inter)
+    d_out = backend.AllocateBuffer(4 * rows * hidden)
+    run(backend, "moe_experts_gate_up_q4k_rows", [d_x, d_gate, d_up, d_ids, d_phi],
+        [hidden, inter, top_k, gs, gs, rows], grid=((inter * top_k + 7) // 8, rows, 1))
+    run(backend, "moe_experts_down_q4k_rows", [d_phi, d_down, d_ids, d_wts, d_out],
+        [hidden, inter, top_k, ds, 0, rows], grid=((hidden + 7) // 8, rows, 1))
+    backend.Synchronize()
+    return backend.CopyD2H(d_out, dtype=np.float32).reshape(rows, hidden)
+
+
+@pytest.mark.parametrize("rows,experts,hidden,inter,top_k", [(7, 16, 512, 256, 4), (33, 12, 256, 512, 3)])
+def test_rows_match_oracle(backend, rows, experts, hidden, inter, top_k):
+    g = synth.rng(rows + experts + hidden)
+    gate, up, down = expert_tensors(g, experts, hidden, inter)
+    x = synth.activations_bf16(g, rows, hidden)
+    ids, vals = synth.moe_routing(g, rows, experts, top_k)
+    wts = np.stack([oracle.moe_gate(v) for v in vals])
+    ref = oracle.moe_batch_forward_q4k(x, ids, wts, gate, up, down, hidden, inter)
+    got = forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
+def test_config4_shapes(backend):
+    """BASELINE configs[4]: 256 experts, hidden 2048, expert FFN 512, softmax top-8; M = 1
+    (decode) and M = 512 (prefill chunk) in one launch each.  The M = 512 result is checked on
+    sampled rows against the oracle, and every row must equal the same token run alone (the
+    kernels treat rows independently)."""
+    g = synth.rng(4)
+    experts, hidden, inter, top_k = 256, 2048, 512, 8
+    one = synth.q4k_weights(g, inter, hidden)          # distinct bytes per expert, cheaply
+    gate = np.concatenate([np.roll(one, 977 * e) for e in range(experts)])
+    up = np.concatenate([np.roll(one, 1931 * e + 5) for e in range(experts)])
+    dn = synth.q4k_weights(g, hidden, inter)
+    down = np.concatenate([np.roll(dn, 1409 * e + 3) for e in range(experts)])
+    # rolled bytes are still valid Q4_K only in the quant area; regenerate headers per expert
+    nb = gate.size // 144
+    for t in (gate, up, down):
+        blocks = t.reshape(-1, 144)
+        hdr = synth.q4k_weights(g, 1, 256 * 64).reshape(-1, 144)[:, :16]
+        blocks[:, :16] = np.tile(hdr, (blocks.shape[0] // hdr.shape[0] + 1, 1))[: blocks.shape[0]]
+    assert nb == experts * inter * (hidden // 256)
+    rows = 512
+    x = synth.activations_bf16(g, rows, hidden)
+    ids, vals = synth.moe_routing(g, rows, experts, top_k)
+    wts = np.stack([oracle.moe_gate(v) for v in vals])
+    got = forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
+    sample = [0, 1, 100, 255, 256, 511]
+    ref = oracle.moe_batch_forward_q4k(x[sample], ids[sample], wts[sample], gate, up, down, hidden, inter)
+    assert rel_err(got[sample], ref) <= TOL, rel_err(got[sample], ref)
+    alone = forward_rows(backend, x[:1], ids[:1], wts[:1], gate, up, down, hidden, inter, experts)
+    assert np.array_equal(alone[0], got[0])
+    assert np.all(np.isfinite(got))

@@ -67,6 +67,129 @@ def cpu_baseline(seconds_budget=12.0):
     }
 
 
+def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
+    """The metric's other parts, each timed with HIP events on the launch stream after warm-up:
+    configs[2] (MXFP4 weights, per-token E4M3 activations, M in {1, 4, 16}), configs[3] (prefill
+    GEMM M=2048 with Q4_K and with MXFP4 weights, plus one rank's N=8704 column shard) and
+    configs[4] (routed Q4_K experts, M=1 and M=512).  Weights rotate over distinct copies so
+    that bandwidth-bound cases stream from HBM."""
+    g = synth.rng(2)
+    stream = torch.cuda.current_stream().cuda_stream
+    backend.SetStream(stream)
+
+    def to_dev(arr):
+        return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+
+    def wrap(t):
+        return backend.WrapBuffer(t.data_ptr(), t.numel() * t.element_size())
+
+    def timed_us(launches, reps, graph=True):
+        """Mean microseconds per pass over `launches` (a list of (kernel, KernelLaunch))."""
+        def once():
+            for kern, l in launches:
+                backend.LaunchKernel(kern, l)
+        for _ in range(3):
+            once()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if graph:
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                backend.SetStream(torch.cuda.current_stream().cuda_stream)
+                for _ in range(reps):
+                    once()
+            backend.SetStream(stream)
+            torch.cuda.synchronize()
+            e0.record()
+            gr.replay()
+            e1.record()
+        else:
+            e0.record()
+            for _ in range(reps):
+                once()
+            e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    out = {}
+    # ---- configs[2]: W4A8 decode / speculative verify -------------------------------------
+    n, k = N_FF, K_HID
+    copies = 8
+    w_mx = to_dev(synth.mxfp4_weights(g, n, k))
+    w_list = [w_mx] + [w_mx.clone() for _ in range(copies - 1)]
+    wref = torch.zeros(n, dtype=torch.uint8, device=dev)
+    kq = backend.LoadKernel("quantize_fp8_pack_rows")
+    kg = backend.LoadKernel("gemm_mxfp4_wmma")
+    w4a8 = {}
+    for m in (1, 4, 16):
+        x = to_dev(synth.activations_bf16_outliers(g, m, k))
+        a8 = torch.empty(m * k, dtype=torch.uint8, device=dev)
+        asc = torch.empty(m, dtype=torch.float32, device=dev)
+        y = torch.empty(m * n, dtype=torch.float32, device=dev)
+        launches = [(kg, KernelLaunch(grid_x=n // 64, buffers=[wrap(a8), wrap(w), wrap(asc), wrap(wref), wrap(y)],
+                                      scalars=[m, n, k, 1, 0])) for w in w_list]
+        backend.LaunchKernel(kq, KernelLaunch(grid_x=m, buffers=[wrap(x), wrap(a8), wrap(asc)], scalars=[m, k]))
+        us = timed_us(launches, 10) / copies
+        nbytes = n * k // 2 + n * k // 32 + m * k + 4 * m + 4 * m * n
+        uq = timed_us([(kq, KernelLaunch(grid_x=m, buffers=[wrap(x), wrap(a8), wrap(asc)], scalars=[m, k]))], 50)
+        w4a8[f"m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                         "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "quantize_us": round(uq, 2)}
+    out["mxfp4_w4a8_gemv_17408x5120"] = w4a8
+    del w_list
+
+    # ---- configs[3]: prefill GEMM M=2048 ---------------------------------------------------
+    m = 2048
+    prefill = {}
+    a = to_dev(synth.activations_bf16(g, m, k))
+    w_q = to_dev(synth.q4k_weights(g, n, k))
+    kw = backend.LoadKernel("gemm_q4k_wmma")
+    a8 = torch.empty(m * k, dtype=torch.uint8, device=dev)
+    asc = torch.empty(m, dtype=torch.float32, device=dev)
+    backend.LaunchKernel(kq, KernelLaunch(grid_x=m, buffers=[wrap(a), wrap(a8), wrap(asc)], scalars=[m, k]))
+    for label, nn in (("n17408", n), ("n8704_shard", n // 2)):
+        y = torch.empty(m * nn, dtype=torch.float32, device=dev)
+        wq = w_q[: nn * (k // 256) * 144]
+        us = timed_us([(kw, KernelLaunch(grid_x=nn // 64, grid_y=m // 128, buffers=[wrap(a), wrap(wq), wrap(y)],
+                                         scalars=[m, nn, k]))], 10, graph=False)
+        prefill[f"q4k_{label}"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * nn * k / us / 1e6, 1),
+                                   "frac_fp16_peak": round(2 * m * nn * k / us / 1e6 / 2500.0, 4)}
+        wm = to_dev(synth.mxfp4_column_shard(w_mx.cpu().numpy(), n, k, 0, nn)) if nn != n else w_mx
+        us = timed_us([(kg, KernelLaunch(grid_x=nn // 64, buffers=[wrap(a8), wrap(wm), wrap(asc), wrap(wref), wrap(y)],
+                                         scalars=[m, nn, k, 1, 0]))], 10, graph=False)
+        prefill[f"mxfp4_{label}"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * nn * k / us / 1e6, 1),
+                                     "frac_fp8_peak": round(2 * m * nn * k / us / 1e6 / 5000.0, 4)}
+    out["prefill_gemm_m2048_k5120"] = prefill
+    del a, w_q, w_mx, a8, y
+
+    # ---- configs[4]: routed Q4_K experts ---------------------------------------------------
+    experts, hidden, inter, top_k = 256, 2048, 512, 8
+    gate = to_dev(synth.q4k_weights(g, experts * inter, hidden))
+    up = to_dev(synth.q4k_weights(g, experts * inter, hidden))
+    down = to_dev(synth.q4k_weights(g, experts * hidden, inter))
+    gs, ds = inter * (hidden // 256) * 144, hidden * (inter // 256) * 144
+    kgu, kdn = backend.LoadKernel("moe_experts_gate_up_q4k_rows"), backend.LoadKernel("moe_experts_down_q4k_rows")
+    moe = {}
+    for rows in (1, 512):
+        x = to_dev(synth.activations_bf16(g, rows, hidden))
+        ids, vals = synth.moe_routing(g, rows, experts, top_k)
+        e = np.exp(vals - vals.max(axis=1, keepdims=True))
+        wts = to_dev((e / e.sum(axis=1, keepdims=True)).astype(np.float32))
+        ids = to_dev(ids)
+        phi = torch.empty(rows * top_k * inter, dtype=torch.float32, device=dev)
+        y = torch.empty(rows * hidden, dtype=torch.float32, device=dev)
+        launches = [(kgu, KernelLaunch(grid_x=inter * top_k // 8, grid_y=rows,
+                                       buffers=[wrap(x), wrap(gate), wrap(up), wrap(ids), wrap(phi)],
+                                       scalars=[hidden, inter, top_k, gs, gs, rows])),
+                    (kdn, KernelLaunch(grid_x=hidden // 8, grid_y=rows,
+                                       buffers=[wrap(phi), wrap(down), wrap(ids), wrap(wts), wrap(y)],
+                                       scalars=[hidden, inter, top_k, ds, 0, rows]))]
+        us = timed_us(launches, 20 if rows == 1 else 5, graph=rows == 1)
+        touched = (min(rows * top_k, experts) if rows > 1 else top_k) * 3 * gs
+        moe[f"m{rows}"] = {"us": round(us, 2), "weight_GBps": round(touched / us / 1e3, 1)}
+    out["moe_q4k_256x2048x512_top8"] = moe
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,6 +197,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=8)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary cases (W4A8 GEMV, prefill GEMMs, MoE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); "
@@ -167,6 +291,8 @@ def main():
                      "down_us_per_launch": round(us_down, 3),
                      "down_GBps": round(gemv_algorithmic_bytes(K_HID, N_FF) / (us_down * 1e-6) / 1e9, 1)},
     }
+    if not args.no_also:
+        result["also"] = other_cases(backend, torch, np, synth, KernelLaunch, dev, args)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

@@ -268,9 +268,152 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// ---- a few activation rows (speculative verify, m <= 32) ----------------------------------
+// Bandwidth-bound: every weight byte is needed once and there is almost no reuse to stage
+// for, so nothing goes through LDS on the way in.  v_mfma_scale_f32_16x16x128_f8f6f4 has the
+// operand shape for that: a lane supplies 16 bytes of one weight row (32 E2M1 values = one
+// MX block, K quarter lane/16), so one load instruction of a wavefront reads 64 contiguous
+// bytes of each of 16 rows, and the E4M3 activation fragment is two such loads
+// (k = 16q + [0,16) and 64 + 16q + [0,16) for K quarter q; layouts probed on hardware).
+// A workgroup of eight wavefronts owns 64 weight rows (four 16-column tiles); the wavefronts
+// split K among themselves and stream their share with a register prefetch; the eight partial
+// tiles are summed in LDS in wavefront order (deterministic) and scaled by the row scale.  Two
+// workgroups share a CU, so the 272 workgroups of N = 17408 are resident at once.
+constexpr int kSkinnyWaves = 8;
+
+template <int MT>   // 16-row activation tiles: 1 (m <= 16) or 2 (m <= 32)
+__global__ __launch_bounds__(64 * kSkinnyWaves, 4) void mxfp4_a8_skinny_kernel(
+    const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k) {
+  constexpr int kDepth = 2;
+  typedef float float4v __attribute__((ext_vector_type(4)));
+  __shared__ float red[kSkinnyWaves][MT][4][4][64];
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t l16 = lane & 15u, kq = lane >> 4;
+  const uint32_t n0 = blockIdx.x * 64u;
+  const uint32_t row_bytes = k / 2, row_blocks = k / 32;
+  const uint8_t* scales = w + static_cast<size_t>(n) * row_bytes;
+
+  // K steps (128 wide) of this wavefront: step index i stands for K step wave + 8 i, so that
+  // at any moment the eight wavefronts read eight neighbouring 64-byte pieces of each row.
+  const uint32_t total = k / 128u;
+  const uint32_t s0 = 0, s1 = total > wave ? (total - wave + kSkinnyWaves - 1) / kSkinnyWaves : 0;
+
+  // Loads use the lane order that coalesces: lane p fetches 16-byte chunk p%4 of row p/4, so
+  // four neighbouring lanes cover 64 contiguous bytes.  The MFMA wants lane q*16 + r to hold
+  // chunk q of row r; ds_bpermute moves the registers into that order (through the LDS
+  // crossbar, no LDS memory), which is far cheaper than letting every lane of a quad address
+  // a different row.
+  const uint32_t ld_row = lane >> 2, ld_chunk = lane & 3u;
+  const int take = static_cast<int>(((lane & 15u) * 4u + (lane >> 4)) * 4u);   // source lane * 4
+  const uint8_t* wq[4];
+  const uint8_t* ws[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint32_t row = n0 + j * 16u + ld_row;
+    row = row < n ? row : n - 1u;
+    wq[j] = w + static_cast<size_t>(row) * row_bytes + ld_chunk * 16u;
+    ws[j] = scales + static_cast<size_t>(row) * row_blocks;
+  }
+  const uint8_t* ap[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const uint32_t row = i * 16u + ld_row;
+    ap[i] = a8 + static_cast<size_t>(row < m ? row : m - 1u) * k + ld_chunk * 16u;
+  }
+
+  struct Stage {
+    uint4 q[4], lo[MT], hi[MT];
+    uint32_t s[4];
+  };
+  auto fetch = [&](uint32_t index, Stage& st) {
+    const uint32_t step = wave + kSkinnyWaves * index;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      st.q[j] = load_u4(wq[j] + step * 64u);
+      st.s[j] = *reinterpret_cast<const uint32_t*>(ws[j] + 4u * step);   // blocks 4 step + 0..3
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      st.lo[i] = load_u4(ap[i] + step * 128u);
+      st.hi[i] = load_u4(ap[i] + step * 128u + 64u);
+    }
+  };
+
+  float4v acc[MT][4];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+  auto to_mfma_order = [&](const uint4& v) {
+    return int4v_t{__builtin_amdgcn_ds_bpermute(take, static_cast<int>(v.x)),
+                   __builtin_amdgcn_ds_bpermute(take, static_cast<int>(v.y)),
+                   __builtin_amdgcn_ds_bpermute(take, static_cast<int>(v.z)),
+                   __builtin_amdgcn_ds_bpermute(take, static_cast<int>(v.w))};
+  };
+  auto consume = [&](const Stage& cur) {
+    int8v_t af[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int4v_t lo = to_mfma_order(cur.lo[i]), hi = to_mfma_order(cur.hi[i]);
+      af[i] = int8v_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int4v_t q = to_mfma_order(cur.q[j]);
+      const int8v_t bf = int8v_t{q[0], q[1], q[2], q[3], 0, 0, 0, 0};
+      // this lane's MX block is byte kq of its row's scale word
+      const int sv = static_cast<int>(static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(take, static_cast<int>(cur.s[j]))) >> (kq * 8u));
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 0, sv);
+      }
+    }
+  };
+
+  // Register pipeline of kDepth steps.  Full groups consume and refill unconditionally (a
+  // refill past this wavefront's range re-reads its last step, a cache hit), so the compiler
+  // counts outstanding loads exactly; the last partial group consumes without refilling.
+  Stage st[kDepth];
+  const uint32_t last = s1 > s0 ? s1 - 1u : s0;   // (a wavefront without steps reloads step `wave`: k >= 1024 keeps that in range)
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) fetch(s0 + d < s1 ? s0 + d : last, st[d]);
+  uint32_t step = s0;
+  for (; step + kDepth <= s1; step += kDepth) {
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      consume(st[d]);
+      fetch(step + d + kDepth < s1 ? step + d + kDepth : last, st[d]);
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < kDepth - 1; ++d) {
+    if (step + d < s1) consume(st[d]);     // uniform
+  }
+
+  // Sum the wavefronts' partial tiles: lane holds column l16 and rows (lane/16)*4 + e.
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave][i][j][e][lane] = acc[i][j][e];
+  __syncthreads();
+  for (uint32_t o = t; o < m * 64u; o += 64u * kSkinnyWaves) {
+    const uint32_t row = o / 64u, col = o % 64u;
+    const uint32_t i = row / 16u, r = row % 16u, ln = (r / 4u) * 16u + col % 16u;
+    float sum = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < kSkinnyWaves; ++wv) sum += red[wv][i][col / 16u][r % 4u][ln];
+    if (n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row];
+  }
+}
+
 }  // namespace
 
-bool gemm_mxfp4_a8_supported(uint64_t k) { return k % 128 == 0; }
+bool gemm_mxfp4_a8_supported(uint64_t k) { return k % 128 == 0 && k <= (1u << 24); }
 
 namespace {
 
@@ -291,6 +434,15 @@ void launch_range(const uint8_t* a8, const float* as, const uint8_t* w, float* c
 // over every CU instead (two such workgroups share a CU).
 hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
+  if (m <= 32 && k >= 128u * kSkinnyWaves) {   // every wavefront of the K split has a step
+    const dim3 grid((n + 63u) / 64u), block(64 * kSkinnyWaves);
+    if (m <= 16) {
+      hipLaunchKernelGGL(mxfp4_a8_skinny_kernel<1>, grid, block, 0, stream, a8, as, w, c, m, n, k);
+    } else {
+      hipLaunchKernelGGL(mxfp4_a8_skinny_kernel<2>, grid, block, 0, stream, a8, as, w, c, m, n, k);
+    }
+    return hipGetLastError();
+  }
   const uint32_t cus = static_cast<uint32_t>(num_cus());
   const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u;
   const uint32_t tiles = tiles_m * tiles_n;

@@ -242,9 +242,9 @@ qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
     return QMM_UNSUPPORTED_FEATURE;
   }
   float* out = c.ptr<float>(4);
-  // Regime: up to four rows stay on the bandwidth-bound VALU GEMV (each weight byte is
-  // read once); from five rows on the scaled MFMA takes over.
-  if (m > 4 && qmm::gemm_mxfp4_a8_supported(k)) {
+  // Regime: a single row stays on the VALU GEMV; from two rows on the scaled MFMA takes over
+  // (a streaming kernel up to 32 rows, the tiled GEMM above that).
+  if (m > 1 && k >= 1024 && qmm::gemm_mxfp4_a8_supported(k)) {
     qmm_status st = map_hip(qmm::launch_mxfp4_a8_gemm(
         c.ptr<const uint8_t>(0), c.ptr<const float>(2), c.ptr<const uint8_t>(1), out,
         static_cast<uint32_t>(m), static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));

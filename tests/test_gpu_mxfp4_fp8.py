@@ -162,9 +162,9 @@ def test_w4a8_wmma_contract(backend, n, k, m, split):
     run(backend, "gemm_mxfp4_wmma_reduce", [part, out], [m * n, split], grid=((m * n + 255) // 256, 1, 1))
     backend.Synchronize()
     got = backend.CopyD2H(out, dtype=np.float32).reshape(m, n)
-    # up to four rows run on the fp32 VALU GEMV (1e-3); from five rows on the scaled MFMA
-    # takes over, whose documented bound is 5e-4 of the rms output (test_gpu_gemm_mxfp4.py)
-    tol = TOL if m <= 4 else 1e-2
+    # a single row runs on the fp32 VALU GEMV (1e-3); from two rows on the scaled MFMA takes
+    # over, whose documented bound is 5e-4 of the rms output (test_gpu_gemm_mxfp4.py)
+    tol = TOL if m <= 1 else 1e-2
     assert rel_err(got, ref) <= tol, rel_err(got, ref)
     assert rms_err(got, ref) <= 5e-4
     want_ref = w[n * k // 2:].reshape(n, -1).max(axis=1)
@@ -226,5 +226,5 @@ def test_full_size_config2(backend):
         got = backend.CopyD2H(out, dtype=np.float32).reshape(m, n)
         rows = [0, m - 1] if m > 1 else [0]
         ref = oracle.gemm_mxfp4_w4a8(codes[rows], scale[rows], w, len(rows), n, k)
-        assert rel_err(got[rows], ref) <= (TOL if m <= 4 else 1e-2), (m, rel_err(got[rows], ref))
+        assert rel_err(got[rows], ref) <= (TOL if m <= 1 else 1e-2), (m, rel_err(got[rows], ref))
         assert rms_err(got[rows], ref) <= 5e-4

@@ -21,6 +21,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per gate/up launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# same counter reads for a device copy of known size (profiles/q4k_gemv_m1_ffn27b_hbm_traffic.md);
+# a counter figure, not measured by this script.
+GATE_UP_HBM_TRAFFIC_BYTES = 50_550_000
 N_FF, K_HID = 17408, 5120
 
 
@@ -284,7 +288,8 @@ def main():
                                "(5120x17408) per step, fp32 activations, fp32 accumulate",
                    "layers_rotated": args.layers, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
                      "kernel": "gemv_kernel<Q4KPairCodec> N=17408 K=5120",
                      "us_per_launch": round(us_per_launch, 3),
                      "algorithmic_bytes_per_launch": gemv_algorithmic_bytes(N_FF, K_HID),

@@ -1,0 +1,189 @@
+// Host-side projection helpers over the Backend: the reference's regime table
+// (src/models/qwen3_5/project.cpp:233-366, thresholds src/core/decode_internal.hpp:1349-1441)
+// and split-K rule (src/core/decode_internal.hpp:840-885), with the same function names.
+// ProjectBatch computes C (m x n fp32) = A (m x k fp32) . deq(W)^T for a quantized weight.
+#pragma once
+
+#include <map>
+#include <string>
+
+#include "backend.hpp"
+
+namespace tessera_amd {
+
+// src/core/decode_internal.hpp:840-885.
+constexpr std::size_t kGemmVecOutputsPerBlock = 8;
+constexpr std::size_t kGemmVecSplitTargetBlocks = 2048;
+constexpr std::size_t kGemmVecMaxSplit = 8;
+// src/core/decode_internal.hpp:1349-1361,1425-1441.
+constexpr std::size_t kGemmWmmaMinRows = 64;
+constexpr std::size_t kGemmWmmaMinCols = 32;
+constexpr std::size_t kTiledMinRows = 16;
+
+// Largest divisor of k/256 that brings the workgroup count of a "_vec"/"_rows" launch up to
+// `target`, capped at kGemmVecMaxSplit; 1 keeps the plain grid.
+inline std::size_t GemmVecSplit(std::size_t outputs, std::size_t k, std::size_t target = kGemmVecSplitTargetBlocks) {
+  const std::size_t blocks_x = (outputs + kGemmVecOutputsPerBlock - 1) / kGemmVecOutputsPerBlock;
+  if (blocks_x == 0 || blocks_x >= target) return 1;
+  const std::size_t superblocks = k / 256;
+  std::size_t split = (target + blocks_x - 1) / blocks_x;
+  if (split > kGemmVecMaxSplit) split = kGemmVecMaxSplit;
+  for (; split > 1; --split) {
+    if (superblocks % split == 0) return split;
+  }
+  return 1;
+}
+
+// Kernels and scratch a sequence of projections shares (the part of Qwen35State that
+// ProjectBatch and ProjectWmma touch: src/models/qwen3_5/internal.hpp:104-199).
+struct ProjectState {
+  std::map<std::string, std::unique_ptr<Kernel>> kernels;
+  std::unique_ptr<Buffer> gemv_part;                     // split-K partials
+  std::unique_ptr<Buffer> wmma_a, wmma_as;               // E4M3 codes and row scales of A
+  std::map<const Buffer*, std::unique_ptr<Buffer>> mxfp4_wref;
+  // The reference splits K to fill a 96-CU card; this backend takes any split (it writes the
+  // whole result to region 0) but gains nothing from it, so the default passes split = 1.
+  bool honour_reference_split = false;
+};
+
+inline Expected<const Kernel*> CachedKernel(Backend& backend, ProjectState& h, const std::string& id) {
+  auto it = h.kernels.find(id);
+  if (it == h.kernels.end()) {
+    auto loaded = backend.LoadKernel(id);
+    if (!loaded) return unexpected(loaded.error());
+    it = h.kernels.emplace(id, std::move(*loaded)).first;
+  }
+  return it->second.get();
+}
+
+inline Expected<void> Grow(Backend& backend, std::unique_ptr<Buffer>& slot, std::size_t bytes) {
+  if (slot != nullptr && slot->Size() >= bytes) return {};
+  auto buf = backend.AllocateBuffer(bytes);
+  if (!buf) return unexpected(buf.error());
+  slot = std::move(*buf);
+  return {};
+}
+
+// "_vec" / "_rows{R}" launch with the split-K partials and the reduce pass
+// (ProjectGemvDevice / ProjectGemvRowsDevice, src/models/qwen3_5/internal.hpp:104-199).
+inline Expected<void> ProjectGemvDevice(Backend& backend, ProjectState& h, const Kernel& gemm, const Buffer& a,
+                                        const Buffer& w, Buffer& out, std::size_t m, std::size_t n, std::size_t k) {
+  const std::size_t split = h.honour_reference_split ? GemmVecSplit(m * n, k) : 1;
+  const Buffer* dst = &out;
+  if (split > 1) {
+    if (auto ok = Grow(backend, h.gemv_part, split * m * n * 4); !ok) return ok;
+    dst = h.gemv_part.get();
+  }
+  KernelLaunch l;
+  l.grid_x = static_cast<std::uint32_t>((m * n + kGemmVecOutputsPerBlock - 1) / kGemmVecOutputsPerBlock);
+  l.grid_y = static_cast<std::uint32_t>(split);
+  l.buffers = {&a, &w, dst};
+  l.scalars = {m, n, k, split};
+  if (auto ok = backend.LaunchKernel(gemm, l); !ok) return ok;
+  if (split > 1) {
+    auto reduce = CachedKernel(backend, h, "gemm_vec_reduce");
+    if (!reduce) return unexpected(reduce.error());
+    KernelLaunch r;
+    r.grid_x = static_cast<std::uint32_t>((m * n + 255) / 256);
+    r.buffers = {h.gemv_part.get(), &out};
+    r.scalars = {m * n, split};
+    return backend.LaunchKernel(**reduce, r);
+  }
+  return {};
+}
+
+// MXFP4 weights with per-token E4M3 activations (ProjectWmma,
+// src/models/qwen3_5/project.cpp:100-232): quantize_fp8_pack_rows, mxfp4_row_ref once per
+// weight, gemm_mxfp4_wmma.  Returns false when the backend lacks the kernel.
+inline Expected<bool> ProjectWmma(Backend& backend, ProjectState& h, const Buffer& a, const Buffer& w, Buffer& out,
+                                  std::size_t m, std::size_t n, std::size_t k) {
+  auto wmma = CachedKernel(backend, h, "gemm_mxfp4_wmma");
+  if (!wmma) {
+    if (wmma.error() == StatusCode::UnsupportedFeature) return false;
+    return unexpected(wmma.error());
+  }
+  auto pack = CachedKernel(backend, h, "quantize_fp8_pack_rows");
+  auto rowref = CachedKernel(backend, h, "mxfp4_row_ref");
+  if (!pack) return unexpected(pack.error());
+  if (!rowref) return unexpected(rowref.error());
+  if (auto ok = Grow(backend, h.wmma_a, m * k); !ok) return unexpected(ok.error());
+  if (auto ok = Grow(backend, h.wmma_as, m * 4); !ok) return unexpected(ok.error());
+  auto it = h.mxfp4_wref.find(&w);
+  if (it == h.mxfp4_wref.end()) {
+    auto buf = backend.AllocateBuffer(n);
+    if (!buf) return unexpected(buf.error());
+    KernelLaunch rl;
+    rl.grid_x = static_cast<std::uint32_t>((n + 255) / 256);
+    rl.buffers = {&w, buf->get()};
+    rl.scalars = {n, k};
+    if (auto ok = backend.LaunchKernel(**rowref, rl); !ok) return unexpected(ok.error());
+    it = h.mxfp4_wref.emplace(&w, std::move(*buf)).first;
+  }
+  KernelLaunch ql;
+  ql.grid_x = static_cast<std::uint32_t>(m);
+  ql.block_x = 1024;
+  ql.buffers = {&a, h.wmma_a.get(), h.wmma_as.get()};
+  ql.scalars = {m, k};
+  if (auto ok = backend.LaunchKernel(**pack, ql); !ok) return unexpected(ok.error());
+  KernelLaunch wl;
+  wl.grid_x = static_cast<std::uint32_t>((n + 63) / 64);
+  wl.block_x = 128;
+  wl.buffers = {h.wmma_a.get(), &w, h.wmma_as.get(), it->second.get(), &out};
+  wl.scalars = {m, n, k, 1, 0};
+  if (auto ok = backend.LaunchKernel(**wmma, wl); !ok) return unexpected(ok.error());
+  return true;
+}
+
+// The regime table.  On this backend every id of a format accepts every m and picks its own
+// gfx950 kernel, so the table only has to name an id the caller's contract allows.
+inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtype, const Buffer& a, const Buffer& w,
+                                   Buffer& out, std::size_t m, std::size_t n, std::size_t k) {
+  if (m == 0 || n == 0 || k == 0) return unexpected(StatusCode::InvalidArgument);
+  if (dtype == DType::F4E2M1) {
+    if (m <= 16 || k % 128 == 0) {             // the reference caps the fp8 path at m = 16; here it scales on
+      auto done = ProjectWmma(backend, h, a, w, out, m, n, k);
+      if (!done) return unexpected(done.error());
+      if (*done) return {};
+    }
+    auto gemm = CachedKernel(backend, h, m == 1 ? "gemm_mxfp4" : (m <= 16 ? "gemm_mxfp4_rows" : "gemm_mxfp4_batched"));
+    if (!gemm) return unexpected(gemm.error());
+    KernelLaunch l;
+    l.grid_x = static_cast<std::uint32_t>(m == 1 ? (n + 7) / 8 : (n + 7) / 8);
+    l.buffers = {&a, &w, &out};
+    l.scalars = {m, n, k};
+    return backend.LaunchKernel(**gemm, l);
+  }
+  if (dtype == DType::Q4K) {
+    if (k % 256 != 0) return unexpected(StatusCode::InvalidArgument);
+    if (m >= 2 && m <= 4) {
+      auto rows = CachedKernel(backend, h, "gemm_q4k_rows" + std::to_string(m));
+      if (!rows) return unexpected(rows.error());
+      return ProjectGemvDevice(backend, h, **rows, a, w, out, m, n, k);
+    }
+    if (m >= kGemmWmmaMinRows && n >= kGemmWmmaMinCols) {
+      auto wmma = CachedKernel(backend, h, "gemm_q4k_wmma");
+      if (!wmma) return unexpected(wmma.error());
+      KernelLaunch l;
+      l.grid_x = static_cast<std::uint32_t>((n + 63) / 64);
+      l.grid_y = static_cast<std::uint32_t>((m + 127) / 128);
+      l.buffers = {&a, &w, &out};
+      l.scalars = {m, n, k};
+      return backend.LaunchKernel(**wmma, l);
+    }
+    if (m >= kTiledMinRows) {
+      auto tiled = CachedKernel(backend, h, "gemm_q4k_batched");
+      if (!tiled) return unexpected(tiled.error());
+      KernelLaunch l;
+      l.grid_x = static_cast<std::uint32_t>(((m + 31) / 32) * ((n + 31) / 32));
+      l.buffers = {&a, &w, &out};
+      l.scalars = {m, n, k};
+      return backend.LaunchKernel(**tiled, l);
+    }
+    auto vec = CachedKernel(backend, h, "gemm_q4k_vec");
+    if (!vec) return unexpected(vec.error());
+    return ProjectGemvDevice(backend, h, **vec, a, w, out, m, n, k);
+  }
+  return unexpected(StatusCode::UnsupportedFeature);
+}
+
+}  // namespace tessera_amd

@@ -1,0 +1,150 @@
+// Parity of the C++ host side (tessera_amd/host) against the CPU oracle, through the C ABI.
+// Test infrastructure: links oracle/liboracle.so as the checker.  Prints one line per case and
+// exits non-zero on the first failure.  `--list` prints the cases without touching a GPU.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../../tessera_amd/host/project.hpp"
+
+extern "C" {
+int orc_gemm_q4k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k);
+int orc_gemm_mxfp4_ref(const float* a, const uint8_t* w, const uint8_t* s, float* c, size_t m, size_t n, size_t k);
+int orc_quantize_fp8_ref(float* data, float* scale, size_t rows, size_t cols);
+}
+
+using namespace tessera_amd;
+
+namespace {
+
+std::mt19937_64 rng(7);
+
+std::vector<uint8_t> Q4KWeights(size_t n, size_t k) {
+  std::vector<uint8_t> w(n * (k / 256) * 144);
+  for (auto& b : w) b = static_cast<uint8_t>(rng());
+  for (size_t blk = 0; blk < w.size() / 144; ++blk) {   // fp16 d, dmin around 1e-2
+    w[blk * 144 + 0] = static_cast<uint8_t>(rng()); w[blk * 144 + 1] = 0x20 + (rng() & 3);
+    w[blk * 144 + 2] = static_cast<uint8_t>(rng()); w[blk * 144 + 3] = 0x20 + (rng() & 3);
+  }
+  return w;
+}
+std::vector<uint8_t> MxFp4Weights(size_t n, size_t k) {
+  std::vector<uint8_t> w(n * k / 2 + n * k / 32);
+  for (size_t i = 0; i < n * k / 2; ++i) w[i] = static_cast<uint8_t>(rng());
+  for (size_t i = n * k / 2; i < w.size(); ++i) w[i] = static_cast<uint8_t>(119 + rng() % 5);
+  return w;
+}
+std::vector<float> Activations(size_t m, size_t k) {
+  std::normal_distribution<float> nd(0.0f, 1.0f);
+  std::vector<float> a(m * k);
+  for (auto& v : a) {
+    v = nd(rng);
+    uint32_t bits; std::memcpy(&bits, &v, 4);             // bf16-valued, like the prefill configuration
+    bits = (bits + 0x7FFFu + ((bits >> 16) & 1u)) & 0xFFFF0000u;
+    std::memcpy(&v, &bits, 4);
+  }
+  return a;
+}
+
+template <class T>
+std::unique_ptr<Buffer> Upload(Backend& b, const std::vector<T>& v) {
+  auto buf = b.AllocateBuffer(v.size() * sizeof(T));
+  if (!buf || !b.CopyH2D(**buf, std::as_bytes(std::span<const T>(v)))) std::exit(3);
+  return std::move(*buf);
+}
+
+// largest |got - ref| over max(|ref|, 0.05 rms(ref)), and over rms(ref)
+void Errors(const std::vector<float>& got, const std::vector<float>& ref, double& rel, double& rms_rel) {
+  double ss = 0;
+  for (float v : ref) ss += double(v) * v;
+  const double rms = std::sqrt(ss / ref.size());
+  rel = rms_rel = 0;
+  for (size_t i = 0; i < ref.size(); ++i) {
+    const double d = std::fabs(double(got[i]) - ref[i]);
+    rel = std::max(rel, d / std::max(std::fabs(double(ref[i])), 0.05 * rms));
+    rms_rel = std::max(rms_rel, d / rms);
+  }
+}
+
+struct Case {
+  const char* name;
+  DType dtype;
+  size_t m, n, k;
+  bool reference_split;
+  double rel_tol, rms_tol;     // see tests/test_gpu_q4k.py, test_gpu_gemm_q4k.py, test_gpu_gemm_mxfp4.py
+};
+const Case kCases[] = {
+    {"q4k decode m=1 (gemm_q4k_vec)", DType::Q4K, 1, 640, 5120, false, 1e-3, 1e-3},
+    {"q4k decode m=1, reference split-K + gemm_vec_reduce", DType::Q4K, 1, 640, 5120, true, 1e-3, 1e-3},
+    {"q4k verify m=3 (gemm_q4k_rows3)", DType::Q4K, 3, 333, 2048, true, 1e-3, 1e-3},
+    {"q4k m=7 (gemm_q4k_vec, m rows)", DType::Q4K, 7, 129, 1280, false, 1e-3, 1e-3},
+    {"q4k m=16 (gemm_q4k_batched)", DType::Q4K, 16, 256, 1024, false, 1e-3, 1e-3},
+    {"q4k prefill m=192 (gemm_q4k_wmma, fp16 MFMA)", DType::Q4K, 192, 320, 1024, false, 1.0, 4e-3},
+    {"mxfp4 w4a8 m=1 (quantize_fp8_pack_rows + gemm_mxfp4_wmma)", DType::F4E2M1, 1, 512, 1024, false, 1e-3, 1e-3},
+    {"mxfp4 w4a8 m=16 (streaming scaled MFMA)", DType::F4E2M1, 16, 512, 2048, false, 1e-2, 5e-4},
+    {"mxfp4 w4a8 m=300 (tiled scaled MFMA)", DType::F4E2M1, 300, 384, 1024, false, 1e-2, 5e-4},
+};
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  if (argc > 1 && std::strcmp(argv[1], "--list") == 0) {
+    for (const Case& c : kCases) std::printf("%s\n", c.name);
+    return 0;
+  }
+  auto backend = CreateBackend();
+  if (auto ok = backend->Init(); !ok) {
+    std::printf("Init failed: status %d (%s)\n", static_cast<int>(ok.error()), backend->LastError());
+    return 2;
+  }
+  // Error behaviour of the reference interface.
+  if (auto k = backend->LoadKernel("attention"); k || k.error() != StatusCode::UnsupportedFeature) return 4;
+  const std::byte blob[4] = {};
+  if (auto k = backend->LoadKernel("gemm_q4k", std::span<const std::byte>(blob)); k || k.error() != StatusCode::UnsupportedFeature) return 4;
+  if (auto b = backend->AllocateBuffer(0); b || b.error() != StatusCode::InvalidArgument) return 4;
+  {
+    auto k = backend->LoadKernel("gemm_q4k");
+    auto buf = backend->AllocateBuffer(1024);
+    KernelLaunch l;
+    l.buffers = {buf->get(), buf->get(), buf->get()};
+    l.scalars = {1, 8, 100};                                // k not a multiple of 256
+    if (auto st = backend->LaunchKernel(**k, l); st || st.error() != StatusCode::InvalidArgument) return 4;
+  }
+  std::printf("ok   error behaviour (unknown id, non-empty code, zero-byte buffer, bad k)\n");
+
+  int failed = 0;
+  for (const Case& c : kCases) {
+    ProjectState h;
+    h.honour_reference_split = c.reference_split;
+    const auto a = Activations(c.m, c.k);
+    const auto w = c.dtype == DType::Q4K ? Q4KWeights(c.n, c.k) : MxFp4Weights(c.n, c.k);
+    std::vector<float> ref(c.m * c.n), got(c.m * c.n);
+    if (c.dtype == DType::Q4K) {
+      orc_gemm_q4k_ref(a.data(), w.data(), ref.data(), c.m, c.n, c.k);
+    } else {
+      std::vector<float> qdq = a, scale(c.m);               // QuantizeFp8Ref then GemmMxFp4Ref
+      orc_quantize_fp8_ref(qdq.data(), scale.data(), c.m, c.k);
+      orc_gemm_mxfp4_ref(qdq.data(), w.data(), w.data() + c.n * c.k / 2, ref.data(), c.m, c.n, c.k);
+    }
+    auto da = Upload(*backend, a);
+    auto dw = Upload(*backend, w);
+    auto out = backend->AllocateBuffer(c.m * c.n * 4);
+    auto st = ProjectBatch(*backend, h, c.dtype, *da, *dw, **out, c.m, c.n, c.k);
+    backend->Synchronize();
+    if (!st) {
+      std::printf("FAIL %s: status %d (%s)\n", c.name, static_cast<int>(st.error()), backend->LastError());
+      ++failed;
+      continue;
+    }
+    if (!backend->CopyD2H(**out, std::as_writable_bytes(std::span<float>(got)))) return 3;
+    double rel, rms;
+    Errors(got, ref, rel, rms);
+    const bool ok = rel <= c.rel_tol && rms <= c.rms_tol;
+    std::printf("%s %s: rel %.2e (<= %.0e) rms %.2e (<= %.0e)\n", ok ? "ok  " : "FAIL", c.name, rel, c.rel_tol, rms, c.rms_tol);
+    failed += ok ? 0 : 1;
+  }
+  return failed == 0 ? 0 : 1;
+}

@@ -190,6 +190,15 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
         us = timed_us(launches, 20 if rows == 1 else 5, graph=rows == 1)
         touched = (min(rows * top_k, experts) if rows > 1 else top_k) * 3 * gs
         moe[f"m{rows}"] = {"us": round(us, 2), "weight_GBps": round(touched / us / 1e3, 1)}
+        if rows > 1:
+            # the same chunk with the tokens grouped by expert (one weight pass per expert, MFMA)
+            kff = backend.LoadKernel("moe_experts_ffn_q4k_rows")
+            grouped = [(kff, KernelLaunch(grid_x=1, buffers=[wrap(x), wrap(gate), wrap(up), wrap(down), wrap(ids),
+                                                             wrap(wts), wrap(y)],
+                                          scalars=[hidden, inter, top_k, gs, gs, ds, rows, 0]))]
+            us = timed_us(grouped, 10, graph=False)
+            moe[f"m{rows}_grouped"] = {"us": round(us, 2), "weight_GBps": round(touched / us / 1e3, 1),
+                                       "frac_hbm": round(touched / us / 1e3 / HBM_PEAK_GBS, 4)}
     out["moe_q4k_256x2048x512_top8"] = moe
     return out
 

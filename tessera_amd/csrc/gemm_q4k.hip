@@ -3,7 +3,8 @@
 // src/backends/rocm/rocm_kernels_wmma.cpp:30-80,334-431, which stages A and the decoded
 // weights in LDS as fp16 and accumulates in fp32).
 //
-// Two launches.  (1) The activations are converted once to fp16 in a workspace (the
+// Two launches.  (1) The activations are converted once to fp16 in a workspace, each row divided
+// by a power-of-two scale that the epilogue multiplies back, so the fp16 range is no limit (the
 // reference converts them again in every workgroup; done once, the GEMM reads 2 bytes per
 // activation instead of 4 and the conversion costs one pass over A).  (2) The GEMM proper:
 // v_mfma_f32_32x32x16_f16, fp32 accumulate.
@@ -32,23 +33,55 @@ __device__ __forceinline__ void direct_load16(const void* base, uint32_t voff, u
                :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
-// fp32 -> fp16 (round to nearest even) with the order 0,2,1,3,4,6,5,7 inside each group of 8.
-__global__ __launch_bounds__(256) void a_to_f16_kernel(const float* __restrict__ a, _Float16* __restrict__ out,
-                                                       uint64_t groups) {
-  const uint64_t g = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
-  if (g >= groups) return;
-  const float4 lo = reinterpret_cast<const float4*>(a)[2 * g];
-  const float4 hi = reinterpret_cast<const float4*>(a)[2 * g + 1];
+// Largest |v| over a 256-thread workgroup (every thread returns it).
+__device__ __forceinline__ float block_amax(float v, float* red) {
+  v = wave_max(v);
+  if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float r = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  return r;
+}
+
+// Power-of-two scale that brings a row with largest magnitude `amax` to [1024, 2048): the
+// fp16 copy then neither overflows nor loses small values to subnormals, and the scaling itself
+// is exact.  Zero rows (and non-finite ones) get scale 1.
+__device__ __forceinline__ float row_scale_for(float amax) {
+  const uint32_t e = (bit_cast<uint32_t>(amax) >> 23) & 0xFFu;
+  if (e == 0u || e == 0xFFu) return 1.0f;
+  const int se = static_cast<int>(e) - 10;
+  return bit_cast<float>(static_cast<uint32_t>(se < 1 ? 1 : se) << 23);
+}
+
+__device__ __forceinline__ half8_t to_f16_group(const float4& lo, const float4& hi, float inv) {
+  // the order 0,2,1,3,4,6,5,7 inside each group of 8 (what the in-register weight decode yields)
   half8_t v;
-  v[0] = static_cast<_Float16>(lo.x);
-  v[1] = static_cast<_Float16>(lo.z);
-  v[2] = static_cast<_Float16>(lo.y);
-  v[3] = static_cast<_Float16>(lo.w);
-  v[4] = static_cast<_Float16>(hi.x);
-  v[5] = static_cast<_Float16>(hi.z);
-  v[6] = static_cast<_Float16>(hi.y);
-  v[7] = static_cast<_Float16>(hi.w);
-  reinterpret_cast<half8_t*>(out)[g] = v;
+  v[0] = static_cast<_Float16>(lo.x * inv), v[1] = static_cast<_Float16>(lo.z * inv);
+  v[2] = static_cast<_Float16>(lo.y * inv), v[3] = static_cast<_Float16>(lo.w * inv);
+  v[4] = static_cast<_Float16>(hi.x * inv), v[5] = static_cast<_Float16>(hi.z * inv);
+  v[6] = static_cast<_Float16>(hi.y * inv), v[7] = static_cast<_Float16>(hi.w * inv);
+  return v;
+}
+
+// One workgroup per destination row: fp32 row -> fp16 (round to nearest even) divided by the
+// row's power-of-two scale, which goes to scale[row] and is multiplied back in the GEMM's
+// epilogue.  With `pos` the rows are gathered: destination row pos[p] takes source row p / top_k.
+__global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restrict__ src, _Float16* __restrict__ dst,
+                                                          float* __restrict__ scale, uint32_t cols,
+                                                          const uint32_t* __restrict__ pos, uint32_t top_k) {
+  __shared__ float red[4];
+  const uint32_t p = blockIdx.x;
+  const uint32_t drow = pos != nullptr ? pos[p] : p, srow = pos != nullptr ? p / top_k : p;
+  const float4* in = reinterpret_cast<const float4*>(src + static_cast<size_t>(srow) * cols);
+  float amax = 0.0f;
+  for (uint32_t g = threadIdx.x; g < cols / 4u; g += 256u) {
+    const float4 v = in[g];
+    amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), amax));
+  }
+  const float s = row_scale_for(block_amax(amax, red)), inv = 1.0f / s;
+  half8_t* out = reinterpret_cast<half8_t*>(dst + static_cast<size_t>(drow) * cols);
+  for (uint32_t g = threadIdx.x; g < cols / 8u; g += 256u) out[g] = to_f16_group(in[2 * g], in[2 * g + 1], inv);
+  if (threadIdx.x == 0) scale[drow] = s;
 }
 
 // Two packed fp16 weights from the nibbles at bits [3:0] and [19:16] of `x`.
@@ -57,10 +90,11 @@ __device__ __forceinline__ half2_t decode_pair(uint32_t x, half2_t scale, half2_
   return __builtin_elementwise_fma(q, scale, neg_min);
 }
 
+// One BM x BN tile of C at (m0, n0); columns at and past n_end are not stored.
 template <int BM, int BN>
-__global__ __launch_bounds__(BN * 2) void q4k_gemm_kernel(
-    const _Float16* __restrict__ a16, const uint8_t* __restrict__ w, float* __restrict__ c,
-    uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end) {
+__device__ __forceinline__ void q4k_gemm_tile(
+    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t m0, uint32_t n0, uint32_t n_end) {
   constexpr int kWaves = BN / 32;                  // one wavefront per 32 output columns
   constexpr int kTI = BM / 32;                     // MFMA tiles per wavefront (all rows of the tile)
   constexpr int kABlk = BM / 16 / kWaves;          // 1 KB activation blocks a wavefront loads per step
@@ -72,8 +106,6 @@ __global__ __launch_bounds__(BN * 2) void q4k_gemm_kernel(
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t l32 = lane & 31u, kg = lane >> 5;
-  const uint32_t tiles_n = (n_end - n_begin + BN - 1) / BN;
-  const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = n_begin + (blockIdx.x % tiles_n) * BN;
   const uint32_t row_blocks = k / 256;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (__attribute__((address_space(3))) uint8_t*)lds));
@@ -203,30 +235,68 @@ __global__ __launch_bounds__(BN * 2) void q4k_gemm_kernel(
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the workgroup
 
-  // Epilogue: lane holds column l32 and rows (e/4)*8 + kg*4 + e%4 of each 32 x 32 tile.
+  // Epilogue: lane holds column l32 and rows (e/4)*8 + kg*4 + e%4 of each 32 x 32 tile; the
+  // four row scales of each e/4 group are one 16-byte load (the scale array is padded, so rows
+  // past m read something harmless).
   const uint32_t col = n0 + wave * 32u + l32;
 #pragma unroll
   for (int i = 0; i < kTI; ++i) {
+    float4 sc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      sc[q] = *reinterpret_cast<const float4*>(a_scale + m0 + i * 32u + q * 8u + kg * 4u);
+    }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const uint32_t row = m0 + i * 32u + (e >> 2) * 8u + kg * 4u + (e & 3u);
-      if (row < m && col < n_end) c[static_cast<size_t>(row) * n + col] = acc[i][e];
+      const float4 s4 = sc[e >> 2];
+      const float rs = (e & 3) == 0 ? s4.x : (e & 3) == 1 ? s4.y : (e & 3) == 2 ? s4.z : s4.w;
+      if (row < m && col < n_end) c[static_cast<size_t>(row) * n + col] = acc[i][e] * rs;
     }
   }
 }
 
 template <int BM, int BN>
-void launch_range(const _Float16* a16, const uint8_t* w, float* c, uint32_t m, uint32_t n, uint32_t k,
-                  uint32_t n_begin, uint32_t n_end, hipStream_t stream) {
+__global__ __launch_bounds__(BN * 2) void q4k_gemm_kernel(
+    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end) {
+  const uint32_t tiles_n = (n_end - n_begin + BN - 1) / BN;
+  q4k_gemm_tile<BM, BN>(a16, a_scale, w, c, m, n, k, (blockIdx.x / tiles_n) * BM, n_begin + (blockIdx.x % tiles_n) * BN,
+                        n_end);
+}
+
+// Grouped form for routed experts: segment e (grid.y) multiplies rows seg[e]..seg[e+1] of a16
+// by expert e's weights (w + e * w_stride) into the same rows of c.  Segment bounds live in
+// device memory (the routing is computed on the device); an empty segment leaves at once.
+template <int BM, int BN>
+__global__ __launch_bounds__(BN * 2) void q4k_gemm_grouped_kernel(
+    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
+    float* __restrict__ c, const uint32_t* __restrict__ seg, uint64_t w_stride, uint32_t n, uint32_t k) {
+  const uint32_t e = blockIdx.y;
+  const uint32_t r0 = seg[e], r1 = seg[e + 1];
+  if (r1 <= r0) return;
+  const _Float16* a_e = a16 + static_cast<size_t>(r0) * k;
+  const uint8_t* w_e = w + e * w_stride;
+  float* c_e = c + static_cast<size_t>(r0) * n;
+  for (uint32_t m0 = 0; m0 < r1 - r0; m0 += BM) {
+    q4k_gemm_tile<BM, BN>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, blockIdx.x * BN, n);
+  }
+}
+
+template <int BM, int BN>
+void launch_range(const _Float16* a16, const float* a_scale, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                  uint32_t k, uint32_t n_begin, uint32_t n_end, hipStream_t stream) {
   const uint32_t tiles = ((m + BM - 1) / BM) * ((n_end - n_begin + BN - 1) / BN);
-  hipLaunchKernelGGL((q4k_gemm_kernel<BM, BN>), dim3(tiles), dim3(BN * 2), 0, stream, a16, w, c, m, n, k, n_begin, n_end);
+  hipLaunchKernelGGL((q4k_gemm_kernel<BM, BN>), dim3(tiles), dim3(BN * 2), 0, stream, a16, a_scale, w, c, m, n, k,
+                     n_begin, n_end);
 }
 
 }  // namespace
 
 bool gemm_q4k_supported(uint64_t m, uint64_t k) { return k % 256 == 0 && k <= (1u << 20) && m * k < (1ull << 31); }
 
-size_t gemm_q4k_workspace_bytes(uint64_t m, uint64_t k) { return static_cast<size_t>(m) * k * 2; }
+// fp16 copy of A, then one scale per row padded by a tile of rows (the epilogue reads scales in fours).
+size_t gemm_q4k_workspace_bytes(uint64_t m, uint64_t k) { return static_cast<size_t>(m) * k * 2 + (static_cast<size_t>(m) + 256) * 4; }
 
 // The bulk of C goes to 256 x 256 tiles, whole rounds of one tile per CU; columns left over
 // when the tile count is not a multiple of the CU count are cut into 128 x 64 tiles that
@@ -234,8 +304,8 @@ size_t gemm_q4k_workspace_bytes(uint64_t m, uint64_t k) { return static_cast<siz
 hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream) {
   _Float16* a16 = static_cast<_Float16*>(workspace);
-  const uint64_t groups = static_cast<uint64_t>(m) * k / 8;
-  hipLaunchKernelGGL(a_to_f16_kernel, dim3(static_cast<uint32_t>((groups + 255) / 256)), dim3(256), 0, stream, a, a16, groups);
+  float* a_scale = reinterpret_cast<float*>(a16 + static_cast<size_t>(m) * k);
+  hipLaunchKernelGGL(rows_to_f16_kernel, dim3(m), dim3(256), 0, stream, a, a16, a_scale, k, nullptr, 1u);
   const uint32_t cus = static_cast<uint32_t>(num_cus());
   const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u;
   const uint32_t tiles = tiles_m * tiles_n;
@@ -246,8 +316,141 @@ hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* wor
     main_tn = 0;
   }
   const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
-  if (n_split > 0) launch_range<256, 256>(a16, w, c, m, n, k, 0u, n_split, stream);
-  if (n_split < n) launch_range<128, 64>(a16, w, c, m, n, k, n_split, n, stream);
+  if (n_split > 0) launch_range<256, 256>(a16, a_scale, w, c, m, n, k, 0u, n_split, stream);
+  if (n_split < n) launch_range<128, 64>(a16, a_scale, w, c, m, n, k, n_split, n, stream);
+  return hipGetLastError();
+}
+
+// ---- routed experts, a whole chunk of tokens grouped by expert -----------------------------
+// (token, slot) pairs are sorted by expert so that each expert's weights are streamed once for
+// all the tokens routed to it, and the three projections run as grouped MFMA GEMMs.
+namespace {
+
+// seg[e] = first sorted position of expert e (seg[experts] = pairs); pos[p] = sorted position
+// of pair p.  Counting sort with LDS atomics: which position inside its expert's segment a pair
+// gets depends on the order the atomics land in, but a row's result does not depend on where the
+// row sits, so the outputs are the same on every run.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restrict__ ids, uint32_t pairs,
+                                                        uint32_t experts, uint32_t* __restrict__ seg,
+                                                        uint32_t* __restrict__ pos) {
+  __shared__ uint32_t cursor[1024];
+  const uint32_t t = threadIdx.x;
+  cursor[t] = 0;
+  __syncthreads();
+  for (uint32_t p = t; p < pairs; p += 1024u) {
+    const uint32_t id = ids[p] < experts ? ids[p] : experts - 1u;   // a bad id cannot leave the tensor
+    atomicAdd(&cursor[id], 1u);
+  }
+  __syncthreads();
+  if (t == 0) {
+    uint32_t run = 0;
+    for (uint32_t i = 0; i < experts; ++i) {
+      const uint32_t c = cursor[i];
+      cursor[i] = run;
+      seg[i] = run;
+      run += c;
+    }
+    seg[experts] = run;
+  }
+  __syncthreads();
+  for (uint32_t p = t; p < pairs; p += 1024u) {
+    const uint32_t id = ids[p] < experts ? ids[p] : experts - 1u;
+    pos[p] = atomicAdd(&cursor[id], 1u);
+  }
+}
+
+// phi = silu(g) * u for one sorted row, written as the fp16 operand of the down GEMM with its
+// own power-of-two row scale (phi can exceed the fp16 range).
+__global__ __launch_bounds__(256) void moe_silu_mul_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                           _Float16* __restrict__ phi16, float* __restrict__ scale,
+                                                           uint32_t inter) {
+  __shared__ float red[4];
+  const size_t base = static_cast<size_t>(blockIdx.x) * inter;
+  const float4* gp = reinterpret_cast<const float4*>(g + base);
+  const float4* up = reinterpret_cast<const float4*>(u + base);
+  auto f = [](float gv, float uv) { return (gv / (1.0f + expf(-gv))) * uv; };
+  auto phi4 = [&](uint32_t q) {
+    const float4 a = gp[q], b = up[q];
+    return make_float4(f(a.x, b.x), f(a.y, b.y), f(a.z, b.z), f(a.w, b.w));
+  };
+  float amax = 0.0f;
+  for (uint32_t q = threadIdx.x; q < inter / 4u; q += 256u) {
+    const float4 v = phi4(q);
+    amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), amax));
+  }
+  const float s = row_scale_for(block_amax(amax, red)), inv = 1.0f / s;
+  half8_t* out = reinterpret_cast<half8_t*>(phi16 + base);
+  for (uint32_t q = threadIdx.x; q < inter / 8u; q += 256u) out[q] = to_f16_group(phi4(2 * q), phi4(2 * q + 1), inv);
+  if (threadIdx.x == 0) scale[blockIdx.x] = s;
+}
+
+// out[t][j] (+)= sum_slot wts[t][slot] * rows[pos[t*top_k + slot]][j], slots in order.
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, const uint32_t* __restrict__ pos,
+                                                          const float* __restrict__ wts, float* __restrict__ out,
+                                                          uint32_t tokens, uint32_t top_k, uint32_t hidden,
+                                                          bool accumulate) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (i >= static_cast<uint64_t>(tokens) * hidden) return;
+  const uint32_t t = static_cast<uint32_t>(i / hidden), j = static_cast<uint32_t>(i % hidden);
+  float acc = 0.0f;
+  for (uint32_t s = 0; s < top_k; ++s) {
+    acc += wts[t * top_k + s] * rows[static_cast<size_t>(pos[t * top_k + s]) * hidden + j];
+  }
+  out[i] = accumulate ? out[i] + acc : acc;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~size_t{255}; }
+
+}  // namespace
+
+bool moe_ffn_q4k_supported(uint64_t hidden, uint64_t inter, uint64_t experts) {
+  return hidden % 256 == 0 && inter % 256 == 0 && hidden <= (1u << 16) && inter <= (1u << 16) && experts >= 1 &&
+         experts <= 1024;
+}
+
+size_t moe_ffn_q4k_workspace_bytes(uint64_t pairs, uint64_t hidden, uint64_t inter, uint64_t experts) {
+  return align256((experts + 1) * 4) + align256(pairs * 4) + 2 * align256((pairs + 256) * 4) + align256(pairs * hidden * 2) +
+         2 * align256(pairs * inter * 4) + align256(pairs * inter * 2) + align256(pairs * hidden * 4);
+}
+
+hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                              const uint32_t* ids, const float* wts, float* out, void* workspace,
+                              uint32_t hidden, uint32_t inter, uint32_t top_k, uint64_t gate_stride,
+                              uint64_t up_stride, uint64_t down_stride, uint32_t experts, uint32_t tokens,
+                              bool accumulate, hipStream_t stream) {
+  const uint32_t pairs = tokens * top_k;
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  uint32_t* seg = reinterpret_cast<uint32_t*>(ws);
+  ws += align256((static_cast<size_t>(experts) + 1) * 4);
+  uint32_t* pos = reinterpret_cast<uint32_t*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * 4);
+  float* x_scale = reinterpret_cast<float*>(ws);
+  ws += align256((static_cast<size_t>(pairs) + 256) * 4);
+  float* phi_scale = reinterpret_cast<float*>(ws);
+  ws += align256((static_cast<size_t>(pairs) + 256) * 4);
+  _Float16* a16 = reinterpret_cast<_Float16*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * hidden * 2);
+  float* g = reinterpret_cast<float*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * inter * 4);
+  float* u = reinterpret_cast<float*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * inter * 4);
+  _Float16* phi16 = reinterpret_cast<_Float16*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * inter * 2);
+  float* rows = reinterpret_cast<float*>(ws);
+
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, seg, pos);
+  hipLaunchKernelGGL(rows_to_f16_kernel, dim3(pairs), dim3(256), 0, stream, x, a16, x_scale, hidden, pos, top_k);
+  constexpr int BM = 32, BN = 64;
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3((inter + BN - 1) / BN, experts), dim3(BN * 2), 0, stream,
+                     a16, x_scale, gate, g, seg, gate_stride, inter, hidden);
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3((inter + BN - 1) / BN, experts), dim3(BN * 2), 0, stream,
+                     a16, x_scale, up, u, seg, up_stride, inter, hidden);
+  hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(pairs), dim3(256), 0, stream, g, u, phi16, phi_scale, inter);
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3((hidden + BN - 1) / BN, experts), dim3(BN * 2), 0, stream,
+                     phi16, phi_scale, down, rows, seg, down_stride, hidden, inter);
+  const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, rows, pos,
+                     wts, out, tokens, top_k, hidden, accumulate);
   return hipGetLastError();
 }
 

@@ -438,6 +438,46 @@ qmm_status run_top_k_rows(const LaunchCtx& c) {
                                         c.stream));
 }
 
+// "moe_experts_ffn_q4k_rows" (not a reference id): the routed-expert feed-forward of a chunk
+// of tokens in one call, tokens grouped by expert.  Buffers x (rows x hidden), gate, up, down
+// (expert tensors), ids, wts (rows x top_k), out (rows x hidden); scalars hidden, inter, top_k,
+// gate_stride, up_stride, down_stride, rows, accumulate.  Same result as gate_up_rows followed
+// by down_rows, on the fp16 MFMA path (bound as for the Q4_K prefill GEMM).
+qmm_status run_moe_ffn_rows(const LaunchCtx& c) {
+  if (!counts(c, 7, 8)) return bad("moe_experts_ffn_q4k_rows: expects 7 buffers and 8 scalars");
+  const uint64_t hidden = c.sc[0], inter = c.sc[1], top_k = c.sc[2], gs = c.sc[3], us = c.sc[4], ds = c.sc[5];
+  const uint64_t rows = c.sc[6], acc = c.sc[7];
+  if (c.bytes == nullptr) return bad("moe_experts_ffn_q4k_rows: buffer sizes are required (they bound the expert ids)");
+  if (hidden == 0 || inter == 0 || top_k == 0 || top_k > 64 || rows == 0 || rows * top_k > (1u << 20)) {
+    return bad("moe_experts_ffn_q4k_rows: bad hidden, inter, top_k or rows");
+  }
+  const u128 eg = q4k_bytes(inter, hidden), ed = q4k_bytes(hidden, inter);
+  if (hidden % 256 != 0 || inter % 256 != 0 || gs < eg || us < eg || ds < ed) {
+    return bad("moe_experts_ffn_q4k_rows: shapes must be multiples of 256 and strides hold one expert");
+  }
+  if (!c.fits(0, static_cast<u128>(rows) * hidden * 4) || !c.fits(1, eg) || !c.fits(2, eg) || !c.fits(3, ed) ||
+      !c.fits(4, static_cast<u128>(rows) * top_k * 4) || !c.fits(5, static_cast<u128>(rows) * top_k * 4) ||
+      !c.fits(6, static_cast<u128>(rows) * hidden * 4)) {
+    return bad("moe_experts_ffn_q4k_rows: a buffer is smaller than the shape requires");
+  }
+  uint64_t experts = (c.bytes[1] - static_cast<uint64_t>(eg)) / gs + 1;
+  const uint64_t eu = (c.bytes[2] - static_cast<uint64_t>(eg)) / us + 1, edn = (c.bytes[3] - static_cast<uint64_t>(ed)) / ds + 1;
+  experts = experts < eu ? experts : eu;
+  experts = experts < edn ? experts : edn;
+  if (!qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
+    g_last_error = "moe_experts_ffn_q4k_rows: more than 1024 experts or a dimension above 65536 is not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  void* ws = nullptr;
+  const qmm_status st = workspace(qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
+  if (st != QMM_OK) return st;
+  return map_hip(qmm::launch_moe_ffn_q4k(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint8_t>(2),
+                                         c.ptr<const uint8_t>(3), c.ptr<const uint32_t>(4), c.ptr<const float>(5),
+                                         c.ptr<float>(6), ws, static_cast<uint32_t>(hidden), static_cast<uint32_t>(inter),
+                                         static_cast<uint32_t>(top_k), gs, us, ds, static_cast<uint32_t>(experts),
+                                         static_cast<uint32_t>(rows), acc != 0, c.stream));
+}
+
 struct Entry {
   const char* id;
   qmm_fn fn;
@@ -469,6 +509,7 @@ const Entry kTable[] = {
     {"moe_experts_down_q4k", run_moe_down},
     {"moe_experts_gate_up_q4k_rows", run_moe_gate_up_rows},
     {"moe_experts_down_q4k_rows", run_moe_down_rows},
+    {"moe_experts_ffn_q4k_rows", run_moe_ffn_rows},
     {"moe_gate", run_moe_gate},
     {"top_k_rows", run_top_k_rows},
     {"dequant_q4k", run_dequant_q4k},

@@ -55,6 +55,16 @@ size_t gemm_q4k_workspace_bytes(uint64_t m, uint64_t k);
 hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream);
 
+// Routed experts for a chunk of tokens, grouped by expert (gemm_q4k.hip): out[t] (+)= sum over
+// the token's top_k experts of wts * down_e(silu(gate_e x) * up_e x), as grouped MFMA GEMMs.
+bool moe_ffn_q4k_supported(uint64_t hidden, uint64_t inter, uint64_t experts);
+size_t moe_ffn_q4k_workspace_bytes(uint64_t pairs, uint64_t hidden, uint64_t inter, uint64_t experts);
+hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                              const uint32_t* ids, const float* wts, float* out, void* workspace,
+                              uint32_t hidden, uint32_t inter, uint32_t top_k, uint64_t gate_stride,
+                              uint64_t up_stride, uint64_t down_stride, uint32_t experts, uint32_t tokens,
+                              bool accumulate, hipStream_t stream);
+
 // ---- element-wise helpers (elementwise.hip) ---------------------------------
 hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64_t split,
                              hipStream_t stream);

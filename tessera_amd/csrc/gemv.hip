@@ -723,35 +723,58 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
     Codec::load(args, tail ? ln_tail : ln, grp * P, cpr, f);
   };
 
-  // Weight loads first, activations second: both are in flight before anything waits.
   typename Codec::Frag frag[D];
-#pragma unroll
-  for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
-
   // Invalid lanes (past the last chunk) carry zero activations, so they add nothing.
   typename Codec::template X<R> x;
   if constexpr (Codec::kStageX) {
     constexpr uint32_t kPiece = R == 1 ? 8192u : (R == 2 ? 4096u : 2048u);  // floats per row
     constexpr uint32_t kStride = kPiece + kPiece / 16u;
+    constexpr int kXPer = 4;                  // float4 a thread may carry of a short activation row
     __shared__ __attribute__((aligned(16))) float xs[R * kStride];
     const uint32_t k = args.k;
     const uint32_t mine = Codec::x_elem0(chunk);
-    for (uint32_t base = 0; base < k; base += kPiece) {
-      const uint32_t len = k - base < kPiece ? k - base : kPiece;
-      if (base != 0) lds_barrier();  // the previous piece has been read
+    if (R == 1 && k <= kPiece && k <= kXPer * 4u * blockDim.x) {   // uniform
+      // Short single row: its loads are requested BEFORE the weight prefetch.  Loads return in
+      // order, so requested after it they would sit behind D fragments per lane (over 100 KB
+      // per workgroup) and the first dot product would start microseconds later.
+      float4 xr[kXPer];
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        for (uint32_t e = t * 4u; e < len; e += blockDim.x * 4u) {
-          *reinterpret_cast<float4*>(&xs[r * kStride + StagedX::pad(e)]) =
-              *reinterpret_cast<const float4*>(args.a + static_cast<size_t>(r) * k + base + e);
-        }
+      for (int i = 0; i < kXPer; ++i) {
+        const uint32_t e = (t + i * blockDim.x) * 4u;
+        xr[i] = *reinterpret_cast<const float4*>(args.a + (e < k ? e : k - 4u));
+      }
+#pragma unroll
+      for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
+#pragma unroll
+      for (int i = 0; i < kXPer; ++i) {
+        const uint32_t e = (t + i * blockDim.x) * 4u;
+        if (e < k) *reinterpret_cast<float4*>(&xs[StagedX::pad(e)]) = xr[i];
       }
       lds_barrier();
-      if (mine >= base && mine < base + len) {
-        Codec::template load_x<R>(args, chunk, valid, x, StagedX{xs, base, kStride});
+      Codec::template load_x<R>(args, chunk, valid, x, StagedX{xs, 0u, kStride});
+    } else {
+      // Weight loads first, activations second: both are in flight before anything waits.
+#pragma unroll
+      for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
+      for (uint32_t base = 0; base < k; base += kPiece) {
+        const uint32_t len = k - base < kPiece ? k - base : kPiece;
+        if (base != 0) lds_barrier();  // the previous piece has been read
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          for (uint32_t e = t * 4u; e < len; e += blockDim.x * 4u) {
+            *reinterpret_cast<float4*>(&xs[r * kStride + StagedX::pad(e)]) =
+                *reinterpret_cast<const float4*>(args.a + static_cast<size_t>(r) * k + base + e);
+          }
+        }
+        lds_barrier();
+        if (mine >= base && mine < base + len) {
+          Codec::template load_x<R>(args, chunk, valid, x, StagedX{xs, base, kStride});
+        }
       }
     }
   } else {
+#pragma unroll
+    for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
     Codec::template load_x<R>(args, chunk, valid, x, 0);
   }
 
@@ -999,21 +1022,23 @@ bool gemv_fp8_supported(uint64_t k) { return k % 16 == 0 && k / 16 <= 1024; }
 
 hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                            uint32_t k, hipStream_t stream) {
-  // Three or four activation rows per pass need 96-128 registers for the activations
-  // alone, which only fits workgroups of up to 576 threads (k <= 18432).
-  const bool wide = (k / 32u + 63u) / 64u * 64u <= 576u;
+  // A lane keeps the 32 activations of its chunk for every row of the pass in registers: 128
+  // registers at four rows, which fits only with two wavefronts per SIMD (workgroups of up to
+  // 512 threads, k <= 16384); two rows fit 768-thread workgroups (k <= 24576); beyond that the
+  // rows run one at a time.
+  const uint32_t row_threads = (k / 32u + 63u) / 64u * 64u;
   for (uint32_t r0 = 0; r0 < m;) {
     const uint32_t left = m - r0;
     Q4KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
     float* out = c + static_cast<size_t>(r0) * n;
     hipError_t e;
     uint32_t took;
-    if (left >= 4 && wide) {
-      e = launch_gemv_r<Q4KCodec, 4, 576, 2>(args, out, n, k, n, stream), took = 4;
-    } else if (left == 3 && wide) {
-      e = launch_gemv_r<Q4KCodec, 3, 576, 2>(args, out, n, k, n, stream), took = 3;
-    } else if (left >= 2) {
-      e = launch_gemv_r<Q4KCodec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
+    if (left >= 4 && row_threads <= 512u) {
+      e = launch_gemv_r<Q4KCodec, 4, 512, 2>(args, out, n, k, n, stream), took = 4;
+    } else if (left == 3 && row_threads <= 512u) {
+      e = launch_gemv_r<Q4KCodec, 3, 512, 2>(args, out, n, k, n, stream), took = 3;
+    } else if (left >= 2 && row_threads <= 768u) {
+      e = launch_gemv_r<Q4KCodec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
     } else {
       e = launch_gemv_r<Q4KPairCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
     }
@@ -1026,19 +1051,20 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
 hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                              uint32_t k, hipStream_t stream) {
   const uint8_t* s = w + static_cast<size_t>(n) * k / 2;
-  const bool wide = (k / 32u + 63u) / 64u * 64u <= 576u;
+  // Register budgets as for Q4_K: four or three rows need two wavefronts per SIMD, two rows three.
+  const uint32_t row_threads = (k / 32u + 63u) / 64u * 64u;
   for (uint32_t r0 = 0; r0 < m;) {
     const uint32_t left = m - r0;
     MxFp4Codec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
     float* out = c + static_cast<size_t>(r0) * n;
     hipError_t e;
     uint32_t took;
-    if (left >= 4 && wide) {
-      e = launch_gemv_r<MxFp4Codec, 4, 576, 2>(args, out, n, k, n, stream), took = 4;
-    } else if (left == 3 && wide) {
-      e = launch_gemv_r<MxFp4Codec, 3, 576, 2>(args, out, n, k, n, stream), took = 3;
-    } else if (left >= 2) {
-      e = launch_gemv_r<MxFp4Codec, 2, 1024, 2>(args, out, n, k, n, stream), took = 2;
+    if (left >= 4 && row_threads <= 512u) {
+      e = launch_gemv_r<MxFp4Codec, 4, 512, 2>(args, out, n, k, n, stream), took = 4;
+    } else if (left == 3 && row_threads <= 512u) {
+      e = launch_gemv_r<MxFp4Codec, 3, 512, 2>(args, out, n, k, n, stream), took = 3;
+    } else if (left >= 2 && row_threads <= 768u) {
+      e = launch_gemv_r<MxFp4Codec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
     } else {
       e = launch_gemv_r<MxFp4Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
     }

@@ -411,6 +411,127 @@ __global__ __launch_bounds__(64 * kSkinnyWaves, 4) void mxfp4_a8_skinny_kernel(
   }
 }
 
+// ---- a few activation rows, streamed through LDS (k a multiple of 512) ----------------------
+// Same arithmetic as the kernel above, fed differently: each direct load moves 256 contiguous
+// bytes of a weight row (four rows per instruction) into a three-stage swizzled LDS ring, so
+// HBM sees long row-contiguous runs instead of 64-byte pieces of sixteen rows, and the
+// fragment reads do the row/K transposition for free.  A workgroup of eight wavefronts owns 64
+// weight rows; per stage (512 of K) the 4 K-steps x 4 column tiles are split two to a wavefront
+// and the two wavefronts of a tile are summed through LDS at the end.
+template <int MT>
+__global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void mxfp4_a8_stream_kernel(
+    const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k) {
+  typedef float float4v __attribute__((ext_vector_type(4)));
+  constexpr uint32_t kBBytes = 64 * 256, kABytes = MT * 16 * 512, kSBytes = 64 * 16;
+  constexpr uint32_t kABase = kBBytes, kSBase = kABase + kABytes, kStage = kSBase + kSBytes;
+  constexpr int kDma = 2 + MT + 1;                      // direct loads a wavefront issues per stage
+  __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kStage];
+
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t l16 = lane & 15u, kq = lane >> 4;
+  const uint32_t n0 = blockIdx.x * 64u;
+  const uint32_t row_bytes = k / 2, row_blocks = k / 32;
+  const uint8_t* w_tile = w + static_cast<size_t>(n0) * row_bytes;
+  const uint8_t* s_tile = w + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(n0) * row_blocks;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) uint8_t*)lds));
+
+  // Direct loads of one stage.  Weight block L (1 KB) = rows 4L..4L+3, sixteen 16-byte chunks
+  // each: lane p fetches row 4L + p/16, chunk (p%16) ^ (row%16).  Activation block L = rows
+  // 2L, 2L+1, thirty-two chunks each: row 2L + p/32, chunk (p%32) ^ (row%16).  Scale words: lane
+  // p < 8 of wavefront v fetches the sixteen E8M0 bytes of row 8v + p.  Rows past the matrix
+  // edge are clamped (never stored).
+  uint32_t b_src[2], a_src[MT], s_src;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t row = 4u * (wave * 2u + i) + lane / 16u;
+    const uint32_t chunk = (lane % 16u) ^ (row % 16u);
+    b_src[i] = (n0 + row < n ? row : n - 1u - n0) * row_bytes + chunk * 16u;
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const uint32_t row = 2u * (wave * MT + i) + lane / 32u;
+    const uint32_t chunk = (lane % 32u) ^ (row % 16u);
+    a_src[i] = (row < m ? row : m - 1u) * k + chunk * 16u;
+  }
+  {
+    const uint32_t row = 8u * wave + (lane & 7u);
+    s_src = (n0 + row < n ? row : n - 1u - n0) * row_blocks;
+  }
+  auto issue_stage = [&](uint32_t stage_off, uint32_t st) {
+    const uint32_t stage = lds_base + stage_off;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) direct_load16(w_tile + st * 256u, b_src[i], stage + (wave * 2u + i) * 1024u);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) direct_load16(a8 + st * 512u, a_src[i], stage + kABase + (wave * MT + i) * 1024u);
+    if (lane < 8u) direct_load16(s_tile + st * 16u, s_src, stage + kSBase + wave * 128u);
+  };
+  auto publish = [&]() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kDma) : "memory");
+  };
+
+  // This wavefront's share of a stage: column tile `tile`, K-steps 2*half and 2*half + 1.
+  const uint32_t tile = wave & 3u, half = wave >> 2;
+  const uint32_t b_row = tile * 16u + l16;
+  float4v acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const uint32_t stages = k / 512u;
+  issue_stage(0, 0);
+  issue_stage(kStage, stages > 1 ? 1 : 0);
+  publish();
+  uint32_t rd = 0, nx = kStage, fill = 2 * kStage;
+  for (uint32_t st = 0; st < stages; ++st) {
+    issue_stage(fill, st + 2 < stages ? st + 2 : stages - 1u);
+    const uint8_t* stage = lds + rd;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t step = half * 2u + u;
+      const uint4 q = *reinterpret_cast<const uint4*>(stage + b_row * 256u + (((step * 4u + kq) ^ l16) * 16u));
+      const int8v_t bf = int8v_t{static_cast<int>(q.x), static_cast<int>(q.y), static_cast<int>(q.z),
+                                 static_cast<int>(q.w), 0, 0, 0, 0};
+      const uint32_t sw = *reinterpret_cast<const uint32_t*>(stage + kSBase + b_row * 16u + step * 4u);
+      const int sv = static_cast<int>(sw >> (kq * 8u));       // this lane's block is byte kq of the step's word
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const uint8_t* arow = stage + kABase + (i * 16u + l16) * 512u;
+        const uint4 lo = *reinterpret_cast<const uint4*>(arow + (((step * 8u + kq) ^ l16) * 16u));
+        const uint4 hi = *reinterpret_cast<const uint4*>(arow + (((step * 8u + 4u + kq) ^ l16) * 16u));
+        const int8v_t af = int8v_t{static_cast<int>(lo.x), static_cast<int>(lo.y), static_cast<int>(lo.z),
+                                   static_cast<int>(lo.w), static_cast<int>(hi.x), static_cast<int>(hi.y),
+                                   static_cast<int>(hi.z), static_cast<int>(hi.w)};
+        acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf, acc[i], 0, 4, 0, 0x7F7F7F7F, 0, sv);
+      }
+    }
+    publish();
+    const uint32_t done = rd;
+    rd = nx;
+    nx = fill;
+    fill = done;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive its workgroup
+  __syncthreads();
+
+  // Sum the two wavefronts of each tile (stage memory is free now): lane holds column l16 and
+  // rows (lane/16)*4 + e of its 16 x 16 tile.
+  float* red = reinterpret_cast<float*>(lds);          // [half][tile][MT][4][64]
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[(((half * 4u + tile) * MT + i) * 4u + e) * 64u + lane] = acc[i][e];
+  __syncthreads();
+  for (uint32_t o = t; o < m * 64u; o += 512u) {
+    const uint32_t row = o / 64u, col = o % 64u;
+    const uint32_t i = row / 16u, r = row % 16u, ln = (r / 4u) * 16u + col % 16u, tl = col / 16u;
+    const float sum = red[(((0u * 4u + tl) * MT + i) * 4u + r % 4u) * 64u + ln] +
+                      red[(((1u * 4u + tl) * MT + i) * 4u + r % 4u) * 64u + ln];
+    if (n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row];
+  }
+}
+
 }  // namespace
 
 bool gemm_mxfp4_a8_supported(uint64_t k) { return k % 128 == 0 && k <= (1u << 24); }
@@ -434,6 +555,15 @@ void launch_range(const uint8_t* a8, const float* as, const uint8_t* w, float* c
 // over every CU instead (two such workgroups share a CU).
 hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
+  if (m <= 32 && k % 512 == 0) {
+    const dim3 grid((n + 63u) / 64u), block(512);
+    if (m <= 16) {
+      hipLaunchKernelGGL(mxfp4_a8_stream_kernel<1>, grid, block, 0, stream, a8, as, w, c, m, n, k);
+    } else {
+      hipLaunchKernelGGL(mxfp4_a8_stream_kernel<2>, grid, block, 0, stream, a8, as, w, c, m, n, k);
+    }
+    return hipGetLastError();
+  }
   if (m <= 32 && k >= 128u * kSkinnyWaves) {   // every wavefront of the K split has a step
     const dim3 grid((n + 63u) / 64u), block(64 * kSkinnyWaves);
     if (m <= 16) {

@@ -686,7 +686,7 @@ struct Fp8Codec {
 // per-wavefront partial sums; a few threads then add them in wavefront order and
 // store (deterministic, no atomics).
 // ----------------------------------------------------------------------------
-template <class Codec, int R, int P, int D, int MAXT>
+template <class Codec, int R, int P, int D, int MAXT, uint32_t XP>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, float* __restrict__ c,
                                                     uint32_t n, uint32_t cpr, uint32_t ldc,
                                                     uint32_t groups_per_wg) {
@@ -727,9 +727,9 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // Invalid lanes (past the last chunk) carry zero activations, so they add nothing.
   typename Codec::template X<R> x;
   if constexpr (Codec::kStageX) {
-    constexpr uint32_t kPiece = R == 1 ? 8192u : (R == 2 ? 4096u : 2048u);  // floats per row
+    constexpr uint32_t kPiece = XP;           // floats of one activation row resident in LDS
     constexpr uint32_t kStride = kPiece + kPiece / 16u;
-    constexpr int kXPer = 4;                  // float4 a thread may carry of a short activation row
+    constexpr int kXPer = XP > 8192u ? 8 : 4; // float4 a thread may carry of a short activation row
     __shared__ __attribute__((aligned(16))) float xs[R * kStride];
     const uint32_t k = args.k;
     const uint32_t mine = Codec::x_elem0(chunk);
@@ -926,8 +926,19 @@ hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n,
   if (grid > groups) grid = groups;
   uint32_t per_wg = (groups + grid - 1) / grid;
   grid = (groups + per_wg - 1) / per_wg;
-  hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT>), dim3(grid), dim3(threads), 0, stream, args,
-                     c, n, cpr, ldc, per_wg);
+  // Activation floats per row kept in LDS at a time.  A single long row (the down
+  // projection) gets the 136 KB variant so that the whole row is staged by one round of
+  // loads instead of three rounds in sequence; those workgroups are alone on their CU anyway.
+  constexpr uint32_t kSmall = R == 1 ? 8192u : (R == 2 ? 4096u : 2048u);
+  if constexpr (R == 1 && Codec::kStageX) {
+    if (args.k > kSmall && args.k <= 32768u && per_cu == 1) {
+      hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, 32768u>), dim3(grid), dim3(threads), 0,
+                         stream, args, c, n, cpr, ldc, per_wg);
+      return hipGetLastError();
+    }
+  }
+  hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall>), dim3(grid), dim3(threads), 0, stream,
+                     args, c, n, cpr, ldc, per_wg);
   return hipGetLastError();
 }
 

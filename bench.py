@@ -141,6 +141,23 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     out["mxfp4_w4a8_gemv_17408x5120"] = w4a8
     del w_list
 
+    # ---- configs[1] weights with 2..16 rows (speculative verify), Q4_K -----------------------
+    w_q1 = to_dev(synth.q4k_weights(g, n, k))
+    wq_list = [w_q1] + [w_q1.clone() for _ in range(copies - 1)]
+    kb = backend.LoadKernel("gemm_q4k_batched")
+    few = {}
+    for m in (2, 4, 8, 16):
+        x = to_dev(synth.activations_f32(g, m, k))
+        y = torch.empty(m * n, dtype=torch.float32, device=dev)
+        launches = [(kb, KernelLaunch(grid_x=(m * n + 7) // 8, buffers=[wrap(x), wrap(w), wrap(y)], scalars=[m, n, k]))
+                    for w in wq_list]
+        us = timed_us(launches, 10) / copies
+        nbytes = n * (k // 256) * 144 + 4 * m * k + 4 * m * n
+        few[f"m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                        "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    out["q4k_few_rows_17408x5120"] = few
+    del wq_list, w_q1
+
     # ---- configs[3]: prefill GEMM M=2048 ---------------------------------------------------
     m = 2048
     prefill = {}

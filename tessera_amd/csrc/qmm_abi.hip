@@ -76,6 +76,11 @@ u128 mxfp4_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * k / 2 +
 // Launches that use it are ordered by the caller's stream, as everything else here.
 void* g_workspace = nullptr;
 size_t g_workspace_bytes = 0;
+// Scratch of the decode-sized kernels (the few-row Q4_K path's activation operand): allocated
+// once by qmm_init and never moved or freed, so a decode step recorded into a HIP graph keeps
+// pointing at live memory whatever the prefill-sized workspace above does later.
+constexpr size_t kDecodeScratchBytes = size_t{16} << 20;
+void* g_decode_scratch = nullptr;
 std::mutex g_workspace_mutex;
 
 qmm_status workspace(size_t bytes, void** out) {
@@ -96,12 +101,31 @@ qmm_status workspace(size_t bytes, void** out) {
   return QMM_OK;
 }
 
-// From this many rows on, Q4_K goes to the fp16 MFMA GEMM; below, the bandwidth-bound GEMV
-// reads each weight once per group of up to four rows.
+// From this many rows on, Q4_K goes to the tiled fp16 MFMA GEMM.  Below it, 2 and more rows of
+// a matrix with at least kQ4KFewRowsMinWeights weights go, eight at a time, to the exact
+// few-row MFMA kernel (weights read once per eight rows); one row and small matrices stay on
+// the VALU GEMV, which needs no activation pre-pass.
 constexpr uint64_t kQ4KGemmMinRows = 24;
+constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{8} << 20;
+constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 
 qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
                       uint64_t k, hipStream_t s) {
+  if (m >= 2 && m < kQ4KGemmMinRows && n * k >= kQ4KFewRowsMinWeights && k <= kQ4KFewRowsMaxK &&
+      qmm::gemv_q4k_mfma_supported(1, n, k)) {
+    void* ws = g_decode_scratch;   // fixed address: a recorded decode step stays valid
+    if (ws == nullptr || qmm::gemv_q4k_mfma_workspace_bytes(8, k) > kDecodeScratchBytes) {
+      g_last_error = "Q4_K: decode scratch missing or too small for this k";
+      return QMM_DEVICE_ERROR;
+    }
+    for (uint64_t r = 0; r < m; r += 8) {
+      const uint64_t rows = m - r < 8 ? m - r : 8;
+      const hipError_t e = qmm::launch_q4k_gemv_mfma(a + r * k, w, c + r * n, ws, static_cast<uint32_t>(rows),
+                                                     static_cast<uint32_t>(n), static_cast<uint32_t>(k), s);
+      if (e != hipSuccess) return map_hip(e);
+    }
+    return QMM_OK;
+  }
   if (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) {
     void* ws = nullptr;
     const qmm_status st = workspace(qmm::gemm_q4k_workspace_bytes(m, k), &ws);
@@ -539,6 +563,13 @@ qmm_status qmm_init(int device) {
   g_device_name = prop.name;
   qmm::set_num_cus(prop.multiProcessorCount);
   g_device = device;
+  if (g_decode_scratch == nullptr) {
+    if ((e = hipMalloc(&g_decode_scratch, kDecodeScratchBytes)) != hipSuccess) {
+      g_decode_scratch = nullptr;
+      g_device = -1;
+      return map_hip(e);
+    }
+  }
   return QMM_OK;
 }
 

@@ -31,6 +31,13 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream);
 
+// Q4_K times 1..4 activation rows on the 4x4x4 fp16 MFMA (gemv_q4k_mfma.hip).  `workspace`
+// holds the fp16 hi/lo activation operand (gemv_q4k_mfma_workspace_bytes).
+bool gemv_q4k_mfma_supported(uint64_t m, uint64_t n, uint64_t k);
+size_t gemv_q4k_mfma_workspace_bytes(uint64_t m, uint64_t k);
+hipError_t launch_q4k_gemv_mfma(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
+                                uint32_t n, uint32_t k, hipStream_t stream);
+
 // ---- routed experts, Q4_K (gemv.hip) ----------------------------------------------
 // phi[t][slot*inter + j] = silu(G_e x_t)[j] * (U_e x_t)[j], e = ids[t][slot]; `rows` tokens.
 hipError_t launch_moe_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up,

@@ -9,7 +9,7 @@ import pytest
 
 import oracle
 from tessera_amd import StatusCode, StatusError, synth
-from util import ref_grid_vec, rel_err, run, same_bits, same_bits_zero_sign_free
+from util import ref_grid_vec, rel_err, rms_err, run, same_bits, same_bits_zero_sign_free
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -112,6 +112,69 @@ def test_rows_kernels(backend, rows):
     with pytest.raises(StatusError) as e:          # the id fixes the row count
         gemm(backend, f"gemm_q4k_rows{rows}", a[:1], w, 1, n, k, extra=(1,))
     assert e.value.code == StatusCode.InvalidArgument
+
+
+# Matrices of 8M weights and more take 2..23 rows through the few-row MFMA kernel (eight rows a
+# pass, activations as fp16 hi/lo pairs with a per-row power-of-two scale); the shapes cover
+# k/256 divisible by 4, by 2 only and odd (its three tilings), ragged n, and every pass count.
+FEW_ROW_SHAPES = [(2048, 4096), (1030, 8192), (515, 17408), (4100, 2048), (3700, 2304), (5500, 1536)]
+
+
+@pytest.mark.parametrize("n,k", FEW_ROW_SHAPES)
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 9, 16, 23])
+def test_few_rows_match_oracle(backend, n, k, m):
+    if m > 9 and (n, k) != FEW_ROW_SHAPES[0]:
+        pytest.skip("several passes are covered on the first shape")
+    g = synth.rng(77 * m + n + k)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
+    got = gemm(backend, "gemm_q4k_batched", a, w, m, n, k)[0]
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    assert rms_err(got, ref) <= 1e-4, rms_err(got, ref)     # the split activations keep 22 bits
+
+
+def test_few_rows_scaling_and_exactness(backend):
+    n, k = 2048, 4096
+    g = synth.rng(31337)
+    w = synth.q4k_weights(g, n, k)
+    deq = oracle.dequantize_q4k(w).reshape(n, k)
+    # one-hot rows reproduce the fp32 block decode bit for bit, whatever the magnitude
+    a = np.zeros((3, k), np.float32)
+    a[0, 5], a[1, 4095], a[2, 1234] = 1.0, 2.0 ** -100, -(2.0 ** 90)
+    got = gemm(backend, "gemm_q4k_batched", a, w, 3, n, k)[0]
+    assert same_bits_zero_sign_free(got[0], deq[:, 5])
+    assert same_bits_zero_sign_free(got[1], deq[:, 4095] * np.float32(2.0 ** -100))
+    assert same_bits_zero_sign_free(got[2], deq[:, 1234] * np.float32(-(2.0 ** 90)))
+    # rows of very different magnitude, a zero row, and a row with a 1000x outlier
+    a = synth.activations_f32(g, 5, k)
+    a[0] *= np.float32(1e-30)
+    a[1] *= np.float32(1e25)
+    a[2] = 0.0
+    a[3, 77] = 1000.0 * np.abs(a[3]).max()
+    ref = oracle.gemm_q4k(a, w, 5, n, k, threads=True)
+    got = gemm(backend, "gemm_q4k_batched", a, w, 5, n, k)[0]
+    assert np.all(got[2] == 0.0)
+    for r in (0, 1, 3, 4):
+        assert rel_err(got[r], ref[r]) <= TOL, (r, rel_err(got[r], ref[r]))
+    # a power-of-two multiple of the input gives exactly that multiple of the output
+    got4 = gemm(backend, "gemm_q4k_batched", 4 * a, w, 5, n, k)[0]
+    assert np.array_equal(got4[3:], 4 * got[3:])
+
+
+def test_few_rows_full_size(backend):
+    """configs[1] shapes with 4 and 8 rows (speculative verify), against the oracle."""
+    for seed, (n, k, m) in enumerate([(17408, 5120, 4), (5120, 17408, 8)]):
+        g = synth.rng(909 + seed)
+        w = synth.q4k_weights(g, n, k)
+        a = synth.activations_f32(g, m, k)
+        ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
+        got = gemm(backend, f"gemm_q4k_rows{m}" if m <= 5 else "gemm_q4k_batched", a, w, m, n, k,
+                   extra=(1,) if m <= 5 else ())[0]
+        assert rel_err(got, ref) <= TOL, (n, k, m, rel_err(got, ref))
+        # each row equals the single-row kernel's answer to fp32 summation-order noise
+        one = gemm(backend, "gemm_q4k_vec", a[:1], w, 1, n, k, extra=(1,))[0]
+        assert rms_err(got[:1], one) <= 2e-5
 
 
 def test_special_inputs(backend):

@@ -103,10 +103,10 @@ qmm_status workspace(size_t bytes, void** out) {
 
 // From this many rows on, Q4_K goes to the tiled fp16 MFMA GEMM.  Below it, 2 and more rows of
 // a matrix with at least kQ4KFewRowsMinWeights weights go, eight at a time, to the exact
-// few-row MFMA kernel (weights read once per eight rows); one row and small matrices stay on
+// few-row MFMA kernels (weights read once per eight rows); one row and small matrices stay on
 // the VALU GEMV, which needs no activation pre-pass.
 constexpr uint64_t kQ4KGemmMinRows = 24;
-constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{8} << 20;
+constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 
 qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,

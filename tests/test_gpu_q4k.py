@@ -114,10 +114,12 @@ def test_rows_kernels(backend, rows):
     assert e.value.code == StatusCode.InvalidArgument
 
 
-# Matrices of 8M weights and more take 2..23 rows through the few-row MFMA kernel (eight rows a
-# pass, activations as fp16 hi/lo pairs with a per-row power-of-two scale); the shapes cover
-# k/256 divisible by 4, by 2 only and odd (its three tilings), ragged n, and every pass count.
-FEW_ROW_SHAPES = [(2048, 4096), (1030, 8192), (515, 17408), (4100, 2048), (3700, 2304), (5500, 1536)]
+# Matrices of 16M weights and more take 2..23 rows through the few-row MFMA kernels (eight rows a
+# pass, activations as fp16 hi/lo pairs with a per-row power-of-two scale; up to four rows with
+# the activations resident in LDS when n is a multiple of 4, else streamed per stage); the shapes
+# cover k/256 divisible by 4, by 2 only and odd (the tilings), k/256 not a multiple of 8 (ragged
+# stages), n not a multiple of 4, and every pass count.
+FEW_ROW_SHAPES = [(4096, 4096), (2060, 8192), (1030, 17408), (8200, 2048), (7400, 2304), (11000, 1536), (8194, 2048)]
 
 
 @pytest.mark.parametrize("n,k", FEW_ROW_SHAPES)
@@ -135,7 +137,7 @@ def test_few_rows_match_oracle(backend, n, k, m):
 
 
 def test_few_rows_scaling_and_exactness(backend):
-    n, k = 2048, 4096
+    n, k = 4096, 4096
     g = synth.rng(31337)
     w = synth.q4k_weights(g, n, k)
     deq = oracle.dequantize_q4k(w).reshape(n, k)

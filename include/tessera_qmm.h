@@ -51,9 +51,12 @@ typedef uintptr_t qmm_kernel;
 
 /* Backend::SetDeviceIndex + Backend::Init (backend.hpp:869-889;
  * rocm_backend.cpp:270-333).  Selects the device, checks that it is a gfx950 part
- * and that the library's code object loads.  Ok when already initialised on the same
- * device; InvalidArgument for an index out of range; UnsupportedFeature on a device
- * that is not gfx950; DeviceError for any HIP failure. */
+ * and that the library's code object loads, and allocates the 16 MB scratch of the
+ * decode-sized kernels (held until the process ends, at a fixed address, so decode
+ * launches never allocate and may be recorded into a HIP graph).  Ok when already
+ * initialised on the same device; InvalidArgument for an index out of range;
+ * UnsupportedFeature on a device that is not gfx950; OutOfMemory / DeviceError for a
+ * HIP failure. */
 qmm_status qmm_init(int device);
 
 /* Backend::DeviceName (backend.hpp:853-854).  Valid after qmm_init; "" before. */

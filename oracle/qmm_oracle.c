@@ -18,6 +18,8 @@
  * Pin status:
  *   fp16/bf16/e4m3/e8m0/e2m1 codecs ......... pinned (exhaustive)
  *   Q4_K scale unpack + block decode ........ pinned (bit-serial brute force, closed form)
+ *   Q6_K block decode + gemm ................ pinned (bit-serial extraction from the layout text,
+ *                                             closed form d*s*(q-32) exact in fp32, one-hot)
  *   fp8 per-row quantize (QDQ and pack) ..... pinned (invariants + torch.float8_e4m3fn)
  *   gemm_* sequential-fma references ........ pinned (one-hot identity, float64 bound)
  *   MXFP4->e4m3 fold table .................. pinned (the reference's literal 16x8 table, kept
@@ -41,6 +43,7 @@
 
 #define Q4K_ELEMS 256u
 #define Q4K_BYTES 144u
+#define Q6K_BYTES 210u
 #define MX_BLOCK 32u
 
 /* quant.hpp:58-64 */
@@ -320,6 +323,69 @@ int orc_gemm_q4k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_
   }
   free(row);
   return ORC_OK;
+}
+
+/* ---- Q6_K block decode (quant.cpp:421-450; layout quant.hpp:597-600): 210 bytes = ql[128]
+ *      low nibbles, qh[64] two high bits each, 16 int8 scales, fp16 d; 256 values.  For half
+ *      n in 0..1 and l in 0..31, is = l / 16:
+ *        out[n*128 +  0 + l] = d * s[n*8 + is + 0] * (((ql[n*64 + l]      & 15) | ((qh[n*32+l] >> 0 & 3) << 4)) - 32)
+ *        out[n*128 + 32 + l] = d * s[n*8 + is + 2] * (((ql[n*64 + 32 + l] & 15) | ((qh[n*32+l] >> 2 & 3) << 4)) - 32)
+ *        out[n*128 + 64 + l] = d * s[n*8 + is + 4] * (((ql[n*64 + l]      >> 4) | ((qh[n*32+l] >> 4 & 3) << 4)) - 32)
+ *        out[n*128 + 96 + l] = d * s[n*8 + is + 6] * (((ql[n*64 + 32 + l] >> 4) | ((qh[n*32+l] >> 6 & 3) << 4)) - 32)
+ *      evaluated as (d * s) * (q - 32) in fp32, both products exact (11 + 8 + 6 bits). ---- */
+void orc_dequantize_q6k(const uint8_t* blk, float* out) {
+  const uint8_t* ql = blk;
+  const uint8_t* qh = blk + 128;
+  const int8_t* sc = (const int8_t*)(blk + 192);
+  const float d = orc_fp16_to_float((uint16_t)(blk[208] | (blk[209] << 8)));
+  for (size_t n = 0; n < 2; ++n) {
+    for (size_t l = 0; l < 32; ++l) {
+      const size_t is = l / 16;
+      const uint8_t h = qh[n * 32 + l];
+      const int q1 = (ql[n * 64 + l] & 0xF) | (((h >> 0) & 3) << 4);
+      const int q2 = (ql[n * 64 + 32 + l] & 0xF) | (((h >> 2) & 3) << 4);
+      const int q3 = (ql[n * 64 + l] >> 4) | (((h >> 4) & 3) << 4);
+      const int q4 = (ql[n * 64 + 32 + l] >> 4) | (((h >> 6) & 3) << 4);
+      out[n * 128 + l] = d * (float)sc[n * 8 + is + 0] * (float)(q1 - 32);
+      out[n * 128 + 32 + l] = d * (float)sc[n * 8 + is + 2] * (float)(q2 - 32);
+      out[n * 128 + 64 + l] = d * (float)sc[n * 8 + is + 4] * (float)(q3 - 32);
+      out[n * 128 + 96 + l] = d * (float)sc[n * 8 + is + 6] * (float)(q4 - 32);
+    }
+  }
+}
+
+void orc_dequantize_q6k_rows(const uint8_t* w, float* out, size_t nblocks) {
+  for (size_t b = 0; b < nblocks; ++b) orc_dequantize_q6k(w + b * Q6K_BYTES, out + b * Q4K_ELEMS);
+}
+
+/* ---- C = A . deq(W)^T, Q6_K rows, sequential fp32 fma (gemm.cpp:18-41,88-99); weight rows
+ *      spread over OpenMP threads when `threads` is non-zero (each output keeps its chain). ---- */
+int orc_gemm_q6k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k,
+                     int threads) {
+  if (m == 0 || n == 0 || k == 0 || k % Q4K_ELEMS != 0) return ORC_INVALID_ARGUMENT;
+  const size_t bpr = k / Q4K_ELEMS;
+  int failed = 0;
+#pragma omp parallel if (threads)
+  {
+    float* row = (float*)malloc(k * sizeof(float));
+    if (!row) {
+#pragma omp atomic write
+      failed = 1;
+    }
+#pragma omp for schedule(static)
+    for (long long j = 0; j < (long long)n; ++j) {
+      if (!row) continue;
+      orc_dequantize_q6k_rows(w + (size_t)j * bpr * Q6K_BYTES, row, bpr);
+      for (size_t i = 0; i < m; ++i) {
+        const float* ar = a + i * k;
+        float acc = 0.0f;
+        for (size_t t = 0; t < k; ++t) acc = fmaf(ar[t], row[t], acc);
+        c[i * n + (size_t)j] = acc;
+      }
+    }
+    free(row);
+  }
+  return failed ? ORC_OOM : ORC_OK;
 }
 
 /* Same arithmetic, weight rows spread over OpenMP threads.  Each output keeps

@@ -129,6 +129,28 @@ __global__ __launch_bounds__(256) void mxfp4_row_ref_kernel(const uint8_t* __res
   if ((threadIdx.x & 63u) == 0) wref[r] = static_cast<uint8_t>(ref);
 }
 
+// fp32 dump of Q6_K blocks, one thread per (half n, lane l): the four values that share the
+// bytes ql[n*64 + l], ql[n*64 + 32 + l] and qh[n*32 + l].  Same arithmetic as the reference
+// decode (src/core/numerics/quant.cpp:421-450): (d * s) * (q - 32), both products exact.
+__global__ __launch_bounds__(256) void dequant_q6k_kernel(const uint8_t* __restrict__ w,
+                                                          float* __restrict__ out, uint64_t nitems) {
+  const uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= nitems) return;
+  const uint64_t blk = t >> 6;
+  const uint32_t n = static_cast<uint32_t>(t >> 5) & 1u, l = static_cast<uint32_t>(t) & 31u, is = l >> 4;
+  const uint8_t* base = w + blk * 210u;
+  const uint32_t a = base[n * 64 + l], b = base[n * 64 + 32 + l], h = base[128 + n * 32 + l];
+  const float d = half_bits_to_float(static_cast<uint32_t>(base[208]) | (static_cast<uint32_t>(base[209]) << 8));
+  const int q[4] = {static_cast<int>((a & 15u) | ((h & 3u) << 4)), static_cast<int>((b & 15u) | (((h >> 2) & 3u) << 4)),
+                    static_cast<int>((a >> 4) | (((h >> 4) & 3u) << 4)), static_cast<int>((b >> 4) | ((h >> 6) << 4))};
+  float* dst = out + blk * 256 + n * 128 + l;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float s = static_cast<float>(static_cast<int8_t>(base[192 + n * 8 + is + 2 * j]));
+    dst[32 * j] = d * s * static_cast<float>(q[j] - 32);
+  }
+}
+
 // fp32 dump of Q4_K blocks, one thread per 16-byte quant chunk (32 values).  Same
 // arithmetic as the reference decode (src/core/numerics/quant.cpp:656-675):
 // (d*sc)*q - dmin*mn with exact products and one rounding.
@@ -322,6 +344,12 @@ hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float
 hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uint64_t k,
                                 hipStream_t stream) {
   hipLaunchKernelGGL(mxfp4_row_ref_kernel, grid_for(n, 4), dim3(256), 0, stream, w, wref, n, k);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant_q6k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream) {
+  hipLaunchKernelGGL(dequant_q6k_kernel, grid_for(nblocks * 64, 256), dim3(256), 0, stream, w, out,
+                     nblocks * 64);
   return hipGetLastError();
 }
 

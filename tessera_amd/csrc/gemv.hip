@@ -420,6 +420,137 @@ struct Q4KPairCodec {
 };
 
 // ----------------------------------------------------------------------------
+// Q6_K: 210-byte super-block = ql[128] low nibbles, qh[64] two high bits each, 16 int8
+// scales, fp16 d; value = d * s * (q - 32) (reference decode src/core/numerics/quant.cpp:421-450,
+// layout quant.hpp:597-600, device twin src/backends/rocm/rocm_kernels_codec.hpp:132-176).
+// A chunk is 64 weights: half n of the block, lanes l = is*16 .. is*16+15 of its four quarters
+// (chunk = 4*block + 2*n + is), i.e. 16 bytes of ql at n*64 + is*16, 16 more 32 bytes further,
+// 16 bytes of qh at 128 + n*32 + is*16, and the scales n*8 + is + {0,2,4,6}.  Blocks are only
+// 2-byte aligned (210 = 2 * 105), so every load is an unaligned one.
+//
+// sum_i x_i * d*s*(q_i - 32) = d * s * (sum_i x_i q_i - 32 * sum_i x_i) per quarter, the second
+// sum a per-thread constant.  The six-bit q of four lanes is assembled in one register (byte
+// masks and shifts) and converted with v_cvt_f32_ubyte*.  d*s and s*(q-32) are exact in fp32, so
+// a one-hot activation returns the reference's dequantized weight bit for bit.
+// ----------------------------------------------------------------------------
+struct Q6KCodec {
+  struct Args {
+    const float* a;
+    const uint8_t* w;
+    uint32_t k;
+  };
+  template <int R>
+  struct X {
+    float v[R][4][16];   // quarter j, lane l - is*16
+    float s32[R][4];     // 32 * sum over the 16 lanes of quarter j
+    uint32_t sc_shift;   // is * 8: byte of the scale words
+  };
+  struct Frag {
+    uint4 ql0, ql1, qh;
+    uint2 sc;            // the eight scales of half n
+    uint32_t d;          // fp16 bits
+  };
+  typedef uint4 uint4_u __attribute__((aligned(2)));
+  typedef uint2 uint2_u __attribute__((aligned(2)));
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 64u; }
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return (chunk >> 1) * 128u; }
+
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    const uint32_t is = chunk & 1u;
+    x.sc_shift = is * 8u;
+    const uint32_t k0 = (chunk >> 1) * 128u + is * 16u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) {
+          float4 f = src(r, k0 + j * 32 + i);
+          if (!valid) f = make_float4(0.f, 0.f, 0.f, 0.f);
+          x.v[r][j][i] = f.x, x.v[r][j][i + 1] = f.y, x.v[r][j][i + 2] = f.z, x.v[r][j][i + 3] = f.w;
+          sum += (f.x + f.y) + (f.z + f.w);
+        }
+        x.s32[r][j] = 32.0f * sum;
+      }
+    }
+  }
+
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t blk = prow * (cpr >> 2) * 210u + (chunk >> 2) * 210u;
+    const uint32_t n = (chunk >> 1) & 1u, is = chunk & 1u;
+    return Lane{blk, n * 64u + is * 16u};   // block start; offset of this chunk's first ql bytes
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const uint8_t* blk = p.w + static_cast<size_t>(row) * ((cpr >> 2) * 210u) + ln.off0;
+    const uint32_t n = ln.off1 >> 6, is16 = ln.off1 & 16u;
+    f.ql0 = *reinterpret_cast<const uint4_u*>(blk + ln.off1);
+    f.ql1 = *reinterpret_cast<const uint4_u*>(blk + ln.off1 + 32u);
+    f.qh = *reinterpret_cast<const uint4_u*>(blk + 128u + n * 32u + is16);
+    f.sc = *reinterpret_cast<const uint2_u*>(blk + 192u + n * 8u);
+    f.d = *reinterpret_cast<const uint16_t*>(blk + 208u);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const float d = half_bits_to_float(f.d);
+    // scales n*8 + is + {0,2,4,6}: bytes is, is+2 of each word
+    const uint32_t w0 = f.sc.x >> x.sc_shift, w1 = f.sc.y >> x.sc_shift;
+    const float s[4] = {static_cast<float>(static_cast<int8_t>(w0 & 0xFFu)),
+                        static_cast<float>(static_cast<int8_t>((w0 >> 16) & 0xFFu)),
+                        static_cast<float>(static_cast<int8_t>(w1 & 0xFFu)),
+                        static_cast<float>(static_cast<int8_t>((w1 >> 16) & 0xFFu))};
+    const uint32_t a4[4] = {f.ql0.x, f.ql0.y, f.ql0.z, f.ql0.w};
+    const uint32_t b4[4] = {f.ql1.x, f.ql1.y, f.ql1.z, f.ql1.w};
+    const uint32_t h4[4] = {f.qh.x, f.qh.y, f.qh.z, f.qh.w};
+    float acc[R][4];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[r][j] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t a = a4[i], b = b4[i], h = h4[i];
+      const uint32_t q[4] = {(a & 0x0F0F0F0Fu) | ((h & 0x03030303u) << 4),
+                             (b & 0x0F0F0F0Fu) | ((h & 0x0C0C0C0Cu) << 2),
+                             ((a >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u),
+                             ((b >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float q0 = static_cast<float>(q[j] & 0xFFu), q1 = static_cast<float>((q[j] >> 8) & 0xFFu);
+        const float q2 = static_cast<float>((q[j] >> 16) & 0xFFu), q3 = static_cast<float>(q[j] >> 24);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          acc[r][j] = fmaf(x.v[r][j][4 * i + 0], q0, acc[r][j]);
+          acc[r][j] = fmaf(x.v[r][j][4 * i + 1], q1, acc[r][j]);
+          acc[r][j] = fmaf(x.v[r][j][4 * i + 2], q2, acc[r][j]);
+          acc[r][j] = fmaf(x.v[r][j][4 * i + 3], q3, acc[r][j]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float t = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t = fmaf(d * s[j], acc[r][j] - x.s32[r][j], t);
+      out[r] = t;
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+
+// ----------------------------------------------------------------------------
 // MXFP4 with fp32 activations: packed buffer = n*k/2 nibble bytes (low nibble =
 // even element) then n*k/32 E8M0 bytes (include/tessera/backend.hpp:195-201;
 // src/core/numerics/gemm.cpp:311-344).  A 16-byte chunk is exactly one 32-element
@@ -1052,6 +1183,29 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
       e = launch_gemv_r<Q4KCodec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
     } else {
       e = launch_gemv_r<Q4KPairCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
+    }
+    if (e != hipSuccess) return e;
+    r0 += took;
+  }
+  return hipSuccess;
+}
+
+// Q6_K: a lane keeps the 64 activations of its chunk per row in registers, so two rows share a
+// weight pass (k <= 32768) and further rows take further passes.
+bool gemv_q6k_supported(uint64_t k) { return k % 256 == 0 && k / 64 <= 768; }
+
+hipError_t launch_q6k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                           uint32_t k, hipStream_t stream) {
+  const uint32_t row_threads = (k / 64u + 63u) / 64u * 64u;
+  for (uint32_t r0 = 0; r0 < m;) {
+    Q6KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
+    float* out = c + static_cast<size_t>(r0) * n;
+    hipError_t e;
+    uint32_t took;
+    if (m - r0 >= 2 && row_threads <= 512u) {
+      e = launch_gemv_r<Q6KCodec, 2, 512, 2, 6>(args, out, n, k, n, stream), took = 2;
+    } else {
+      e = launch_gemv_r<Q6KCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;

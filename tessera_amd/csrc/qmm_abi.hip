@@ -48,7 +48,7 @@ qmm_status map_hip(hipError_t e) {
   return QMM_DEVICE_ERROR;
 }
 
-qmm_status bad(const char* why) {
+qmm_status bad(const std::string& why) {
   g_last_error = why;
   return QMM_INVALID_ARGUMENT;
 }
@@ -202,6 +202,58 @@ qmm_status run_dequant_q4k(const LaunchCtx& c) {
     return bad("dequant_q4k: a buffer is smaller than nblocks requires");
   }
   return map_hip(qmm::launch_dequant_q4k(c.ptr<const uint8_t>(0), c.ptr<float>(1), nb, c.stream));
+}
+
+// ---- Q6_K ---------------------------------------------------------------------
+// "gemm_q6k", "gemm_q6k_batched": buffers A, W, C; scalars m, n, k, k a multiple of 256
+// (include/tessera/backend.hpp:202-206,524-536).  "gemm_q6k_vec", "gemm_q6k_rows{R}": the same
+// plus `split`, with the partials contract of the Q4_K ids
+// (src/backends/rocm/rocm_backend.cpp:102-108; rocm_kernels_gemv.cpp:19-24,107-156).
+u128 q6k_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * (k / 256) * 210; }
+
+qmm_status q6k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, uint64_t split, const char* who) {
+  if (!dims_ok(m, n, k) || k % 256 != 0) return bad(std::string(who) + ": m, n, k must be non-zero and k a multiple of 256");
+  if (split == 0 || split > 64 || (k / 256) % split != 0) return bad(std::string(who) + ": split must divide k/256");
+  const u128 region = static_cast<u128>(m) * n * 4;
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, q6k_bytes(n, k)) || !c.fits(2, region * split)) {
+    return bad(std::string(who) + ": a buffer is smaller than m, n, k require");
+  }
+  if (!qmm::gemv_q6k_supported(k)) {
+    g_last_error = "Q6_K: k above 49152 is not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  float* out = c.ptr<float>(2);
+  qmm_status st = map_hip(qmm::launch_q6k_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out,
+                                               static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                               static_cast<uint32_t>(k), c.stream));
+  if (st == QMM_OK && split > 1) st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
+  return st;
+}
+
+qmm_status run_gemm_q6k(const LaunchCtx& c) {
+  if (!counts(c, 3, 3)) return bad("gemm_q6k: expects 3 buffers and 3 scalars");
+  return q6k_matmul(c, c.sc[0], c.sc[1], c.sc[2], 1, "gemm_q6k");
+}
+qmm_status run_gemm_q6k_split(const LaunchCtx& c, uint64_t rows_required) {
+  if (!counts(c, 3, 4)) return bad("gemm_q6k_vec/rows: expects 3 buffers and 4 scalars");
+  if (rows_required != 0 && c.sc[0] != rows_required) return bad("gemm_q6k_rowsR: m must equal R");
+  return q6k_matmul(c, c.sc[0], c.sc[1], c.sc[2], c.sc[3], "gemm_q6k_vec/rows");
+}
+qmm_status run_gemm_q6k_vec(const LaunchCtx& c) { return run_gemm_q6k_split(c, 0); }
+qmm_status run_gemm_q6k_rows2(const LaunchCtx& c) { return run_gemm_q6k_split(c, 2); }
+qmm_status run_gemm_q6k_rows3(const LaunchCtx& c) { return run_gemm_q6k_split(c, 3); }
+qmm_status run_gemm_q6k_rows4(const LaunchCtx& c) { return run_gemm_q6k_split(c, 4); }
+qmm_status run_gemm_q6k_rows5(const LaunchCtx& c) { return run_gemm_q6k_split(c, 5); }
+
+// "dequant_q6k" (not a reference id): buffers W, Out (fp32); scalar nblocks.
+qmm_status run_dequant_q6k(const LaunchCtx& c) {
+  if (!counts(c, 2, 1)) return bad("dequant_q6k: expects 2 buffers and 1 scalar");
+  const uint64_t nb = c.sc[0];
+  if (nb == 0 || nb > (1ull << 32)) return bad("dequant_q6k: bad block count");
+  if (!c.fits(0, static_cast<u128>(nb) * 210) || !c.fits(1, static_cast<u128>(nb) * 1024)) {
+    return bad("dequant_q6k: a buffer is smaller than nblocks requires");
+  }
+  return map_hip(qmm::launch_dequant_q6k(c.ptr<const uint8_t>(0), c.ptr<float>(1), nb, c.stream));
 }
 
 // ---- MXFP4 / FP8 ---------------------------------------------------------------
@@ -537,6 +589,14 @@ const Entry kTable[] = {
     {"moe_gate", run_moe_gate},
     {"top_k_rows", run_top_k_rows},
     {"dequant_q4k", run_dequant_q4k},
+    {"gemm_q6k", run_gemm_q6k},
+    {"gemm_q6k_batched", run_gemm_q6k},
+    {"gemm_q6k_vec", run_gemm_q6k_vec},
+    {"gemm_q6k_rows2", run_gemm_q6k_rows2},
+    {"gemm_q6k_rows3", run_gemm_q6k_rows3},
+    {"gemm_q6k_rows4", run_gemm_q6k_rows4},
+    {"gemm_q6k_rows5", run_gemm_q6k_rows5},
+    {"dequant_q6k", run_dequant_q6k},
     {"dequant_mxfp4", run_dequant_mxfp4},
     {"quantize_fp8_pack_a16", run_quantize_fp8_pack_a16},
 };

@@ -50,6 +50,22 @@ def q4k_weights(g: np.random.Generator, n: int, k: int) -> np.ndarray:
     return blocks.reshape(-1)
 
 
+Q6K_BYTES = 210
+
+
+def q6k_weights(g: np.random.Generator, n: int, k: int) -> np.ndarray:
+    """n x k Q6_K matrix (210-byte super-blocks: 128 low-nibble bytes, 64 bytes of 2-bit highs,
+    16 int8 scales, fp16 d): quants and scales uniform over their whole ranges (scales include
+    negative values and -128), d ~ U[1e-4, 2e-3] rounded to fp16.  Flat uint8 array."""
+    assert k % Q4K_ELEMS == 0
+    nb = n * (k // Q4K_ELEMS)
+    blocks = np.empty((nb, Q6K_BYTES), dtype=np.uint8)
+    blocks[:, 0:208] = g.integers(0, 256, size=(nb, 208), dtype=np.uint8)
+    d = g.uniform(1e-4, 2e-3, size=(nb, 1)).astype(np.float32).astype(np.float16)
+    blocks[:, 208:210] = d.view(np.uint8).reshape(nb, 2)
+    return blocks.reshape(-1)
+
+
 def mxfp4_weights(g: np.random.Generator, n: int, k: int, exp_lo: int = -8,
                   exp_hi: int = -4) -> np.ndarray:
     """Packed MXFP4: E2M1 codes uniform over the 16 values, E8M0 exponent uniform in

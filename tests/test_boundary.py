@@ -20,7 +20,8 @@ REFERENCE_IDS = [
     "gemm_mxfp4_rows", "gemm_mxfp4_batched", "mxfp4_row_ref", "gemm_mxfp4_wmma",
     "gemm_mxfp4_wmma_reduce", "quantize_fp8", "quantize_fp8_pack", "quantize_fp8_pack_rows",
     "gemm_fp8", "moe_scale_add", "moe_experts_gate_up_q4k", "moe_experts_down_q4k", "moe_gate",
-    "top_k_rows",
+    "top_k_rows", "gemm_q6k", "gemm_q6k_vec", "gemm_q6k_rows2", "gemm_q6k_rows3", "gemm_q6k_rows4",
+    "gemm_q6k_rows5", "gemm_q6k_batched",
 ]
 
 

@@ -158,23 +158,24 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     out["q4k_few_rows_17408x5120"] = few
     del wq_list, w_q1
 
-    # ---- Q6_K (the other block format of Q4_K_M files), gate/up and down shapes, M = 1 and 2 ----
-    q6 = {}
-    kv6 = backend.LoadKernel("gemm_q6k_batched")
-    for label, (nn, kk) in (("17408x5120", (n, k)), ("5120x17408", (k, n))):
-        w6 = to_dev(synth.q6k_weights(g, nn, kk))
-        w6_list = [w6] + [w6.clone() for _ in range(5)]
-        for m in (1, 2):
-            x = to_dev(synth.activations_f32(g, m, kk))
-            y = torch.empty(m * nn, dtype=torch.float32, device=dev)
-            launches = [(kv6, KernelLaunch(grid_x=(m * nn + 7) // 8, buffers=[wrap(x), wrap(w), wrap(y)],
-                                           scalars=[m, nn, kk])) for w in w6_list]
-            us = timed_us(launches, 10) / len(w6_list)
-            nbytes = nn * (kk // 256) * 210 + 4 * m * kk + 4 * m * nn
-            q6[f"{label}_m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
-                                   "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-        del w6_list, w6
-    out["q6k_gemv"] = q6
+    # ---- Q6_K and Q5_K (the other block formats of K-quant files), gate/up and down shapes --------
+    for fmt, block_bytes, gen, rows in (("q6k", 210, synth.q6k_weights, (1, 2)), ("q5k", 176, synth.q5k_weights, (1,))):
+        res = {}
+        kern = backend.LoadKernel(f"gemm_{fmt}_batched")
+        for label, (nn, kk) in (("17408x5120", (n, k)), ("5120x17408", (k, n))):
+            wf = to_dev(gen(g, nn, kk))
+            wf_list = [wf] + [wf.clone() for _ in range(5)]
+            for m in rows:
+                x = to_dev(synth.activations_f32(g, m, kk))
+                y = torch.empty(m * nn, dtype=torch.float32, device=dev)
+                launches = [(kern, KernelLaunch(grid_x=(m * nn + 7) // 8, buffers=[wrap(x), wrap(w), wrap(y)],
+                                                scalars=[m, nn, kk])) for w in wf_list]
+                us = timed_us(launches, 10) / len(wf_list)
+                nbytes = nn * (kk // 256) * block_bytes + 4 * m * kk + 4 * m * nn
+                res[f"{label}_m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                        "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+            del wf_list, wf
+        out[f"{fmt}_gemv"] = res
 
     # ---- configs[3]: prefill GEMM M=2048 ---------------------------------------------------
     m = 2048

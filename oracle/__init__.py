@@ -18,6 +18,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 Q4K_ELEMS = 256
 Q4K_BYTES = 144
+Q5K_BYTES = 176
 Q6K_BYTES = 210
 
 
@@ -51,6 +52,9 @@ def _load() -> C.CDLL:
         "orc_quantize_fp8_pack_ref": (C.c_int, [f32p, u8p, f32p, sz, sz]),
         "orc_gemm_q4k_ref": (C.c_int, [f32p, u8p, f32p, sz, sz, sz]),
         "orc_gemm_q4k_ref_omp": (C.c_int, [f32p, u8p, f32p, sz, sz, sz]),
+        "orc_dequantize_q5k": (None, [u8p, f32p]),
+        "orc_dequantize_q5k_rows": (None, [u8p, f32p, sz]),
+        "orc_gemm_q5k_ref": (C.c_int, [f32p, u8p, f32p, sz, sz, sz, C.c_int]),
         "orc_dequantize_q6k": (None, [u8p, f32p]),
         "orc_dequantize_q6k_rows": (None, [u8p, f32p, sz]),
         "orc_gemm_q6k_ref": (C.c_int, [f32p, u8p, f32p, sz, sz, sz, C.c_int]),
@@ -182,6 +186,26 @@ def gemm_q4k(a, w, m: int, n: int, k: int, threads: bool = False) -> np.ndarray:
     c = np.empty((m, n), dtype=np.float32)
     fn = _lib.orc_gemm_q4k_ref_omp if threads else _lib.orc_gemm_q4k_ref
     _check(fn(_p(a, C.c_float), _p(w, C.c_uint8), _p(c, C.c_float), m, n, k))
+    return c
+
+
+# ---- Q5_K ----------------------------------------------------------------
+def dequantize_q5k(w) -> np.ndarray:
+    """Any whole number of 176-byte super-blocks -> fp32, 256 values per block."""
+    w = _u8(w).reshape(-1)
+    assert w.size % Q5K_BYTES == 0
+    nb = w.size // Q5K_BYTES
+    out = np.empty(nb * Q4K_ELEMS, dtype=np.float32)
+    _lib.orc_dequantize_q5k_rows(_p(w, C.c_uint8), _p(out, C.c_float), nb)
+    return out
+
+
+def gemm_q5k(a, w, m: int, n: int, k: int, threads: bool = False) -> np.ndarray:
+    a, w = _f32(a), _u8(w)
+    if k % Q4K_ELEMS == 0 and k and n and m:
+        assert a.size == m * k and w.size == n * (k // Q4K_ELEMS) * Q5K_BYTES
+    c = np.empty((m, n), dtype=np.float32)
+    _check(_lib.orc_gemm_q5k_ref(_p(a, C.c_float), _p(w, C.c_uint8), _p(c, C.c_float), m, n, k, int(threads)))
     return c
 
 

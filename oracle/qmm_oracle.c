@@ -18,6 +18,8 @@
  * Pin status:
  *   fp16/bf16/e4m3/e8m0/e2m1 codecs ......... pinned (exhaustive)
  *   Q4_K scale unpack + block decode ........ pinned (bit-serial brute force, closed form)
+ *   Q5_K block decode + gemm ................ pinned (bit-serial extraction from the layout text,
+ *                                             closed form RN32(d*sc*q - dmin*mn), one-hot)
  *   Q6_K block decode + gemm ................ pinned (bit-serial extraction from the layout text,
  *                                             closed form d*s*(q-32) exact in fp32, one-hot)
  *   fp8 per-row quantize (QDQ and pack) ..... pinned (invariants + torch.float8_e4m3fn)
@@ -43,6 +45,7 @@
 
 #define Q4K_ELEMS 256u
 #define Q4K_BYTES 144u
+#define Q5K_BYTES 176u
 #define Q6K_BYTES 210u
 #define MX_BLOCK 32u
 
@@ -323,6 +326,65 @@ int orc_gemm_q4k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_
   }
   free(row);
   return ORC_OK;
+}
+
+/* ---- Q5_K block decode (quant.cpp:388-419; layout quant.hpp:592-595): 176 bytes = fp16 d, fp16
+ *      dmin, 12 bytes of 6-bit scales/mins packed as in Q4_K, qh[32] high bits, qs[128] low
+ *      nibbles; 256 values.  For group g in 0..3 and l in 0..31:
+ *        out[g*64 + l]      = d*sc[2g]   * ((qs[g*32+l] & 15) + 16*bit(qh[l], 2g))   - dmin*mn[2g]
+ *        out[g*64 + 32 + l] = d*sc[2g+1] * ((qs[g*32+l] >> 4) + 16*bit(qh[l], 2g+1)) - dmin*mn[2g+1]
+ *      with d*sc and dmin*mn formed first in fp32 (both exact), one rounding at the subtract. ---- */
+void orc_dequantize_q5k(const uint8_t* blk, float* out) {
+  const float d = orc_fp16_to_float((uint16_t)(blk[0] | (blk[1] << 8)));
+  const float dmin = orc_fp16_to_float((uint16_t)(blk[2] | (blk[3] << 8)));
+  const uint8_t* scales = blk + 4;
+  const uint8_t* qh = blk + 16;
+  const uint8_t* qs = blk + 48;
+  for (size_t g = 0; g < 4; ++g) {
+    uint8_t sc0, mn0, sc1, mn1;
+    orc_get_scale_min(2 * g, scales, &sc0, &mn0);
+    orc_get_scale_min(2 * g + 1, scales, &sc1, &mn1);
+    const float d1 = d * (float)sc0, m1 = dmin * (float)mn0;
+    const float d2 = d * (float)sc1, m2 = dmin * (float)mn1;
+    for (size_t l = 0; l < 32; ++l) {
+      const uint8_t low = qs[g * 32 + l], high = qh[l];
+      out[g * 64 + l] = d1 * ((float)(low & 0xF) + (((high >> (2 * g)) & 1) ? 16.0f : 0.0f)) - m1;
+      out[g * 64 + 32 + l] = d2 * ((float)(low >> 4) + (((high >> (2 * g + 1)) & 1) ? 16.0f : 0.0f)) - m2;
+    }
+  }
+}
+
+void orc_dequantize_q5k_rows(const uint8_t* w, float* out, size_t nblocks) {
+  for (size_t b = 0; b < nblocks; ++b) orc_dequantize_q5k(w + b * Q5K_BYTES, out + b * Q4K_ELEMS);
+}
+
+/* ---- C = A . deq(W)^T, Q5_K rows, sequential fp32 fma (gemm.cpp:18-41,75-86). ---- */
+int orc_gemm_q5k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k,
+                     int threads) {
+  if (m == 0 || n == 0 || k == 0 || k % Q4K_ELEMS != 0) return ORC_INVALID_ARGUMENT;
+  const size_t bpr = k / Q4K_ELEMS;
+  int failed = 0;
+#pragma omp parallel if (threads)
+  {
+    float* row = (float*)malloc(k * sizeof(float));
+    if (!row) {
+#pragma omp atomic write
+      failed = 1;
+    }
+#pragma omp for schedule(static)
+    for (long long j = 0; j < (long long)n; ++j) {
+      if (!row) continue;
+      orc_dequantize_q5k_rows(w + (size_t)j * bpr * Q5K_BYTES, row, bpr);
+      for (size_t i = 0; i < m; ++i) {
+        const float* ar = a + i * k;
+        float acc = 0.0f;
+        for (size_t t = 0; t < k; ++t) acc = fmaf(ar[t], row[t], acc);
+        c[i * n + (size_t)j] = acc;
+      }
+    }
+    free(row);
+  }
+  return failed ? ORC_OOM : ORC_OK;
 }
 
 /* ---- Q6_K block decode (quant.cpp:421-450; layout quant.hpp:597-600): 210 bytes = ql[128]

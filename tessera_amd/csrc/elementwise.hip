@@ -129,6 +129,39 @@ __global__ __launch_bounds__(256) void mxfp4_row_ref_kernel(const uint8_t* __res
   if ((threadIdx.x & 63u) == 0) wref[r] = static_cast<uint8_t>(ref);
 }
 
+// fp32 dump of Q5_K blocks, one thread per quant byte (group g, lane l): the two values that
+// share qs[g*32 + l].  Same arithmetic as the reference decode
+// (src/core/numerics/quant.cpp:388-419): (d*sc)*q - dmin*mn, products exact, one rounding.
+__global__ __launch_bounds__(256) void dequant_q5k_kernel(const uint8_t* __restrict__ w,
+                                                          float* __restrict__ out, uint64_t nitems) {
+  const uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= nitems) return;
+  const uint64_t blk = t >> 7;
+  const uint32_t g = static_cast<uint32_t>(t >> 5) & 3u, l = static_cast<uint32_t>(t) & 31u;
+  const uint8_t* base = w + blk * 176u;
+  const uint8_t* p = base + 4;
+  auto scale_min = [&](uint32_t sb, uint32_t& sc, uint32_t& mn) {
+    if (sb < 4) {
+      sc = p[sb] & 63u;
+      mn = p[sb + 4] & 63u;
+    } else {
+      sc = (p[sb + 4] & 15u) | ((p[sb - 4] >> 6) << 4);
+      mn = (p[sb + 4] >> 4) | ((p[sb] >> 6) << 4);
+    }
+  };
+  uint32_t sca, mna, scb, mnb;
+  scale_min(2 * g, sca, mna);
+  scale_min(2 * g + 1, scb, mnb);
+  const float d = half_bits_to_float(static_cast<uint32_t>(base[0]) | (static_cast<uint32_t>(base[1]) << 8));
+  const float dmin = half_bits_to_float(static_cast<uint32_t>(base[2]) | (static_cast<uint32_t>(base[3]) << 8));
+  const uint32_t low = base[48 + g * 32 + l], high = base[16 + l];
+  const float q0 = static_cast<float>((low & 15u) + (((high >> (2 * g)) & 1u) << 4));
+  const float q1 = static_cast<float>((low >> 4) + (((high >> (2 * g + 1)) & 1u) << 4));
+  float* dst = out + blk * 256 + g * 64 + l;
+  dst[0] = d * static_cast<float>(sca) * q0 - dmin * static_cast<float>(mna);
+  dst[32] = d * static_cast<float>(scb) * q1 - dmin * static_cast<float>(mnb);
+}
+
 // fp32 dump of Q6_K blocks, one thread per (half n, lane l): the four values that share the
 // bytes ql[n*64 + l], ql[n*64 + 32 + l] and qh[n*32 + l].  Same arithmetic as the reference
 // decode (src/core/numerics/quant.cpp:421-450): (d * s) * (q - 32), both products exact.
@@ -344,6 +377,12 @@ hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float
 hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uint64_t k,
                                 hipStream_t stream) {
   hipLaunchKernelGGL(mxfp4_row_ref_kernel, grid_for(n, 4), dim3(256), 0, stream, w, wref, n, k);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant_q5k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream) {
+  hipLaunchKernelGGL(dequant_q5k_kernel, grid_for(nblocks * 128, 256), dim3(256), 0, stream, w, out,
+                     nblocks * 128);
   return hipGetLastError();
 }
 

@@ -420,6 +420,134 @@ struct Q4KPairCodec {
 };
 
 // ----------------------------------------------------------------------------
+// Q5_K: 176-byte super-block = fp16 d, fp16 dmin, 12 bytes of 6-bit scales/mins (packed as in
+// Q4_K), qh[32] fifth bits, qs[128] low nibbles; value = d*sc*(nibble + 16*bit) - dmin*mn
+// (reference decode src/core/numerics/quant.cpp:388-419, layout quant.hpp:592-595).  A chunk is
+// one 64-weight group g of a block, as in Q4KPairCodec: 32 bytes of qs (sub-block 2g in the low
+// nibbles, 2g+1 in the high nibbles) plus bits 2g and 2g+1 of the block's 32 qh bytes, which all
+// four chunks of a block load.  Four five-bit quants are assembled per register with byte masks
+// and converted with v_cvt_f32_ubyte*; d*sc, dmin*mn and sc*q are exact in fp32, so a one-hot
+// activation returns the reference's dequantized weight bit for bit.
+// ----------------------------------------------------------------------------
+struct Q5KCodec {
+  using Args = Q4KCodec::Args;
+  template <int R>
+  struct X {
+    float lo[R][32];
+    float hi[R][32];
+    float slo[R];
+    float shi[R];
+    uint32_t sh;       // scale words: bit offset of the sub-block pair
+    uint32_t lm, hm;   // scale byte-pair masks, as in Q4KPairCodec
+    uint32_t hs;       // 2g: position of the group's bit pair in a qh byte
+    bool upper;
+  };
+  struct Frag {
+    uint4 h;
+    uint4 qh0, qh1;
+    uint4 q0, q1;
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 64u; }
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 64u; }
+
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    const uint32_t blk = chunk >> 2, g = chunk & 3u;
+    x.sh = (g & 1u) * 16u;
+    x.upper = g >= 2u;
+    x.lm = x.upper ? 0x0F0Fu : 0x3F3Fu;
+    x.hm = x.upper ? 0x3030u : 0u;
+    x.hs = 2u * g;
+    const uint32_t k0 = blk * 256u + g * 64u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float sl = 0.0f, sh = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 32; i += 4) {
+        float4 lo = src(r, k0 + i);
+        float4 hi = src(r, k0 + 32 + i);
+        if (!valid) lo = hi = make_float4(0.f, 0.f, 0.f, 0.f);
+        x.lo[r][i] = lo.x, x.lo[r][i + 1] = lo.y, x.lo[r][i + 2] = lo.z, x.lo[r][i + 3] = lo.w;
+        x.hi[r][i] = hi.x, x.hi[r][i + 1] = hi.y, x.hi[r][i + 2] = hi.z, x.hi[r][i + 3] = hi.w;
+        sl += (lo.x + lo.y) + (lo.z + lo.w);
+        sh += (hi.x + hi.y) + (hi.z + hi.w);
+      }
+      x.slo[r] = sl;
+      x.shi[r] = sh;
+    }
+  }
+
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t hdr = prow * (cpr >> 2) * 176u + (chunk >> 2) * 176u;
+    return Lane{hdr, hdr + 48u + (chunk & 3u) * 32u};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const uint8_t* base = p.w + static_cast<size_t>(row) * ((cpr >> 2) * 176u);
+    f.h = load_u4(base + ln.off0);
+    f.qh0 = load_u4(base + ln.off0 + 16u);
+    f.qh1 = load_u4(base + ln.off0 + 32u);
+    f.q0 = load_u4(base + ln.off1);
+    f.q1 = load_u4(base + ln.off1 + 16u);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const uint32_t s0 = f.h.y, s1 = f.h.z, s2 = f.h.w;
+    const uint32_t ls = x.upper ? s2 : s0;
+    const uint32_t lmn = x.upper ? (s2 >> 4) : s1;
+    const uint32_t sc2 = ((ls >> x.sh) & x.lm) | ((s0 >> (x.sh + 2u)) & x.hm);
+    const uint32_t mn2 = ((lmn >> x.sh) & x.lm) | ((s1 >> (x.sh + 2u)) & x.hm);
+    const float sca = static_cast<float>(sc2 & 0xFFu), scb = static_cast<float>((sc2 >> 8) & 0xFFu);
+    const float mna = static_cast<float>(mn2 & 0xFFu), mnb = static_cast<float>((mn2 >> 8) & 0xFFu);
+    const float d = half_bits_to_float(f.h.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(f.h.x >> 16);
+    const uint32_t qw[8] = {f.q0.x, f.q0.y, f.q0.z, f.q0.w, f.q1.x, f.q1.y, f.q1.z, f.q1.w};
+    const uint32_t hw[8] = {f.qh0.x, f.qh0.y, f.qh0.z, f.qh0.w, f.qh1.x, f.qh1.y, f.qh1.z, f.qh1.w};
+    float al[R], ah[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) al[r] = ah[r] = 0.0f;
+#pragma unroll
+    for (int wi = 0; wi < 8; ++wi) {
+      const uint32_t w = qw[wi], t = hw[wi] >> x.hs;
+      const uint32_t lo4 = (w & 0x0F0F0F0Fu) | ((t & 0x01010101u) << 4);
+      const uint32_t hi4 = ((w >> 4) & 0x0F0F0F0Fu) | ((t << 3) & 0x10101010u);
+      const float l0 = static_cast<float>(lo4 & 0xFFu), l1 = static_cast<float>((lo4 >> 8) & 0xFFu);
+      const float l2 = static_cast<float>((lo4 >> 16) & 0xFFu), l3 = static_cast<float>(lo4 >> 24);
+      const float h0 = static_cast<float>(hi4 & 0xFFu), h1 = static_cast<float>((hi4 >> 8) & 0xFFu);
+      const float h2 = static_cast<float>((hi4 >> 16) & 0xFFu), h3 = static_cast<float>(hi4 >> 24);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        al[r] = fmaf(x.lo[r][4 * wi + 0], l0, al[r]);
+        ah[r] = fmaf(x.hi[r][4 * wi + 0], h0, ah[r]);
+        al[r] = fmaf(x.lo[r][4 * wi + 1], l1, al[r]);
+        ah[r] = fmaf(x.hi[r][4 * wi + 1], h1, ah[r]);
+        al[r] = fmaf(x.lo[r][4 * wi + 2], l2, al[r]);
+        ah[r] = fmaf(x.hi[r][4 * wi + 2], h2, ah[r]);
+        al[r] = fmaf(x.lo[r][4 * wi + 3], l3, al[r]);
+        ah[r] = fmaf(x.hi[r][4 * wi + 3], h3, ah[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float t1 = fmaf(scb, ah[r], sca * al[r]);
+      const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
+      out[r] = fmaf(d, t1, -(dmin * t2));
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+
+// ----------------------------------------------------------------------------
 // Q6_K: 210-byte super-block = ql[128] low nibbles, qh[64] two high bits each, 16 int8
 // scales, fp16 d; value = d * s * (q - 32) (reference decode src/core/numerics/quant.cpp:421-450,
 // layout quant.hpp:597-600, device twin src/backends/rocm/rocm_kernels_codec.hpp:132-176).
@@ -1186,6 +1314,19 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     }
     if (e != hipSuccess) return e;
     r0 += took;
+  }
+  return hipSuccess;
+}
+
+// Q5_K: one row per weight pass (a lane keeps 64 activations and five 16-byte loads per stage).
+bool gemv_q5k_supported(uint64_t k) { return k % 256 == 0 && k / 64 <= 768; }
+
+hipError_t launch_q5k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                           uint32_t k, hipStream_t stream) {
+  for (uint32_t r0 = 0; r0 < m; ++r0) {
+    Q5KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
+    const hipError_t e = launch_gemv_r<Q5KCodec, 1, 768, 3, 9>(args, c + static_cast<size_t>(r0) * n, n, k, n, stream);
+    if (e != hipSuccess) return e;
   }
   return hipSuccess;
 }

@@ -204,6 +204,54 @@ qmm_status run_dequant_q4k(const LaunchCtx& c) {
   return map_hip(qmm::launch_dequant_q4k(c.ptr<const uint8_t>(0), c.ptr<float>(1), nb, c.stream));
 }
 
+// ---- Q5_K ---------------------------------------------------------------------
+// "gemm_q5k", "gemm_q5k_batched", "gemm_q5k_vec", "gemm_q5k_rows{R}": as the Q6_K ids below, with
+// 176-byte blocks (include/tessera/backend.hpp:202-206,524-536; rocm_backend.cpp:95-101).
+qmm_status q5k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, uint64_t split, const char* who) {
+  if (!dims_ok(m, n, k) || k % 256 != 0) return bad(std::string(who) + ": m, n, k must be non-zero and k a multiple of 256");
+  if (split == 0 || split > 64 || (k / 256) % split != 0) return bad(std::string(who) + ": split must divide k/256");
+  const u128 region = static_cast<u128>(m) * n * 4;
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, static_cast<u128>(n) * (k / 256) * 176) ||
+      !c.fits(2, region * split)) {
+    return bad(std::string(who) + ": a buffer is smaller than m, n, k require");
+  }
+  if (!qmm::gemv_q5k_supported(k)) {
+    g_last_error = "Q5_K: k above 49152 is not implemented";
+    return QMM_UNSUPPORTED_FEATURE;
+  }
+  float* out = c.ptr<float>(2);
+  qmm_status st = map_hip(qmm::launch_q5k_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out,
+                                               static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                               static_cast<uint32_t>(k), c.stream));
+  if (st == QMM_OK && split > 1) st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
+  return st;
+}
+qmm_status run_gemm_q5k(const LaunchCtx& c) {
+  if (!counts(c, 3, 3)) return bad("gemm_q5k: expects 3 buffers and 3 scalars");
+  return q5k_matmul(c, c.sc[0], c.sc[1], c.sc[2], 1, "gemm_q5k");
+}
+qmm_status run_gemm_q5k_split(const LaunchCtx& c, uint64_t rows_required) {
+  if (!counts(c, 3, 4)) return bad("gemm_q5k_vec/rows: expects 3 buffers and 4 scalars");
+  if (rows_required != 0 && c.sc[0] != rows_required) return bad("gemm_q5k_rowsR: m must equal R");
+  return q5k_matmul(c, c.sc[0], c.sc[1], c.sc[2], c.sc[3], "gemm_q5k_vec/rows");
+}
+qmm_status run_gemm_q5k_vec(const LaunchCtx& c) { return run_gemm_q5k_split(c, 0); }
+qmm_status run_gemm_q5k_rows2(const LaunchCtx& c) { return run_gemm_q5k_split(c, 2); }
+qmm_status run_gemm_q5k_rows3(const LaunchCtx& c) { return run_gemm_q5k_split(c, 3); }
+qmm_status run_gemm_q5k_rows4(const LaunchCtx& c) { return run_gemm_q5k_split(c, 4); }
+qmm_status run_gemm_q5k_rows5(const LaunchCtx& c) { return run_gemm_q5k_split(c, 5); }
+
+// "dequant_q5k" (not a reference id): buffers W, Out (fp32); scalar nblocks.
+qmm_status run_dequant_q5k(const LaunchCtx& c) {
+  if (!counts(c, 2, 1)) return bad("dequant_q5k: expects 2 buffers and 1 scalar");
+  const uint64_t nb = c.sc[0];
+  if (nb == 0 || nb > (1ull << 32)) return bad("dequant_q5k: bad block count");
+  if (!c.fits(0, static_cast<u128>(nb) * 176) || !c.fits(1, static_cast<u128>(nb) * 1024)) {
+    return bad("dequant_q5k: a buffer is smaller than nblocks requires");
+  }
+  return map_hip(qmm::launch_dequant_q5k(c.ptr<const uint8_t>(0), c.ptr<float>(1), nb, c.stream));
+}
+
 // ---- Q6_K ---------------------------------------------------------------------
 // "gemm_q6k", "gemm_q6k_batched": buffers A, W, C; scalars m, n, k, k a multiple of 256
 // (include/tessera/backend.hpp:202-206,524-536).  "gemm_q6k_vec", "gemm_q6k_rows{R}": the same
@@ -589,6 +637,14 @@ const Entry kTable[] = {
     {"moe_gate", run_moe_gate},
     {"top_k_rows", run_top_k_rows},
     {"dequant_q4k", run_dequant_q4k},
+    {"gemm_q5k", run_gemm_q5k},
+    {"gemm_q5k_batched", run_gemm_q5k},
+    {"gemm_q5k_vec", run_gemm_q5k_vec},
+    {"gemm_q5k_rows2", run_gemm_q5k_rows2},
+    {"gemm_q5k_rows3", run_gemm_q5k_rows3},
+    {"gemm_q5k_rows4", run_gemm_q5k_rows4},
+    {"gemm_q5k_rows5", run_gemm_q5k_rows5},
+    {"dequant_q5k", run_dequant_q5k},
     {"gemm_q6k", run_gemm_q6k},
     {"gemm_q6k_batched", run_gemm_q6k},
     {"gemm_q6k_vec", run_gemm_q6k_vec},
@@ -620,7 +676,7 @@ qmm_status qmm_init(int device) {
     g_last_error = std::string("qmm_init: device is ") + prop.gcnArchName + ", this library holds gfx950 code only";
     return QMM_UNSUPPORTED_FEATURE;
   }
-  g_device_name = prop.name;
+  g_device_name = prop.name[0] != '\0' ? prop.name : prop.gcnArchName;   // some hosts report no marketing name
   qmm::set_num_cus(prop.multiProcessorCount);
   g_device = device;
   if (g_decode_scratch == nullptr) {

@@ -15,12 +15,16 @@ int num_cus();
 
 // ---- decode GEMV family (gemv.hip) -----------------------------------------
 bool gemv_q4k_supported(uint64_t k);
+bool gemv_q5k_supported(uint64_t k);
 bool gemv_q6k_supported(uint64_t k);
 bool gemv_mxfp4_supported(uint64_t k);
 bool gemv_fp8_supported(uint64_t k);
 
 // C (m x n fp32) = A (m x k fp32) . deq(W)^T, W = n rows of k/256 Q4_K blocks.
 hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                           uint32_t k, hipStream_t stream);
+// W = n rows of k/256 Q5_K blocks (176 bytes each).
+hipError_t launch_q5k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                            uint32_t k, hipStream_t stream);
 // W = n rows of k/256 Q6_K blocks (210 bytes each).
 hipError_t launch_q6k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
@@ -89,6 +93,7 @@ hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float
 hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uint64_t k,
                                 hipStream_t stream);
 hipError_t launch_dequant_q4k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream);
+hipError_t launch_dequant_q5k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream);
 hipError_t launch_dequant_q6k(const uint8_t* w, float* out, uint64_t nblocks, hipStream_t stream);
 hipError_t launch_dequant_mxfp4(const uint8_t* w, float* out, uint64_t n, uint64_t k,
                                 hipStream_t stream);

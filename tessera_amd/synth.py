@@ -50,7 +50,24 @@ def q4k_weights(g: np.random.Generator, n: int, k: int) -> np.ndarray:
     return blocks.reshape(-1)
 
 
+Q5K_BYTES = 176
 Q6K_BYTES = 210
+
+
+def q5k_weights(g: np.random.Generator, n: int, k: int) -> np.ndarray:
+    """n x k Q5_K matrix (176-byte super-blocks: fp16 d, dmin, 12 packed scale/min bytes, 32 bytes
+    of high bits, 128 bytes of low nibbles): d, dmin ~ U[5e-4, 1e-2] (rounded to fp16),
+    scales/mins ~ U{0..63}, quants uniform.  Flat uint8 array."""
+    assert k % Q4K_ELEMS == 0
+    nb = n * (k // Q4K_ELEMS)
+    blocks = np.empty((nb, Q5K_BYTES), dtype=np.uint8)
+    d = g.uniform(5e-4, 1e-2, size=(nb, 2)).astype(np.float32).astype(np.float16)
+    blocks[:, 0:4] = d.view(np.uint8).reshape(nb, 4)
+    sc = g.integers(0, 64, size=(nb, 8), dtype=np.uint8)
+    mn = g.integers(0, 64, size=(nb, 8), dtype=np.uint8)
+    blocks[:, 4:16] = pack_q4k_scales(sc, mn)
+    blocks[:, 16:] = g.integers(0, 256, size=(nb, 160), dtype=np.uint8)
+    return blocks.reshape(-1)
 
 
 def q6k_weights(g: np.random.Generator, n: int, k: int) -> np.ndarray:

@@ -21,7 +21,8 @@ REFERENCE_IDS = [
     "gemm_mxfp4_wmma_reduce", "quantize_fp8", "quantize_fp8_pack", "quantize_fp8_pack_rows",
     "gemm_fp8", "moe_scale_add", "moe_experts_gate_up_q4k", "moe_experts_down_q4k", "moe_gate",
     "top_k_rows", "gemm_q6k", "gemm_q6k_vec", "gemm_q6k_rows2", "gemm_q6k_rows3", "gemm_q6k_rows4",
-    "gemm_q6k_rows5", "gemm_q6k_batched",
+    "gemm_q6k_rows5", "gemm_q6k_batched", "gemm_q5k", "gemm_q5k_vec", "gemm_q5k_rows2", "gemm_q5k_rows3",
+    "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched",
 ]
 
 
@@ -50,7 +51,7 @@ def test_kernel_table_and_unknown_ids_without_a_device():
     for kid in REFERENCE_IDS:
         assert kid in names
         assert b.LoadKernel(kid).Id() == kid
-    for kid in ("gemm_q5k", "attention", "", "gemm_q4k "):
+    for kid in ("gemm_q3k", "attention", "", "gemm_q4k "):
         with pytest.raises(StatusError) as e:
             b.LoadKernel(kid)
         assert e.value.code == StatusCode.UnsupportedFeature   # callers fall through on this code

@@ -678,6 +678,50 @@ struct Q6KCodec {
   }
 };
 
+// Down projection of the selected experts with Q6_K expert tensors (reference kernel
+// src/backends/rocm/rocm_kernels_moe.cpp:81-110, loaded next to the Q4_K one by
+// src/models/qwen3_5/moe.cpp:107-115): a row is one dot product over top_k * inter, slot s
+// reading expert ids[s], with the routing weight folded into the activations.
+struct Q6KExpertDownCodec : Q6KCodec {
+  using Args = Q4KExpertDownCodec::Args;
+  static __device__ __forceinline__ void batch(Args& p, uint32_t y) { Q4KExpertDownCodec::batch(p, y); }
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    Q6KCodec::load_x<R>(Q6KCodec::Args{p.a, p.w, p.k}, chunk, valid, x, src);
+    const float wt = p.wts[chunk / (p.inter / 64u)];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x.v[r][j][i] *= wt;
+        x.s32[r][j] *= wt;
+      }
+    }
+  }
+  // Offsets are relative to row 0 of expert 0; they stay below 4 GB (checked by the caller).
+  static __device__ __forceinline__ Lane make_lane(const Args& p, uint32_t, uint32_t chunk, uint32_t) {
+    const uint32_t per_slot = p.inter / 64u, slot = chunk / per_slot, cin = chunk - slot * per_slot;
+    const uint32_t e = p.ids[slot] < p.n_experts ? p.ids[slot] : p.n_experts - 1u;
+    const uint32_t blk = static_cast<uint32_t>(e * p.stride) + (cin >> 2) * 210u;
+    return Lane{blk, ((cin >> 1) & 1u) * 64u + (cin & 1u) * 16u};
+  }
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row, uint32_t, Frag& f) {
+    const uint8_t* blk = p.w + static_cast<size_t>(row) * ((p.inter / 256u) * 210u) + ln.off0;
+    const uint32_t n = ln.off1 >> 6, is16 = ln.off1 & 16u;
+    f.ql0 = *reinterpret_cast<const uint4_u*>(blk + ln.off1);
+    f.ql1 = *reinterpret_cast<const uint4_u*>(blk + ln.off1 + 32u);
+    f.qh = *reinterpret_cast<const uint4_u*>(blk + 128u + n * 32u + is16);
+    f.sc = *reinterpret_cast<const uint2_u*>(blk + 192u + n * 8u);
+    f.d = *reinterpret_cast<const uint16_t*>(blk + 208u);
+  }
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args& p, uint32_t row, int, float v) {
+    return p.prev != nullptr ? p.prev[row] + v : v;
+  }
+};
+
 // ----------------------------------------------------------------------------
 // MXFP4 with fp32 activations: packed buffer = n*k/2 nibble bytes (low nibble =
 // even element) then n*k/32 E8M0 bytes (include/tessera/backend.hpp:195-201;
@@ -1446,6 +1490,18 @@ hipError_t launch_moe_down_q4k(const float* phi, const uint8_t* down, const uint
   Q4KExpertDownCodec::Args a{phi, down, k, ids, down_stride, inter, top_k, hidden, n_experts, wts,
                              accumulate ? out : nullptr};
   hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertDownCodec>), dim3((hidden + 3u) / 4u, rows), dim3(256), 0,
+                     stream, a, out, hidden, cpr, hidden);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_down_q6k(const float* phi, const uint8_t* down, const uint32_t* ids,
+                               const float* wts, float* out, uint32_t hidden, uint32_t inter,
+                               uint32_t top_k, uint64_t down_stride, bool accumulate, uint32_t n_experts,
+                               uint32_t rows, hipStream_t stream) {
+  const uint32_t k = top_k * inter, cpr = Q6KCodec::chunks_per_row(k);
+  Q6KExpertDownCodec::Args a{phi, down, k, ids, down_stride, inter, top_k, hidden, n_experts, wts,
+                             accumulate ? out : nullptr};
+  hipLaunchKernelGGL((gemv_generic_kernel<Q6KExpertDownCodec>), dim3((hidden + 3u) / 4u, rows), dim3(256), 0,
                      stream, a, out, hidden, cpr, hidden);
   return hipGetLastError();
 }

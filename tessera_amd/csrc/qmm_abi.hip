@@ -501,33 +501,40 @@ qmm_status run_moe_gate_up_rows(const LaunchCtx& c) { return run_moe_gate_up_n(c
 // "moe_experts_down_q4k": buffers phi, down, ids, wts, out; scalars hidden, inter, top_k,
 // down_stride, accumulate (src/backends/rocm/rocm_kernels_moe.cpp:49-79;
 // src/models/qwen3_5/moe.cpp:413-423).  "..._rows" adds a trailing `rows` as above.
-qmm_status run_moe_down_n(const LaunchCtx& c, bool batched) {
-  if (!counts(c, 5, batched ? 6 : 5)) return bad("moe_experts_down_q4k: expects 5 buffers and 5 (6) scalars");
+qmm_status run_moe_down_n(const LaunchCtx& c, bool batched, bool q6k) {
+  const char* who = q6k ? "moe_experts_down_q6k" : "moe_experts_down_q4k";
+  if (!counts(c, 5, batched ? 6 : 5)) return bad(std::string(who) + ": expects 5 buffers and 5 (6) scalars");
   const uint64_t hidden = c.sc[0], inter = c.sc[1], top_k = c.sc[2], ds = c.sc[3], acc = c.sc[4];
   const uint64_t rows = batched ? c.sc[5] : 1;
   if (hidden == 0 || inter == 0 || inter % 256 != 0 || hidden > (1u << 24) || inter > (1u << 20) ||
       top_k == 0 || top_k > 64 || top_k * inter / 32 > 32768 || rows == 0 || rows > 65535) {
-    return bad("moe_experts_down_q4k: bad hidden, inter, top_k or rows");
+    return bad(std::string(who) + ": bad hidden, inter, top_k or rows");
   }
-  if (ds < q4k_bytes(hidden, inter)) return bad("moe_experts_down_q4k: expert stride smaller than one expert");
-  if (!c.fits(0, static_cast<u128>(rows) * top_k * inter * 4) || !c.fits(1, q4k_bytes(hidden, inter)) ||
+  const u128 expert_bytes = q6k ? q6k_bytes(hidden, inter) : q4k_bytes(hidden, inter);
+  if (ds < expert_bytes) return bad(std::string(who) + ": expert stride smaller than one expert");
+  if (!c.fits(0, static_cast<u128>(rows) * top_k * inter * 4) || !c.fits(1, expert_bytes) ||
       !c.fits(2, static_cast<u128>(rows) * top_k * 4) || !c.fits(3, static_cast<u128>(rows) * top_k * 4) ||
       !c.fits(4, static_cast<u128>(rows) * hidden * 4)) {
-    return bad("moe_experts_down_q4k: a buffer is smaller than the shape requires");
+    return bad(std::string(who) + ": a buffer is smaller than the shape requires");
   }
   if (c.bytes != nullptr && c.bytes[1] >= (1ull << 32)) {
-    g_last_error = "moe_experts_down_q4k: expert tensors of 4 GB and more are not implemented";
+    g_last_error = std::string(who) + ": expert tensors of 4 GB and more are not implemented";
     return QMM_UNSUPPORTED_FEATURE;
   }
   uint64_t experts = 0xFFFFFFFFull;
-  if (c.bytes != nullptr) experts = (c.bytes[1] - static_cast<uint64_t>(q4k_bytes(hidden, inter))) / ds + 1;
-  return map_hip(qmm::launch_moe_down_q4k(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint32_t>(2),
-                                          c.ptr<const float>(3), c.ptr<float>(4), static_cast<uint32_t>(hidden),
-                                          static_cast<uint32_t>(inter), static_cast<uint32_t>(top_k), ds, acc != 0,
-                                          static_cast<uint32_t>(experts), static_cast<uint32_t>(rows), c.stream));
+  if (c.bytes != nullptr) experts = (c.bytes[1] - static_cast<uint64_t>(expert_bytes)) / ds + 1;
+  const auto launch = q6k ? qmm::launch_moe_down_q6k : qmm::launch_moe_down_q4k;
+  return map_hip(launch(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint32_t>(2),
+                        c.ptr<const float>(3), c.ptr<float>(4), static_cast<uint32_t>(hidden),
+                        static_cast<uint32_t>(inter), static_cast<uint32_t>(top_k), ds, acc != 0,
+                        static_cast<uint32_t>(experts), static_cast<uint32_t>(rows), c.stream));
 }
-qmm_status run_moe_down(const LaunchCtx& c) { return run_moe_down_n(c, false); }
-qmm_status run_moe_down_rows(const LaunchCtx& c) { return run_moe_down_n(c, true); }
+qmm_status run_moe_down(const LaunchCtx& c) { return run_moe_down_n(c, false, false); }
+qmm_status run_moe_down_rows(const LaunchCtx& c) { return run_moe_down_n(c, true, false); }
+// "moe_experts_down_q6k": the same contract with Q6_K expert tensors
+// (src/backends/rocm/rocm_kernels_moe.cpp:81-110).
+qmm_status run_moe_down_q6k(const LaunchCtx& c) { return run_moe_down_n(c, false, true); }
+qmm_status run_moe_down_q6k_rows(const LaunchCtx& c) { return run_moe_down_n(c, true, true); }
 
 // "moe_gate": buffers vals (top_k), x, w (hidden), wts (top_k), sig (1); scalars top_k, hidden
 // (src/backends/rocm/rocm_kernels_basic.cpp:1896-1929).
@@ -633,6 +640,8 @@ const Entry kTable[] = {
     {"moe_experts_down_q4k", run_moe_down},
     {"moe_experts_gate_up_q4k_rows", run_moe_gate_up_rows},
     {"moe_experts_down_q4k_rows", run_moe_down_rows},
+    {"moe_experts_down_q6k", run_moe_down_q6k},
+    {"moe_experts_down_q6k_rows", run_moe_down_q6k_rows},
     {"moe_experts_ffn_q4k_rows", run_moe_ffn_rows},
     {"moe_gate", run_moe_gate},
     {"top_k_rows", run_top_k_rows},

@@ -58,6 +58,12 @@ hipError_t launch_moe_down_q4k(const float* phi, const uint8_t* down, const uint
                                uint32_t top_k, uint64_t down_stride, bool accumulate, uint32_t n_experts,
                                uint32_t rows, hipStream_t stream);
 
+// The same with Q6_K expert tensors.
+hipError_t launch_moe_down_q6k(const float* phi, const uint8_t* down, const uint32_t* ids,
+                               const float* wts, float* out, uint32_t hidden, uint32_t inter,
+                               uint32_t top_k, uint64_t down_stride, bool accumulate, uint32_t n_experts,
+                               uint32_t rows, hipStream_t stream);
+
 // ---- MFMA GEMMs (gemm_mxfp4.hip, gemm_q4k.hip) --------------------------------------
 bool gemm_mxfp4_a8_supported(uint64_t k);
 // W4A8 on the scaled MFMA: A = m x k E4M3 codes + per-row scales, W packed MXFP4.

@@ -177,3 +177,39 @@ def test_grouped_ffn_matches_oracle(backend, rows, experts, hidden, inter, top_k
     # the sorted position of a pair may differ from run to run (atomics), its result may not
     again = forward_grouped(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
     assert np.array_equal(again, got)
+
+
+@pytest.mark.parametrize("experts,hidden,inter,top_k,rows", [(16, 512, 256, 4, 1), (8, 2048, 512, 8, 1),
+                                                              (5, 260, 768, 2, 3), (256, 2048, 512, 8, 2)])
+def test_down_q6k_matches_oracle(backend, experts, hidden, inter, top_k, rows):
+    """moe_experts_down_q6k (the reference loads it next to the Q4_K one,
+    src/models/qwen3_5/moe.cpp:107-115): out[t] (+)= sum_slot wts[t][slot] * D_{ids[t][slot]} phi[t][slot],
+    expert tensors Q6_K [hidden, inter]."""
+    g = synth.rng(9000 + experts + hidden + inter + rows)
+    down = np.concatenate([synth.q6k_weights(g, hidden, inter) for _ in range(experts)])
+    ds = down.size // experts
+    phi = synth.activations_f32(g, rows * top_k, inter).reshape(rows, top_k, inter)
+    ids = np.stack([g.permutation(experts)[:top_k] for _ in range(rows)]).astype(np.uint32)
+    wts = g.uniform(0.05, 1.0, size=(rows, top_k)).astype(np.float32)
+    want = np.zeros((rows, hidden), np.float64)
+    for t in range(rows):
+        for s in range(top_k):
+            e = int(ids[t, s])
+            y = oracle.gemm_q6k(phi[t, s:s + 1], down[e * ds:(e + 1) * ds], 1, hidden, inter)[0]
+            want[t] += np.float64(wts[t, s]) * y.astype(np.float64)
+    d_phi, d_down = backend.Upload(phi), backend.Upload(down)
+    d_ids, d_wts = backend.Upload(ids), backend.Upload(wts)
+    prev = synth.activations_f32(g, rows, hidden)
+    for accumulate in (0, 1):
+        d_out = backend.Upload(prev.copy())
+        if rows == 1:
+            run(backend, "moe_experts_down_q6k", [d_phi, d_down, d_ids, d_wts, d_out],
+                [hidden, inter, top_k, ds, accumulate], grid=((hidden + 7) // 8, 1, 1))
+        else:
+            run(backend, "moe_experts_down_q6k_rows", [d_phi, d_down, d_ids, d_wts, d_out],
+                [hidden, inter, top_k, ds, accumulate, rows], grid=((hidden + 7) // 8, rows, 1))
+        backend.Synchronize()
+        got = backend.CopyD2H(d_out, dtype=np.float32).reshape(rows, hidden)
+        ref = want + (prev.astype(np.float64) if accumulate else 0.0)
+        base = want      # the bound is relative to the routed sum, not to what it is added to
+        assert rel_err(got - (prev if accumulate else 0), base) <= TOL, (accumulate, rel_err(got, ref))

@@ -198,6 +198,16 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
                                          scalars=[m, nn, k, 1, 0]))], 10, graph=False)
         prefill[f"mxfp4_{label}"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * nn * k / us / 1e6, 1),
                                      "frac_fp8_peak": round(2 * m * nn * k / us / 1e6 / 5000.0, 4)}
+    # Q6_K and Q5_K prefill: weights decoded to fp16 per call, then the dense fp16 MFMA GEMM
+    for fmt, gen in (("q6k", synth.q6k_weights), ("q5k", synth.q5k_weights)):
+        wf = to_dev(gen(g, n, k))
+        kf = backend.LoadKernel(f"gemm_{fmt}_wmma")
+        y = torch.empty(m * n, dtype=torch.float32, device=dev)
+        us = timed_us([(kf, KernelLaunch(grid_x=n // 64, grid_y=m // 128, buffers=[wrap(a), wrap(wf), wrap(y)],
+                                         scalars=[m, n, k]))], 10, graph=False)
+        prefill[f"{fmt}_n17408"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * n * k / us / 1e6, 1),
+                                    "frac_fp16_peak": round(2 * m * n * k / us / 1e6 / 2500.0, 4)}
+        del wf
     out["prefill_gemm_m2048_k5120"] = prefill
     del a, w_q, w_mx, a8, y
 

@@ -321,6 +321,196 @@ hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* wor
   return hipGetLastError();
 }
 
+// ---- Q5_K / Q6_K prefill: weights decoded once to fp16, then a dense fp16 MFMA GEMM ----------
+// Their blocks (176 and 210 bytes, the latter only 2-byte aligned) do not suit the in-register
+// decode above, and they are the minority of a K-quant file's tensors, so the weights take a
+// pre-pass: every value is formed exactly in fp32 as the reference decodes it and rounded once
+// to fp16 (the same operand precision as the Q4_K path), in the 0,2,1,3,4,6,5,7 order that the
+// activation copy uses.  The GEMM then streams both operands as 32-K slices through four-stage
+// swizzled LDS rings.
+namespace {
+
+__device__ __forceinline__ uint32_t perm8(uint32_t e) {   // position of element e inside its group of 8
+  const uint32_t i = e & 7u;
+  return (e & ~7u) | ((i == 1u || i == 5u) ? i + 1u : (i == 2u || i == 6u) ? i - 1u : i);
+}
+
+// One thread per (block, half n, lane l): the four values sharing ql[n*64+l], ql[n*64+32+l],
+// qh[n*32+l] (src/core/numerics/quant.cpp:421-450).
+__global__ __launch_bounds__(256) void q6k_to_f16_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ out,
+                                                         uint64_t nitems) {
+  const uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= nitems) return;
+  const uint64_t blk = t >> 6;
+  const uint32_t n = static_cast<uint32_t>(t >> 5) & 1u, l = static_cast<uint32_t>(t) & 31u, is = l >> 4;
+  const uint8_t* base = w + blk * 210u;
+  const uint32_t a = base[n * 64 + l], b = base[n * 64 + 32 + l], h = base[128 + n * 32 + l];
+  const float d = half_bits_to_float(static_cast<uint32_t>(base[208]) | (static_cast<uint32_t>(base[209]) << 8));
+  const int q[4] = {static_cast<int>((a & 15u) | ((h & 3u) << 4)), static_cast<int>((b & 15u) | (((h >> 2) & 3u) << 4)),
+                    static_cast<int>((a >> 4) | (((h >> 4) & 3u) << 4)), static_cast<int>((b >> 4) | ((h >> 6) << 4))};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float s = static_cast<float>(static_cast<int8_t>(base[192 + n * 8 + is + 2 * j]));
+    out[blk * 256 + perm8(n * 128 + 32 * j + l)] = static_cast<_Float16>(d * s * static_cast<float>(q[j] - 32));
+  }
+}
+
+// One thread per quant byte (block, group g, lane l) (src/core/numerics/quant.cpp:388-419).
+__global__ __launch_bounds__(256) void q5k_to_f16_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ out,
+                                                         uint64_t nitems) {
+  const uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= nitems) return;
+  const uint64_t blk = t >> 7;
+  const uint32_t g = static_cast<uint32_t>(t >> 5) & 3u, l = static_cast<uint32_t>(t) & 31u;
+  const uint8_t* base = w + blk * 176u;
+  const uint8_t* p = base + 4;
+  auto scale_min = [&](uint32_t sb, uint32_t& sc, uint32_t& mn) {
+    if (sb < 4) {
+      sc = p[sb] & 63u;
+      mn = p[sb + 4] & 63u;
+    } else {
+      sc = (p[sb + 4] & 15u) | ((p[sb - 4] >> 6) << 4);
+      mn = (p[sb + 4] >> 4) | ((p[sb] >> 6) << 4);
+    }
+  };
+  uint32_t sca, mna, scb, mnb;
+  scale_min(2 * g, sca, mna);
+  scale_min(2 * g + 1, scb, mnb);
+  const float d = half_bits_to_float(static_cast<uint32_t>(base[0]) | (static_cast<uint32_t>(base[1]) << 8));
+  const float dmin = half_bits_to_float(static_cast<uint32_t>(base[2]) | (static_cast<uint32_t>(base[3]) << 8));
+  const uint32_t low = base[48 + g * 32 + l], high = base[16 + l];
+  const float q0 = static_cast<float>((low & 15u) + (((high >> (2 * g)) & 1u) << 4));
+  const float q1 = static_cast<float>((low >> 4) + (((high >> (2 * g + 1)) & 1u) << 4));
+  out[blk * 256 + perm8(g * 64 + l)] = static_cast<_Float16>(d * static_cast<float>(sca) * q0 - dmin * static_cast<float>(mna));
+  out[blk * 256 + perm8(g * 64 + 32 + l)] = static_cast<_Float16>(d * static_cast<float>(scb) * q1 - dmin * static_cast<float>(mnb));
+}
+
+// C tile = A16 (rows scaled by a_scale) . W16^T, both operands fp16 row-major with row length k.
+template <int BM, int BN>
+__global__ __launch_bounds__(BN * 2) void f16w_gemm_kernel(
+    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const _Float16* __restrict__ w16,
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k) {
+  constexpr int kWaves = BN / 32, kTI = BM / 32;
+  constexpr int kABlk = BM / 16 / kWaves, kWBlk = BN / 16 / kWaves;   // 1 KB blocks per wavefront and slice
+  constexpr int kDma = kABlk + kWBlk;
+  constexpr uint32_t kAStage = BM * 64, kWStage = BN * 64, kStage = kAStage + kWStage;
+  static_assert(BM % (16 * kWaves) == 0 && BN % (16 * kWaves) == 0, "tile shape");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[4 * kStage];
+
+  const uint32_t tiles_n = (n + BN - 1) / BN;
+  const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t l32 = lane & 31u, kg = lane >> 5;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) uint8_t*)lds));
+  const uint8_t* a_tile = reinterpret_cast<const uint8_t*>(a16) + static_cast<size_t>(m0) * k * 2;
+  const uint8_t* w_tile = reinterpret_cast<const uint8_t*>(w16) + static_cast<size_t>(n0) * k * 2;
+
+  // Block L of a slice = rows 16L..16L+15, four 16-byte chunks a row: lane p fetches row
+  // 16L + p/4, chunk (p%4) ^ ((row>>2)&3).  Rows past the matrix edge are clamped (never stored).
+  uint32_t a_src[kABlk], w_src[kWBlk];
+#pragma unroll
+  for (int i = 0; i < kABlk; ++i) {
+    const uint32_t row = 16u * (wave * kABlk + i) + lane / 4u;
+    a_src[i] = (m0 + row < m ? row : m - 1u - m0) * (k * 2u) + (((lane % 4u) ^ ((row >> 2) & 3u)) * 16u);
+  }
+#pragma unroll
+  for (int i = 0; i < kWBlk; ++i) {
+    const uint32_t row = 16u * (wave * kWBlk + i) + lane / 4u;
+    w_src[i] = (n0 + row < n ? row : n - 1u - n0) * (k * 2u) + (((lane % 4u) ^ ((row >> 2) & 3u)) * 16u);
+  }
+  auto issue = [&](uint32_t stage, uint32_t slice_any) {
+    const uint32_t slice = __builtin_amdgcn_readfirstlane(slice_any);
+#pragma unroll
+    for (int i = 0; i < kABlk; ++i)
+      direct_load16(a_tile + slice * 64u, a_src[i], lds_base + stage * kStage + (wave * kABlk + i) * 1024u);
+#pragma unroll
+    for (int i = 0; i < kWBlk; ++i)
+      direct_load16(w_tile + slice * 64u, w_src[i], lds_base + stage * kStage + kAStage + (wave * kWBlk + i) * 1024u);
+  };
+
+  float16_t acc[kTI];
+#pragma unroll
+  for (int i = 0; i < kTI; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+  uint32_t fr[2];   // fragment offset inside a 32-row group: MFMA step tt takes chunk 2tt + kg
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) fr[tt] = l32 * 64u + (((tt * 2u + kg) ^ ((l32 >> 2) & 3u)) * 16u);
+
+  const uint32_t slices = k / 32;
+  issue(0, 0);
+  issue(1, slices > 1 ? 1 : 0);
+  issue(2, slices > 2 ? 2 : slices - 1);
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * kDma) : "memory");
+  for (uint32_t slice = 0; slice < slices; ++slice) {
+    issue((slice + 3u) & 3u, slice + 3u < slices ? slice + 3u : slices - 1u);
+    const uint8_t* stage = lds + (slice & 3u) * kStage;
+    half8_t b[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) b[tt] = *reinterpret_cast<const half8_t*>(stage + kAStage + wave * 32 * 64 + fr[tt]);
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int i = 0; i < kTI; ++i) {
+        const half8_t af = *reinterpret_cast<const half8_t*>(stage + fr[tt] + i * 32 * 64);
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[tt], acc[i], 0, 0, 0);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * kDma) : "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the workgroup
+
+  const uint32_t col = n0 + wave * 32u + l32;
+#pragma unroll
+  for (int i = 0; i < kTI; ++i) {
+    float4 sc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) sc[q] = *reinterpret_cast<const float4*>(a_scale + m0 + i * 32u + q * 8u + kg * 4u);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const uint32_t row = m0 + i * 32u + (e >> 2) * 8u + kg * 4u + (e & 3u);
+      const float4 s4 = sc[e >> 2];
+      const float rs = (e & 3) == 0 ? s4.x : (e & 3) == 1 ? s4.y : (e & 3) == 2 ? s4.z : s4.w;
+      if (row < m && col < n) c[static_cast<size_t>(row) * n + col] = acc[i][e] * rs;
+    }
+  }
+}
+
+}  // namespace
+
+bool gemm_kquant_f16_supported(uint64_t m, uint64_t n, uint64_t k) {
+  return k % 256 == 0 && k <= (1u << 20) && m * k < (1ull << 31) && n * k < (1ull << 31);
+}
+
+// fp16 copy of A, its row scales (padded by a tile of rows), then the fp16 copy of W.
+size_t gemm_kquant_f16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k) {
+  return static_cast<size_t>(m) * k * 2 + (static_cast<size_t>(m) + 256) * 4 + static_cast<size_t>(n) * k * 2;
+}
+
+// block_bytes selects the format: 176 = Q5_K, 210 = Q6_K.
+hipError_t launch_kquant_f16_gemm(const float* a, const uint8_t* w, uint32_t block_bytes, float* c, void* workspace,
+                                  uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
+  _Float16* a16 = static_cast<_Float16*>(workspace);
+  float* a_scale = reinterpret_cast<float*>(a16 + static_cast<size_t>(m) * k);
+  _Float16* w16 = reinterpret_cast<_Float16*>(a_scale + m + 256);
+  const uint64_t blocks = static_cast<uint64_t>(n) * (k / 256);
+  if (block_bytes == 210) {
+    hipLaunchKernelGGL(q6k_to_f16_kernel, dim3(static_cast<uint32_t>((blocks * 64 + 255) / 256)), dim3(256), 0, stream,
+                       w, w16, blocks * 64);
+  } else if (block_bytes == 176) {
+    hipLaunchKernelGGL(q5k_to_f16_kernel, dim3(static_cast<uint32_t>((blocks * 128 + 255) / 256)), dim3(256), 0, stream,
+                       w, w16, blocks * 128);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  hipLaunchKernelGGL(rows_to_f16_kernel, dim3(m), dim3(256), 0, stream, a, a16, a_scale, k, nullptr, 1u);
+  const uint32_t tiles = ((m + 255u) / 256u) * ((n + 255u) / 256u);
+  hipLaunchKernelGGL((f16w_gemm_kernel<256, 256>), dim3(tiles), dim3(512), 0, stream, a16, a_scale, w16, c, m, n, k);
+  return hipGetLastError();
+}
+
 // ---- routed experts, a whole chunk of tokens grouped by expert -----------------------------
 // (token, slot) pairs are sorted by expert so that each expert's weights are streamed once for
 // all the tokens routed to it, and the three projections run as grouped MFMA GEMMs.

@@ -204,6 +204,21 @@ qmm_status run_dequant_q4k(const LaunchCtx& c) {
   return map_hip(qmm::launch_dequant_q4k(c.ptr<const uint8_t>(0), c.ptr<float>(1), nb, c.stream));
 }
 
+// Q5_K / Q6_K from kQ4KGemmMinRows rows up: weights decoded once to fp16 in the library
+// workspace, then the dense fp16 MFMA GEMM.
+qmm_status kquant_prefill(const LaunchCtx& c, uint32_t block_bytes, uint64_t m, uint64_t n, uint64_t k,
+                          uint64_t split) {
+  void* ws = nullptr;
+  qmm_status st = workspace(qmm::gemm_kquant_f16_workspace_bytes(m, n, k), &ws);
+  if (st != QMM_OK) return st;
+  float* out = c.ptr<float>(2);
+  st = map_hip(qmm::launch_kquant_f16_gemm(c.ptr<const float>(0), c.ptr<const uint8_t>(1), block_bytes, out, ws,
+                                           static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                           static_cast<uint32_t>(k), c.stream));
+  if (st == QMM_OK && split > 1) st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
+  return st;
+}
+
 // ---- Q5_K ---------------------------------------------------------------------
 // "gemm_q5k", "gemm_q5k_batched", "gemm_q5k_vec", "gemm_q5k_rows{R}": as the Q6_K ids below, with
 // 176-byte blocks (include/tessera/backend.hpp:202-206,524-536; rocm_backend.cpp:95-101).
@@ -215,11 +230,14 @@ qmm_status q5k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, ui
       !c.fits(2, region * split)) {
     return bad(std::string(who) + ": a buffer is smaller than m, n, k require");
   }
+  float* out = c.ptr<float>(2);
+  if (m >= kQ4KGemmMinRows && qmm::gemm_kquant_f16_supported(m, n, k)) {
+    return kquant_prefill(c, 176, m, n, k, split);
+  }
   if (!qmm::gemv_q5k_supported(k)) {
     g_last_error = "Q5_K: k above 49152 is not implemented";
     return QMM_UNSUPPORTED_FEATURE;
   }
-  float* out = c.ptr<float>(2);
   qmm_status st = map_hip(qmm::launch_q5k_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out,
                                                static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                                static_cast<uint32_t>(k), c.stream));
@@ -266,11 +284,14 @@ qmm_status q6k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, ui
   if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, q6k_bytes(n, k)) || !c.fits(2, region * split)) {
     return bad(std::string(who) + ": a buffer is smaller than m, n, k require");
   }
+  float* out = c.ptr<float>(2);
+  if (m >= kQ4KGemmMinRows && qmm::gemm_kquant_f16_supported(m, n, k)) {
+    return kquant_prefill(c, 210, m, n, k, split);
+  }
   if (!qmm::gemv_q6k_supported(k)) {
     g_last_error = "Q6_K: k above 49152 is not implemented";
     return QMM_UNSUPPORTED_FEATURE;
   }
-  float* out = c.ptr<float>(2);
   qmm_status st = map_hip(qmm::launch_q6k_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out,
                                                static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                                static_cast<uint32_t>(k), c.stream));
@@ -648,6 +669,7 @@ const Entry kTable[] = {
     {"dequant_q4k", run_dequant_q4k},
     {"gemm_q5k", run_gemm_q5k},
     {"gemm_q5k_batched", run_gemm_q5k},
+    {"gemm_q5k_wmma", run_gemm_q5k},
     {"gemm_q5k_vec", run_gemm_q5k_vec},
     {"gemm_q5k_rows2", run_gemm_q5k_rows2},
     {"gemm_q5k_rows3", run_gemm_q5k_rows3},
@@ -656,6 +678,7 @@ const Entry kTable[] = {
     {"dequant_q5k", run_dequant_q5k},
     {"gemm_q6k", run_gemm_q6k},
     {"gemm_q6k_batched", run_gemm_q6k},
+    {"gemm_q6k_wmma", run_gemm_q6k},
     {"gemm_q6k_vec", run_gemm_q6k_vec},
     {"gemm_q6k_rows2", run_gemm_q6k_rows2},
     {"gemm_q6k_rows3", run_gemm_q6k_rows3},

@@ -76,6 +76,13 @@ size_t gemm_q4k_workspace_bytes(uint64_t m, uint64_t k);
 hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream);
 
+// Q5_K (block_bytes 176) and Q6_K (210) prefill: weights decoded once to fp16 in the workspace,
+// then a dense fp16 MFMA GEMM (gemm_q4k.hip).
+bool gemm_kquant_f16_supported(uint64_t m, uint64_t n, uint64_t k);
+size_t gemm_kquant_f16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k);
+hipError_t launch_kquant_f16_gemm(const float* a, const uint8_t* w, uint32_t block_bytes, float* c, void* workspace,
+                                  uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
+
 // Routed experts for a chunk of tokens, grouped by expert (gemm_q4k.hip): out[t] (+)= sum over
 // the token's top_k experts of wts * down_e(silu(gate_e x) * up_e x), as grouped MFMA GEMMs.
 bool moe_ffn_q4k_supported(uint64_t hidden, uint64_t inter, uint64_t experts);

@@ -22,7 +22,7 @@ REFERENCE_IDS = [
     "gemm_fp8", "moe_scale_add", "moe_experts_gate_up_q4k", "moe_experts_down_q4k", "moe_gate",
     "top_k_rows", "gemm_q6k", "gemm_q6k_vec", "gemm_q6k_rows2", "gemm_q6k_rows3", "gemm_q6k_rows4",
     "gemm_q6k_rows5", "gemm_q6k_batched", "gemm_q5k", "gemm_q5k_vec", "gemm_q5k_rows2", "gemm_q5k_rows3",
-    "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched", "moe_experts_down_q6k",
+    "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched", "moe_experts_down_q6k", "gemm_q5k_wmma", "gemm_q6k_wmma",
 ]
 
 

@@ -101,3 +101,25 @@ def test_full_size_and_linearity(backend):
         assert rel_err(got, ref) <= TOL, (n, k, rel_err(got, ref))
         got2 = gemm(backend, "gemm_q5k_vec", 2 * a, w, 1, n, k, extra=(1,))[0]
         assert np.array_equal(got2, 2 * got)
+# From 24 rows up the weights are decoded once to fp16 and multiplied on the fp16 MFMA: weights
+# carry one rounding of 2^-11, activations a second (per-row scaled), accumulation is fp32.
+RMS_TOL, NORM_TOL = 4e-3, 1e-3
+
+
+@pytest.mark.parametrize("m,n,k", [(24, 300, 512), (64, 512, 1024), (100, 257, 2304), (300, 1000, 5120), (256, 256, 256)])
+def test_prefill_fp16_mfma_matches_oracle(backend, m, n, k):
+    from util import norm_err, rms_err
+    g = synth.rng(5900 + m + n + k)
+    w = synth.q5k_weights(g, n, k)
+    a = synth.activations_bf16(g, m, k)
+    ref = oracle.gemm_q5k(a, w, m, n, k, threads=True)
+    for name in ("gemm_q5k_wmma", "gemm_q5k_batched"):
+        got = gemm(backend, name, a, w, m, n, k)[0]
+        assert rms_err(got, ref) <= RMS_TOL, (name, rms_err(got, ref))
+        assert norm_err(got, ref) <= NORM_TOL, (name, norm_err(got, ref))
+    # one-hot rows return the fp16 rounding of the exact decode
+    hot = synth.one_hot_rows(k, [t % k for t in range(0, 32 * 37, 37)])
+    deq = oracle.dequantize_q5k(w).reshape(n, k)
+    got = gemm(backend, "gemm_q5k_wmma", hot, w, 32, n, k)[0]
+    for r, t in enumerate([t % k for t in range(0, 32 * 37, 37)]):
+        assert same_bits_zero_sign_free(got[r], deq[:, t].astype(np.float16).astype(np.float32)), t

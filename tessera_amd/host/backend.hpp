@@ -65,7 +65,7 @@ class Expected<void> {
 enum class MemoryKind { Device };
 
 // Weight formats of the quantized-matmul path (include/tessera/types.hpp:89-113).
-enum class DType { F32, Q4K, F4E2M1, F8E4M3 };
+enum class DType { F32, Q4K, Q5K, Q6K, F4E2M1, F8E4M3 };
 
 class Backend;
 

@@ -153,15 +153,19 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
     l.scalars = {m, n, k};
     return backend.LaunchKernel(**gemm, l);
   }
-  if (dtype == DType::Q4K) {
+  if (dtype == DType::Q4K || dtype == DType::Q5K || dtype == DType::Q6K) {
+    // The K-quant formats share one table (src/core/decode_internal.hpp:1256-1276,1365-1460):
+    // rows{m} for m in 2..4 (the ids exist up to 5), the tensor-core tile from 64 rows and 32
+    // columns, the batched id from kTiledMinRows, the vec id otherwise.
     if (k % 256 != 0) return unexpected(StatusCode::InvalidArgument);
+    const std::string fmt = dtype == DType::Q4K ? "q4k" : dtype == DType::Q5K ? "q5k" : "q6k";
     if (m >= 2 && m <= 4) {
-      auto rows = CachedKernel(backend, h, "gemm_q4k_rows" + std::to_string(m));
+      auto rows = CachedKernel(backend, h, "gemm_" + fmt + "_rows" + std::to_string(m));
       if (!rows) return unexpected(rows.error());
       return ProjectGemvDevice(backend, h, **rows, a, w, out, m, n, k);
     }
     if (m >= kGemmWmmaMinRows && n >= kGemmWmmaMinCols) {
-      auto wmma = CachedKernel(backend, h, "gemm_q4k_wmma");
+      auto wmma = CachedKernel(backend, h, "gemm_" + fmt + "_wmma");
       if (!wmma) return unexpected(wmma.error());
       KernelLaunch l;
       l.grid_x = static_cast<std::uint32_t>((n + 63) / 64);
@@ -171,7 +175,7 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
       return backend.LaunchKernel(**wmma, l);
     }
     if (m >= kTiledMinRows) {
-      auto tiled = CachedKernel(backend, h, "gemm_q4k_batched");
+      auto tiled = CachedKernel(backend, h, "gemm_" + fmt + "_batched");
       if (!tiled) return unexpected(tiled.error());
       KernelLaunch l;
       l.grid_x = static_cast<std::uint32_t>(((m + 31) / 32) * ((n + 31) / 32));
@@ -179,7 +183,7 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
       l.scalars = {m, n, k};
       return backend.LaunchKernel(**tiled, l);
     }
-    auto vec = CachedKernel(backend, h, "gemm_q4k_vec");
+    auto vec = CachedKernel(backend, h, "gemm_" + fmt + "_vec");
     if (!vec) return unexpected(vec.error());
     return ProjectGemvDevice(backend, h, **vec, a, w, out, m, n, k);
   }

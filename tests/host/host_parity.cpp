@@ -12,6 +12,8 @@
 
 extern "C" {
 int orc_gemm_q4k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k);
+int orc_gemm_q5k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k, int threads);
+int orc_gemm_q6k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k, int threads);
 int orc_gemm_mxfp4_ref(const float* a, const uint8_t* w, const uint8_t* s, float* c, size_t m, size_t n, size_t k);
 int orc_quantize_fp8_ref(float* data, float* scale, size_t rows, size_t cols);
 }
@@ -29,6 +31,21 @@ std::vector<uint8_t> Q4KWeights(size_t n, size_t k) {
     w[blk * 144 + 0] = static_cast<uint8_t>(rng()); w[blk * 144 + 1] = 0x20 + (rng() & 3);
     w[blk * 144 + 2] = static_cast<uint8_t>(rng()); w[blk * 144 + 3] = 0x20 + (rng() & 3);
   }
+  return w;
+}
+std::vector<uint8_t> Q5KWeights(size_t n, size_t k) {
+  std::vector<uint8_t> w(n * (k / 256) * 176);
+  for (auto& b : w) b = static_cast<uint8_t>(rng());
+  for (size_t blk = 0; blk < w.size() / 176; ++blk) {   // fp16 d, dmin around 1e-2
+    w[blk * 176 + 1] = 0x20 + (rng() & 3);
+    w[blk * 176 + 3] = 0x20 + (rng() & 3);
+  }
+  return w;
+}
+std::vector<uint8_t> Q6KWeights(size_t n, size_t k) {
+  std::vector<uint8_t> w(n * (k / 256) * 210);
+  for (auto& b : w) b = static_cast<uint8_t>(rng());
+  for (size_t blk = 0; blk < w.size() / 210; ++blk) w[blk * 210 + 209] = 0x14 + (rng() & 3);   // fp16 d around 1e-3
   return w;
 }
 std::vector<uint8_t> MxFp4Weights(size_t n, size_t k) {
@@ -83,6 +100,12 @@ const Case kCases[] = {
     {"q4k m=7 (gemm_q4k_vec, m rows)", DType::Q4K, 7, 129, 1280, false, 1e-3, 1e-3},
     {"q4k m=16 (gemm_q4k_batched)", DType::Q4K, 16, 256, 1024, false, 1e-3, 1e-3},
     {"q4k prefill m=192 (gemm_q4k_wmma, fp16 MFMA)", DType::Q4K, 192, 320, 1024, false, 1.0, 4e-3},
+    {"q6k decode m=1, reference split-K (gemm_q6k_vec)", DType::Q6K, 1, 640, 5120, true, 1e-3, 1e-3},
+    {"q6k verify m=3 (gemm_q6k_rows3)", DType::Q6K, 3, 333, 2048, true, 1e-3, 1e-3},
+    {"q6k prefill m=192 (gemm_q6k_wmma, fp16 MFMA)", DType::Q6K, 192, 320, 1024, false, 1.0, 4e-3},
+    {"q5k decode m=1 (gemm_q5k_vec)", DType::Q5K, 1, 640, 5120, false, 1e-3, 1e-3},
+    {"q5k m=16 (gemm_q5k_batched)", DType::Q5K, 16, 256, 1024, false, 1e-3, 1e-3},
+    {"q5k prefill m=100 (gemm_q5k_wmma, fp16 MFMA)", DType::Q5K, 100, 257, 2304, false, 1.0, 4e-3},
     {"mxfp4 w4a8 m=1 (quantize_fp8_pack_rows + gemm_mxfp4_wmma)", DType::F4E2M1, 1, 512, 1024, false, 1e-3, 1e-3},
     {"mxfp4 w4a8 m=16 (streaming scaled MFMA)", DType::F4E2M1, 16, 512, 2048, false, 1e-2, 5e-4},
     {"mxfp4 w4a8 m=300 (tiled scaled MFMA)", DType::F4E2M1, 300, 384, 1024, false, 1e-2, 5e-4},
@@ -120,10 +143,17 @@ int main(int argc, char** argv) {
     ProjectState h;
     h.honour_reference_split = c.reference_split;
     const auto a = Activations(c.m, c.k);
-    const auto w = c.dtype == DType::Q4K ? Q4KWeights(c.n, c.k) : MxFp4Weights(c.n, c.k);
+    const auto w = c.dtype == DType::Q4K   ? Q4KWeights(c.n, c.k)
+                   : c.dtype == DType::Q5K ? Q5KWeights(c.n, c.k)
+                   : c.dtype == DType::Q6K ? Q6KWeights(c.n, c.k)
+                                           : MxFp4Weights(c.n, c.k);
     std::vector<float> ref(c.m * c.n), got(c.m * c.n);
     if (c.dtype == DType::Q4K) {
       orc_gemm_q4k_ref(a.data(), w.data(), ref.data(), c.m, c.n, c.k);
+    } else if (c.dtype == DType::Q5K) {
+      orc_gemm_q5k_ref(a.data(), w.data(), ref.data(), c.m, c.n, c.k, 1);
+    } else if (c.dtype == DType::Q6K) {
+      orc_gemm_q6k_ref(a.data(), w.data(), ref.data(), c.m, c.n, c.k, 1);
     } else {
       std::vector<float> qdq = a, scale(c.m);               // QuantizeFp8Ref then GemmMxFp4Ref
       orc_quantize_fp8_ref(qdq.data(), scale.data(), c.m, c.k);

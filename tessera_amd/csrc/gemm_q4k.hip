@@ -330,38 +330,57 @@ hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* wor
 // swizzled LDS rings.
 namespace {
 
-__device__ __forceinline__ uint32_t perm8(uint32_t e) {   // position of element e inside its group of 8
-  const uint32_t i = e & 7u;
-  return (e & ~7u) | ((i == 1u || i == 5u) ? i + 1u : (i == 2u || i == 6u) ? i - 1u : i);
+// Eight consecutive values of a group in the stored order 0,2,1,3,4,6,5,7.
+__device__ __forceinline__ void store_perm8(_Float16* dst, const float (&v)[8]) {
+  half8_t h;
+  h[0] = static_cast<_Float16>(v[0]), h[1] = static_cast<_Float16>(v[2]);
+  h[2] = static_cast<_Float16>(v[1]), h[3] = static_cast<_Float16>(v[3]);
+  h[4] = static_cast<_Float16>(v[4]), h[5] = static_cast<_Float16>(v[6]);
+  h[6] = static_cast<_Float16>(v[5]), h[7] = static_cast<_Float16>(v[7]);
+  *reinterpret_cast<half8_t*>(dst) = h;
 }
 
-// One thread per (block, half n, lane l): the four values sharing ql[n*64+l], ql[n*64+32+l],
-// qh[n*32+l] (src/core/numerics/quant.cpp:421-450).
+__device__ __forceinline__ uint64_t load8_a2(const uint8_t* p) {   // eight bytes from a 2-byte aligned address
+  const uint16_t* q = reinterpret_cast<const uint16_t*>(p);
+  return static_cast<uint64_t>(q[0]) | (static_cast<uint64_t>(q[1]) << 16) | (static_cast<uint64_t>(q[2]) << 32) |
+         (static_cast<uint64_t>(q[3]) << 48);
+}
+
+// One thread per (block, half n, eight lanes l = 8o..8o+7): 32 values, four 16-byte stores
+// (src/core/numerics/quant.cpp:421-450).
 __global__ __launch_bounds__(256) void q6k_to_f16_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ out,
                                                          uint64_t nitems) {
   const uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (t >= nitems) return;
-  const uint64_t blk = t >> 6;
-  const uint32_t n = static_cast<uint32_t>(t >> 5) & 1u, l = static_cast<uint32_t>(t) & 31u, is = l >> 4;
+  const uint64_t blk = t >> 3;
+  const uint32_t n = static_cast<uint32_t>(t >> 2) & 1u, o = static_cast<uint32_t>(t) & 3u, is = o >> 1;
   const uint8_t* base = w + blk * 210u;
-  const uint32_t a = base[n * 64 + l], b = base[n * 64 + 32 + l], h = base[128 + n * 32 + l];
-  const float d = half_bits_to_float(static_cast<uint32_t>(base[208]) | (static_cast<uint32_t>(base[209]) << 8));
-  const int q[4] = {static_cast<int>((a & 15u) | ((h & 3u) << 4)), static_cast<int>((b & 15u) | (((h >> 2) & 3u) << 4)),
-                    static_cast<int>((a >> 4) | (((h >> 4) & 3u) << 4)), static_cast<int>((b >> 4) | ((h >> 6) << 4))};
+  const uint64_t a = load8_a2(base + n * 64 + o * 8), b = load8_a2(base + n * 64 + 32 + o * 8);
+  const uint64_t h = load8_a2(base + 128 + n * 32 + o * 8);
+  const float d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(base + 208));
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const float s = static_cast<float>(static_cast<int8_t>(base[192 + n * 8 + is + 2 * j]));
-    out[blk * 256 + perm8(n * 128 + 32 * j + l)] = static_cast<_Float16>(d * s * static_cast<float>(q[j] - 32));
+    const float ds = d * static_cast<float>(static_cast<int8_t>(base[192 + n * 8 + is + 2 * j]));
+    const uint64_t lo = (j & 1) ? b : a;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t nib = static_cast<uint32_t>(lo >> (8 * i + 4 * (j >> 1))) & 15u;
+      const uint32_t top = static_cast<uint32_t>(h >> (8 * i + 2 * j)) & 3u;
+      v[i] = ds * static_cast<float>(static_cast<int>(nib | (top << 4)) - 32);
+    }
+    store_perm8(out + blk * 256 + n * 128 + 32 * j + o * 8, v);
   }
 }
 
-// One thread per quant byte (block, group g, lane l) (src/core/numerics/quant.cpp:388-419).
+// One thread per (block, group g, eight lanes): 16 values, two 16-byte stores
+// (src/core/numerics/quant.cpp:388-419).
 __global__ __launch_bounds__(256) void q5k_to_f16_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ out,
                                                          uint64_t nitems) {
   const uint64_t t = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (t >= nitems) return;
-  const uint64_t blk = t >> 7;
-  const uint32_t g = static_cast<uint32_t>(t >> 5) & 3u, l = static_cast<uint32_t>(t) & 31u;
+  const uint64_t blk = t >> 4;
+  const uint32_t g = static_cast<uint32_t>(t >> 2) & 3u, o = static_cast<uint32_t>(t) & 3u;
   const uint8_t* base = w + blk * 176u;
   const uint8_t* p = base + 4;
   auto scale_min = [&](uint32_t sb, uint32_t& sc, uint32_t& mn) {
@@ -376,20 +395,28 @@ __global__ __launch_bounds__(256) void q5k_to_f16_kernel(const uint8_t* __restri
   uint32_t sca, mna, scb, mnb;
   scale_min(2 * g, sca, mna);
   scale_min(2 * g + 1, scb, mnb);
-  const float d = half_bits_to_float(static_cast<uint32_t>(base[0]) | (static_cast<uint32_t>(base[1]) << 8));
-  const float dmin = half_bits_to_float(static_cast<uint32_t>(base[2]) | (static_cast<uint32_t>(base[3]) << 8));
-  const uint32_t low = base[48 + g * 32 + l], high = base[16 + l];
-  const float q0 = static_cast<float>((low & 15u) + (((high >> (2 * g)) & 1u) << 4));
-  const float q1 = static_cast<float>((low >> 4) + (((high >> (2 * g + 1)) & 1u) << 4));
-  out[blk * 256 + perm8(g * 64 + l)] = static_cast<_Float16>(d * static_cast<float>(sca) * q0 - dmin * static_cast<float>(mna));
-  out[blk * 256 + perm8(g * 64 + 32 + l)] = static_cast<_Float16>(d * static_cast<float>(scb) * q1 - dmin * static_cast<float>(mnb));
+  const uint32_t dd = *reinterpret_cast<const uint32_t*>(base);
+  const float d = half_bits_to_float(dd & 0xFFFFu), dmin = half_bits_to_float(dd >> 16);
+  const float d1 = d * static_cast<float>(sca), m1 = dmin * static_cast<float>(mna);
+  const float d2 = d * static_cast<float>(scb), m2 = dmin * static_cast<float>(mnb);
+  const uint64_t low = *reinterpret_cast<const uint64_t*>(base + 48 + g * 32 + o * 8);
+  const uint64_t high = *reinterpret_cast<const uint64_t*>(base + 16 + o * 8);
+  float v0[8], v1[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t lb = static_cast<uint32_t>(low >> (8 * i)) & 0xFFu, hb = static_cast<uint32_t>(high >> (8 * i)) & 0xFFu;
+    v0[i] = d1 * static_cast<float>((lb & 15u) + (((hb >> (2 * g)) & 1u) << 4)) - m1;
+    v1[i] = d2 * static_cast<float>((lb >> 4) + (((hb >> (2 * g + 1)) & 1u) << 4)) - m2;
+  }
+  store_perm8(out + blk * 256 + g * 64 + o * 8, v0);
+  store_perm8(out + blk * 256 + g * 64 + 32 + o * 8, v1);
 }
 
 // C tile = A16 (rows scaled by a_scale) . W16^T, both operands fp16 row-major with row length k.
 template <int BM, int BN>
 __global__ __launch_bounds__(BN * 2) void f16w_gemm_kernel(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const _Float16* __restrict__ w16,
-    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k) {
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end) {
   constexpr int kWaves = BN / 32, kTI = BM / 32;
   constexpr int kABlk = BM / 16 / kWaves, kWBlk = BN / 16 / kWaves;   // 1 KB blocks per wavefront and slice
   constexpr int kDma = kABlk + kWBlk;
@@ -397,8 +424,8 @@ __global__ __launch_bounds__(BN * 2) void f16w_gemm_kernel(
   static_assert(BM % (16 * kWaves) == 0 && BN % (16 * kWaves) == 0, "tile shape");
   __shared__ __attribute__((aligned(16))) uint8_t lds[4 * kStage];
 
-  const uint32_t tiles_n = (n + BN - 1) / BN;
-  const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+  const uint32_t tiles_n = (n_end - n_begin + BN - 1) / BN;
+  const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = n_begin + (blockIdx.x % tiles_n) * BN;
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t l32 = lane & 31u, kg = lane >> 5;
@@ -473,7 +500,7 @@ __global__ __launch_bounds__(BN * 2) void f16w_gemm_kernel(
       const uint32_t row = m0 + i * 32u + (e >> 2) * 8u + kg * 4u + (e & 3u);
       const float4 s4 = sc[e >> 2];
       const float rs = (e & 3) == 0 ? s4.x : (e & 3) == 1 ? s4.y : (e & 3) == 2 ? s4.z : s4.w;
-      if (row < m && col < n) c[static_cast<size_t>(row) * n + col] = acc[i][e] * rs;
+      if (row < m && col < n_end) c[static_cast<size_t>(row) * n + col] = acc[i][e] * rs;
     }
   }
 }
@@ -497,17 +524,34 @@ hipError_t launch_kquant_f16_gemm(const float* a, const uint8_t* w, uint32_t blo
   _Float16* w16 = reinterpret_cast<_Float16*>(a_scale + m + 256);
   const uint64_t blocks = static_cast<uint64_t>(n) * (k / 256);
   if (block_bytes == 210) {
-    hipLaunchKernelGGL(q6k_to_f16_kernel, dim3(static_cast<uint32_t>((blocks * 64 + 255) / 256)), dim3(256), 0, stream,
-                       w, w16, blocks * 64);
+    hipLaunchKernelGGL(q6k_to_f16_kernel, dim3(static_cast<uint32_t>((blocks * 8 + 255) / 256)), dim3(256), 0, stream,
+                       w, w16, blocks * 8);
   } else if (block_bytes == 176) {
-    hipLaunchKernelGGL(q5k_to_f16_kernel, dim3(static_cast<uint32_t>((blocks * 128 + 255) / 256)), dim3(256), 0, stream,
-                       w, w16, blocks * 128);
+    hipLaunchKernelGGL(q5k_to_f16_kernel, dim3(static_cast<uint32_t>((blocks * 16 + 255) / 256)), dim3(256), 0, stream,
+                       w, w16, blocks * 16);
   } else {
     return hipErrorInvalidValue;
   }
   hipLaunchKernelGGL(rows_to_f16_kernel, dim3(m), dim3(256), 0, stream, a, a16, a_scale, k, nullptr, 1u);
-  const uint32_t tiles = ((m + 255u) / 256u) * ((n + 255u) / 256u);
-  hipLaunchKernelGGL((f16w_gemm_kernel<256, 256>), dim3(tiles), dim3(512), 0, stream, a16, a_scale, w16, c, m, n, k);
+  // whole rounds of 256 x 256 tiles, leftover columns as 128 x 64 tiles (as launch_q4k_gemm)
+  const uint32_t cus = static_cast<uint32_t>(num_cus());
+  const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u, tiles = tiles_m * tiles_n;
+  uint32_t main_tn = tiles_n;
+  if (tiles > cus && tiles % cus != 0 && tiles % cus <= cus / 2) {
+    main_tn = (tiles / cus) * cus / tiles_m;
+  } else if (tiles < cus / 2) {
+    main_tn = 0;
+  }
+  const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
+  if (n_split > 0) {
+    hipLaunchKernelGGL((f16w_gemm_kernel<256, 256>), dim3(tiles_m * main_tn), dim3(512), 0, stream, a16, a_scale, w16,
+                       c, m, n, k, 0u, n_split);
+  }
+  if (n_split < n) {
+    const uint32_t t2 = ((m + 127u) / 128u) * ((n - n_split + 63u) / 64u);
+    hipLaunchKernelGGL((f16w_gemm_kernel<128, 64>), dim3(t2), dim3(128), 0, stream, a16, a_scale, w16, c, m, n, k,
+                       n_split, n);
+  }
   return hipGetLastError();
 }
 

@@ -156,7 +156,22 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
         few[f"m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                         "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
     out["q4k_few_rows_17408x5120"] = few
-    del wq_list, w_q1
+    del wq_list
+
+    # ---- gate and up stored as one 34816 x 5120 tensor (a loader may concatenate them): the same
+    # id and kernel, one launch instead of two, so the fixed cost of a launch is paid once ----------
+    w_gu = torch.cat([w_q1, w_q1.clone()])
+    gu_list = [w_gu] + [w_gu.clone() for _ in range(3)]
+    kvec = backend.LoadKernel("gemm_q4k_vec")
+    x = to_dev(synth.activations_f32(g, 1, k))
+    y = torch.empty(2 * n, dtype=torch.float32, device=dev)
+    launches = [(kvec, KernelLaunch(grid_x=(2 * n + 7) // 8, buffers=[wrap(x), wrap(w), wrap(y)], scalars=[1, 2 * n, k, 1]))
+                for w in gu_list]
+    us = timed_us(launches, 20) / len(gu_list)
+    nbytes = 2 * n * (k // 256) * 144 + 4 * k + 4 * 2 * n
+    out["q4k_gemv_m1_gate_up_as_one_34816x5120"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                                    "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    del gu_list, w_gu, w_q1
 
     # ---- Q6_K and Q5_K (the other block formats of K-quant files), gate/up and down shapes --------
     for fmt, block_bytes, gen, rows in (("q6k", 210, synth.q6k_weights, (1, 2)), ("q5k", 176, synth.q5k_weights, (1,))):

@@ -315,6 +315,16 @@ hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* wor
   } else if (tiles < cus / 2) {
     main_tn = 0;
   }
+  if (m <= 64) {
+    // A short stack of rows is bound by the weight stream: narrow tiles (one wavefront, 32
+    // columns) give every CU several workgroups' worth of super-blocks in flight.
+    if (m <= 32) {
+      launch_range<32, 32>(a16, a_scale, w, c, m, n, k, 0u, n, stream);
+    } else {
+      launch_range<64, 32>(a16, a_scale, w, c, m, n, k, 0u, n, stream);
+    }
+    return hipGetLastError();
+  }
   const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
   if (n_split > 0) launch_range<256, 256>(a16, a_scale, w, c, m, n, k, 0u, n_split, stream);
   if (n_split < n) launch_range<128, 64>(a16, a_scale, w, c, m, n, k, n_split, n, stream);

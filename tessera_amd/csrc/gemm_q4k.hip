@@ -265,21 +265,24 @@ __global__ __launch_bounds__(BN * 2) void q4k_gemm_kernel(
                         n_end);
 }
 
-// Grouped form for routed experts: segment e (grid.y) multiplies rows seg[e]..seg[e+1] of a16
+// Grouped form for routed experts: segment e (grid.x) multiplies rows seg[e]..seg[e+1] of a16
 // by expert e's weights (w + e * w_stride) into the same rows of c.  Segment bounds live in
 // device memory (the routing is computed on the device); an empty segment leaves at once.
 template <int BM, int BN>
 __global__ __launch_bounds__(BN * 2) void q4k_gemm_grouped_kernel(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
     float* __restrict__ c, const uint32_t* __restrict__ seg, uint64_t w_stride, uint32_t n, uint32_t k) {
-  const uint32_t e = blockIdx.y;
+  // Expert on grid.x: workgroups are dealt to the eight XCDs by linear index, so with the
+  // expert varying fastest all column tiles of an expert land on one XCD and its activation
+  // rows are fetched into one L2 instead of eight.
+  const uint32_t e = blockIdx.x;
   const uint32_t r0 = seg[e], r1 = seg[e + 1];
   if (r1 <= r0) return;
   const _Float16* a_e = a16 + static_cast<size_t>(r0) * k;
   const uint8_t* w_e = w + e * w_stride;
   float* c_e = c + static_cast<size_t>(r0) * n;
   for (uint32_t m0 = 0; m0 < r1 - r0; m0 += BM) {
-    q4k_gemm_tile<BM, BN>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, blockIdx.x * BN, n);
+    q4k_gemm_tile<BM, BN>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, blockIdx.y * BN, n);
   }
 }
 
@@ -685,12 +688,12 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
   hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, seg, pos);
   hipLaunchKernelGGL(rows_to_f16_kernel, dim3(pairs), dim3(256), 0, stream, x, a16, x_scale, hidden, pos, top_k);
   constexpr int BM = 32, BN = 64;
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3((inter + BN - 1) / BN, experts), dim3(BN * 2), 0, stream,
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (inter + BN - 1) / BN), dim3(BN * 2), 0, stream,
                      a16, x_scale, gate, g, seg, gate_stride, inter, hidden);
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3((inter + BN - 1) / BN, experts), dim3(BN * 2), 0, stream,
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (inter + BN - 1) / BN), dim3(BN * 2), 0, stream,
                      a16, x_scale, up, u, seg, up_stride, inter, hidden);
   hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(pairs), dim3(256), 0, stream, g, u, phi16, phi_scale, inter);
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3((hidden + BN - 1) / BN, experts), dim3(BN * 2), 0, stream,
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (hidden + BN - 1) / BN), dim3(BN * 2), 0, stream,
                      phi16, phi_scale, down, rows, seg, down_stride, hidden, inter);
   const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, rows, pos,

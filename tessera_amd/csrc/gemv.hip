@@ -1011,9 +1011,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   const bool two = row_a != row_b;  // wavefront-uniform
   const float in_a = (prow == row_a) ? 1.0f : 0.0f, in_b = 1.0f - in_a;
 
-  // Groups [g0, g1) belong to this workgroup.  A group index past the end is clamped
-  // for the loads and dropped at the store; rows past n inside the last group re-read
-  // the group's first row.
+  // Groups [g0, g1) belong to this workgroup.  A group index past its end is clamped to its
+  // last group for the loads (a prefetch must not pull the next workgroup's rows, which would
+  // come from HBM a second time through another XCD's L2) and dropped at the store; rows past
+  // n inside the last group re-read the group's first row.
   const uint32_t groups = (n + P - 1) / P;
   const uint32_t g0 = blockIdx.x * groups_per_wg;
   const uint32_t g1 = g0 + groups_per_wg < groups ? g0 + groups_per_wg : groups;
@@ -1021,7 +1022,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   const Lane ln_tail = Codec::make_lane(args, cpr, chunk, (groups - 1u) * P + prow < n ? prow : 0u);
   const bool ragged = n % P != 0;
   auto fetch = [&](uint32_t grp, typename Codec::Frag& f) {
-    grp = grp < groups ? grp : groups - 1u;
+    grp = grp < g1 ? grp : g1 - 1u;
     const bool tail = ragged && grp == groups - 1u;
     Codec::load(args, tail ? ln_tail : ln, grp * P, cpr, f);
   };

@@ -11,16 +11,23 @@
 //
 // Weights never exist dequantized in memory: the raw 144-byte super-blocks travel
 // HBM -> LDS by direct loads, and each wavefront decodes the eight weights a lane owes the
-// B operand of one MFMA straight from those bytes into registers -- nibbles to fp16 with
-// the 0x6400 exponent trick, then one packed fma with the sub-block's (d*sc, dmin*mn) pair,
-// i.e. w16 = fma(q, RN16(d*sc), -RN16(dmin*mn)).  A wavefront owns 32 output columns and all
-// of the tile's rows, so no two wavefronts decode the same weight.  The nibble pairs come out
-// of a dword in the order (k0,k2),(k1,k3); instead of un-shuffling them, the fp16 copy of A
-// is written with the same order inside every group of 8, which a dot product cannot see.
+// B operand of one MFMA straight from those bytes into registers -- a nibble pair is masked
+// into the mantissa of an fp16 constant in one v_and_or_b32 (1024.0 for low nibbles, 64.0 for
+// high ones, so neither needs a shift), the constant subtracted, then one packed fma with the
+// sub-block's (d*sc, dmin*mn) pair, i.e. w16 = fma(q, RN16(d*sc), -RN16(dmin*mn)): three VALU
+// instructions per two weights.  The nibble pairs come out of a dword in the order
+// (k0,k2),(k1,k3); instead of un-shuffling them, the fp16 copy of A is written with the same
+// order inside every group of 8, which a dot product cannot see.
+//
+// A wavefront owns WM rows x WN columns of the workgroup's tile.  Small tiles (a short stack of
+// rows) use WN = 32 and all rows, so no two wavefronts decode the same weight; the 256 x 256
+// prefill tile uses 128 x 64, where each activation fragment read from LDS feeds two MFMAs.
 //
 // K advances one 32-wide sub-block per step: activation slices (BM x 64 bytes) run through
 // a four-stage XOR-swizzled LDS ring, raw weight super-blocks through a two-stage ring that
 // is refilled once per eight steps; waits are counted by hand as in gemm_mxfp4.hip.
+
+#include <type_traits>
 
 #include "qmm_device.hpp"
 #include "qmm_kernels.hpp"
@@ -84,27 +91,99 @@ __global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restric
   if (threadIdx.x == 0) scale[drow] = s;
 }
 
-// Two packed fp16 weights from the nibbles at bits [3:0] and [19:16] of `x`.
-__device__ __forceinline__ half2_t decode_pair(uint32_t x, half2_t scale, half2_t neg_min) {
-  const half2_t q = bit_cast<half2_t>((x & 0x000F000Fu) | 0x64006400u) - half2_t{1024, 1024};  // exact 0..15
-  return __builtin_elementwise_fma(q, scale, neg_min);
+// body(integral_constant<int, 0>) ... body(integral_constant<int, N - 1>), in order.
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void unrolled(F&& body) {
+  if constexpr (I < N) {
+    body(std::integral_constant<int, I>{});
+    unrolled<N, I + 1>(body);
+  }
 }
 
-// One BM x BN tile of C at (m0, n0); columns at and past n_end are not stored.
-template <int BM, int BN>
+// (x & mask) | magic in one instruction.  With the two constants in registers the three-operand
+// form applies; as literals they would cost an AND and an OR (one literal an instruction).
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(mask), "v"(magic));
+  return r;
+}
+
+// Nibble decode constants, kept in registers for and_or.  Low nibbles (bits [3:0] and [19:16])
+// are or-ed into the mantissa of 1024.0, high nibbles (bits [7:4] and [23:20]) into that of 64.0,
+// where the same four bits weigh 1: no shift is needed for either, and subtracting the base
+// leaves the exact integer 0..15.
+struct NibbleConsts {
+  uint32_t mask[2], magic[2];
+  half2_t base[2];
+};
+__device__ __forceinline__ NibbleConsts nibble_consts() {
+  NibbleConsts c;
+  c.mask[0] = 0x000F000Fu, c.mask[1] = 0x00F000F0u;
+  c.magic[0] = 0x64006400u, c.magic[1] = 0x54005400u;
+  asm volatile("" : "+v"(c.mask[0]), "+v"(c.mask[1]), "+v"(c.magic[0]), "+v"(c.magic[1]));  // not literals
+  c.base[0] = half2_t{1024, 1024}, c.base[1] = half2_t{64, 64};
+  return c;
+}
+
+// Two packed fp16 weights q * scale - min from the nibbles (low: HI = 0, high: HI = 1) of bytes 0
+// and 2 of `x`; `sm` holds the sub-block's fp16 scale in its low half and minus its min in the
+// high half.
+template <int HI>
+__device__ __forceinline__ half2_t decode_pair(uint32_t x, const NibbleConsts& c, half2_t sm) {
+  const half2_t q = bit_cast<half2_t>(and_or(x, c.mask[HI], c.magic[HI])) - c.base[HI];   // exact 0..15
+  return __builtin_elementwise_fma(q, half2_t{sm[0], sm[0]}, half2_t{sm[1], sm[1]});
+}
+
+// The 6-bit scales and mins of a super-block, one byte each (src/core/numerics/quant.cpp:58-70):
+// sc[0], mn[0] hold sub-blocks 0..3, sc[1], mn[1] sub-blocks 4..7.
+struct ScaleBytes {
+  uint32_t sc[2], mn[2];
+};
+__device__ __forceinline__ ScaleBytes unpack_scales(uint32_t s0, uint32_t s1, uint32_t s2) {
+  ScaleBytes r;
+  r.sc[0] = s0 & 0x3F3F3F3Fu;
+  r.mn[0] = s1 & 0x3F3F3F3Fu;
+  r.sc[1] = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+  r.mn[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+  return r;
+}
+
+// (d * sc, -(dmin * mn)) of sub-block SB as packed fp16, each product rounded once to nearest
+// even (the 6-bit integers are exact in fp16).  `d_negdmin` is the block header with the sign of
+// its high half flipped.
+template <int SB>
+__device__ __forceinline__ half2_t scale_min_f16(const ScaleBytes& sbytes, half2_t d_negdmin) {
+  constexpr uint32_t kSel = 0x0C000C00u | ((4u + (SB & 3)) << 16) | (SB & 3);   // bytes: sc, 0, mn, 0
+  const uint32_t pair = __builtin_amdgcn_perm(sbytes.mn[SB >> 2], sbytes.sc[SB >> 2], kSel);
+  const half2_t ints = bit_cast<half2_t>(pair | 0x64006400u) - half2_t{1024, 1024};
+  return ints * d_negdmin;
+}
+
+// Wavefronts of a BM x BN tile whose wavefronts each own WM rows x WN columns.
+template <int BM, int BN, int WM, int WN>
+constexpr int tile_waves() { return (BM / WM) * (BN / WN); }
+
+// One BM x BN tile of C at (m0, n0); columns at and past n_end are not stored.  A wavefront owns
+// WM rows x WN columns of it.  Every MFMA takes its activation fragment from LDS (1 KB a
+// wavefront, against 128 bytes a clock for the whole CU, which four SIMDs running 32-clock MFMAs
+// would need in full); with WN = 64 a fragment read feeds two MFMAs.  The price is that the
+// BM / WM wavefronts that share a column range each decode its weights.
+template <int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void q4k_gemm_tile(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
     float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t m0, uint32_t n0, uint32_t n_end) {
-  constexpr int kWaves = BN / 32;                  // one wavefront per 32 output columns
-  constexpr int kTI = BM / 32;                     // MFMA tiles per wavefront (all rows of the tile)
+  constexpr int kWaves = tile_waves<BM, BN, WM, WN>();
+  constexpr int kWavesN = BN / WN;
+  constexpr int kTI = WM / 32, kTJ = WN / 32;      // MFMA tiles per wavefront: rows x columns
   constexpr int kABlk = BM / 16 / kWaves;          // 1 KB activation blocks a wavefront loads per step
   constexpr int kWL = (BN * 9 + 64 * kWaves - 1) / (64 * kWaves);  // 1 KB weight blocks per super-block
   constexpr uint32_t kAStage = BM * 64, kWStage = kWL * kWaves * 1024;
-  static_assert(BM % (16 * kWaves) == 0 && BN % 32 == 0, "tile shape");
+  static_assert(BM % WM == 0 && BN % WN == 0 && WM % 32 == 0 && WN % 32 == 0 && BM % (16 * kWaves) == 0, "tile shape");
   __shared__ __attribute__((aligned(16))) uint8_t lds[4 * kAStage + 2 * kWStage];
 
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t wave_m = wave / kWavesN, wave_n = wave % kWavesN;
   const uint32_t l32 = lane & 31u, kg = lane >> 5;
   const uint32_t row_blocks = k / 256;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
@@ -142,21 +221,24 @@ __device__ __forceinline__ void q4k_gemm_tile(
     for (int i = 0; i < kWL; ++i) direct_load16(g, w_src[i], lds_base + 4 * kAStage + stage * kWStage + (wave * kWL + i) * 1024u);
   };
 
-  float16_t acc[kTI];
+  float16_t acc[kTI][kTJ];
 #pragma unroll
   for (int i = 0; i < kTI; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+    for (int j = 0; j < kTJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  // This lane's weight row inside a raw stage, and its activation fragment offsets: MFMA
-  // step t of a slice takes chunk 2t + kg of the row (k = 16t + 8kg + [0,8)).
-  const uint32_t w_row = (wave * 32u + l32) * 144u;
+  // This lane's first weight row inside a raw stage (column tile j is 32 rows further), and its
+  // activation fragment offsets: MFMA step t of a slice takes chunk 2t + kg of the row
+  // (k = 16t + 8kg + [0,8)).
+  const uint32_t w_row = (wave_n * WN + l32) * 144u;
   uint32_t a_fr[2];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) a_fr[tt] = l32 * 64u + (((tt * 2u + kg) ^ ((l32 >> 2) & 3u)) * 16u);
+  for (int tt = 0; tt < 2; ++tt) a_fr[tt] = (wave_m * WM + l32) * 64u + (((tt * 2u + kg) ^ ((l32 >> 2) & 3u)) * 16u);
 
   const uint32_t slices = k / 32;
-  uint32_t d_bits = 0, sc0 = 0, sc1 = 0, sc2 = 0;   // header and packed scales of the current super-block
+  const NibbleConsts nc = nibble_consts();
 
   // Prologue: first super-block and three activation slices in flight, then the first of each
   // is waited for.
@@ -169,48 +251,44 @@ __device__ __forceinline__ void q4k_gemm_tile(
   for (uint32_t blk = 0; blk < row_blocks; ++blk) {
     const uint8_t* raw = lds + 4 * kAStage + (blk & 1u) * kWStage + w_row;
     const bool more = blk + 1 < row_blocks;        // uniform
-    d_bits = *reinterpret_cast<const uint32_t*>(raw);
-    sc0 = *reinterpret_cast<const uint32_t*>(raw + 4);
-    sc1 = *reinterpret_cast<const uint32_t*>(raw + 8);
-    sc2 = *reinterpret_cast<const uint32_t*>(raw + 12);
-    const float d = half_bits_to_float(d_bits & 0xFFFFu), dmin = half_bits_to_float(d_bits >> 16);
+    half2_t d_negdmin[kTJ];                        // block header, sign of dmin flipped
+    ScaleBytes sbytes[kTJ];
 #pragma unroll
-    for (int sb = 0; sb < 8; ++sb) {
+    for (int j = 0; j < kTJ; ++j) {
+      const uint4 head = *reinterpret_cast<const uint4*>(raw + j * 32 * 144);
+      d_negdmin[j] = bit_cast<half2_t>(head.x ^ 0x80000000u);
+      sbytes[j] = unpack_scales(head.y, head.z, head.w);
+    }
+    uint32_t qw[kTJ][4], qs8[kTJ][4];
+    unrolled<8>([&](auto step) {
+      constexpr int sb = decltype(step)::value;
+      constexpr int kHi = sb & 1;
       const uint32_t slice = blk * 8u + sb;
       if (sb == 0 && more) issue_w((blk + 1u) & 1u, blk + 1u);
       issue_a((slice + 3u) & 3u, slice + 3u < slices ? slice + 3u : slices - 1u);
 
-      // 6-bit scale and min of sub-block sb (src/core/numerics/quant.cpp:58-70).
-      uint32_t sc, mn;
-      if (sb < 4) {
-        sc = (sc0 >> (8 * sb)) & 63u;
-        mn = (sc1 >> (8 * sb)) & 63u;
-      } else {
-        const uint32_t hi = (sc2 >> (8 * (sb - 4))) & 0xFFu;
-        sc = (hi & 15u) | (((sc0 >> (8 * (sb - 4) + 6)) & 3u) << 4);
-        mn = (hi >> 4) | (((sc1 >> (8 * (sb - 4) + 6)) & 3u) << 4);
-      }
-      const _Float16 s16 = static_cast<_Float16>(d * static_cast<float>(sc));
-      const _Float16 m16 = static_cast<_Float16>(-(dmin * static_cast<float>(mn)));
-      const half2_t scale = {s16, s16}, neg_min = {m16, m16};
-
-      // Quant bytes of this lane's 16 weights: sub-block sb lives in the low (even sb) or high
-      // nibbles of bytes (sb/2)*32 + [0,32) (src/core/numerics/quant.cpp:656-675).
-      const uint8_t* qp = raw + 16 + (sb >> 1) * 32 + kg * 8u;
-      const uint2 q0 = *reinterpret_cast<const uint2*>(qp);
-      const uint2 q1 = *reinterpret_cast<const uint2*>(qp + 16);
-      constexpr int kNoShift = 0;
-      const int sh = (sb & 1) ? 4 : kNoShift;
-      half8_t b[2];
-      {
-        const half2_t p0 = decode_pair(q0.x >> sh, scale, neg_min), p1 = decode_pair(q0.x >> (sh + 8), scale, neg_min);
-        const half2_t p2 = decode_pair(q0.y >> sh, scale, neg_min), p3 = decode_pair(q0.y >> (sh + 8), scale, neg_min);
-        b[0] = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
-      }
-      {
-        const half2_t p0 = decode_pair(q1.x >> sh, scale, neg_min), p1 = decode_pair(q1.x >> (sh + 8), scale, neg_min);
-        const half2_t p2 = decode_pair(q1.y >> sh, scale, neg_min), p3 = decode_pair(q1.y >> (sh + 8), scale, neg_min);
-        b[1] = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+      // Quant bytes of this lane's 16 weights a column: sub-block sb lives in the low (even sb)
+      // or high nibbles of bytes (sb/2)*32 + [0,32) (src/core/numerics/quant.cpp:656-675).  An
+      // odd step decodes the same bytes as the even step before it: the words shifted down by
+      // one byte (for bytes 1 and 3) are kept from there.
+      half8_t b[kTJ][2];
+#pragma unroll
+      for (int j = 0; j < kTJ; ++j) {
+        const half2_t sm = scale_min_f16<sb>(sbytes[j], d_negdmin[j]);
+        if (kHi == 0) {
+          const uint8_t* qp = raw + j * 32 * 144 + 16 + (sb >> 1) * 32 + kg * 8u;
+          const uint2 q0 = *reinterpret_cast<const uint2*>(qp);
+          const uint2 q1 = *reinterpret_cast<const uint2*>(qp + 16);
+          qw[j][0] = q0.x, qw[j][1] = q0.y, qw[j][2] = q1.x, qw[j][3] = q1.y;
+#pragma unroll
+          for (int x = 0; x < 4; ++x) qs8[j][x] = qw[j][x] >> 8;
+        }
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const half2_t p0 = decode_pair<kHi>(qw[j][2 * tt], nc, sm), p1 = decode_pair<kHi>(qs8[j][2 * tt], nc, sm);
+          const half2_t p2 = decode_pair<kHi>(qw[j][2 * tt + 1], nc, sm), p3 = decode_pair<kHi>(qs8[j][2 * tt + 1], nc, sm);
+          b[j][tt] = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+        }
       }
 
       const uint8_t* a_stage = lds + (slice & 3u) * kAStage;
@@ -219,7 +297,8 @@ __device__ __forceinline__ void q4k_gemm_tile(
 #pragma unroll
         for (int i = 0; i < kTI; ++i) {
           const half8_t af = *reinterpret_cast<const half8_t*>(a_stage + a_fr[tt] + i * 32 * 64);
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[tt], acc[i], 0, 0, 0);
+#pragma unroll
+          for (int j = 0; j < kTJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[j][tt], acc[i][j], 0, 0, 0);
         }
       }
 
@@ -231,37 +310,39 @@ __device__ __forceinline__ void q4k_gemm_tile(
       } else {
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * kABlk) : "memory");
       }
-    }
+    });
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the workgroup
 
   // Epilogue: lane holds column l32 and rows (e/4)*8 + kg*4 + e%4 of each 32 x 32 tile; the
   // four row scales of each e/4 group are one 16-byte load (the scale array is padded, so rows
   // past m read something harmless).
-  const uint32_t col = n0 + wave * 32u + l32;
 #pragma unroll
   for (int i = 0; i < kTI; ++i) {
+    const uint32_t row0 = m0 + wave_m * WM + i * 32u + kg * 4u;
     float4 sc[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      sc[q] = *reinterpret_cast<const float4*>(a_scale + m0 + i * 32u + q * 8u + kg * 4u);
-    }
+    for (int q = 0; q < 4; ++q) sc[q] = *reinterpret_cast<const float4*>(a_scale + row0 + q * 8u);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const uint32_t row = m0 + i * 32u + (e >> 2) * 8u + kg * 4u + (e & 3u);
-      const float4 s4 = sc[e >> 2];
-      const float rs = (e & 3) == 0 ? s4.x : (e & 3) == 1 ? s4.y : (e & 3) == 2 ? s4.z : s4.w;
-      if (row < m && col < n_end) c[static_cast<size_t>(row) * n + col] = acc[i][e] * rs;
+    for (int j = 0; j < kTJ; ++j) {
+      const uint32_t col = n0 + wave_n * WN + j * 32u + l32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t row = row0 + (e >> 2) * 8u + (e & 3u);
+        const float4 s4 = sc[e >> 2];
+        const float rs = (e & 3) == 0 ? s4.x : (e & 3) == 1 ? s4.y : (e & 3) == 2 ? s4.z : s4.w;
+        if (row < m && col < n_end) c[static_cast<size_t>(row) * n + col] = acc[i][j][e] * rs;
+      }
     }
   }
 }
 
-template <int BM, int BN>
-__global__ __launch_bounds__(BN * 2) void q4k_gemm_kernel(
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void q4k_gemm_kernel(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
     float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end) {
   const uint32_t tiles_n = (n_end - n_begin + BN - 1) / BN;
-  q4k_gemm_tile<BM, BN>(a16, a_scale, w, c, m, n, k, (blockIdx.x / tiles_n) * BM, n_begin + (blockIdx.x % tiles_n) * BN,
+  q4k_gemm_tile<BM, BN, WM, WN>(a16, a_scale, w, c, m, n, k, (blockIdx.x / tiles_n) * BM, n_begin + (blockIdx.x % tiles_n) * BN,
                         n_end);
 }
 
@@ -282,16 +363,16 @@ __global__ __launch_bounds__(BN * 2) void q4k_gemm_grouped_kernel(
   const uint8_t* w_e = w + e * w_stride;
   float* c_e = c + static_cast<size_t>(r0) * n;
   for (uint32_t m0 = 0; m0 < r1 - r0; m0 += BM) {
-    q4k_gemm_tile<BM, BN>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, blockIdx.y * BN, n);
+    q4k_gemm_tile<BM, BN, BM, 32>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, blockIdx.y * BN, n);
   }
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int WM = BM, int WN = 32>
 void launch_range(const _Float16* a16, const float* a_scale, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                   uint32_t k, uint32_t n_begin, uint32_t n_end, hipStream_t stream) {
   const uint32_t tiles = ((m + BM - 1) / BM) * ((n_end - n_begin + BN - 1) / BN);
-  hipLaunchKernelGGL((q4k_gemm_kernel<BM, BN>), dim3(tiles), dim3(BN * 2), 0, stream, a16, a_scale, w, c, m, n, k,
-                     n_begin, n_end);
+  hipLaunchKernelGGL((q4k_gemm_kernel<BM, BN, WM, WN>), dim3(tiles), dim3(tile_waves<BM, BN, WM, WN>() * 64), 0, stream,
+                     a16, a_scale, w, c, m, n, k, n_begin, n_end);
 }
 
 }  // namespace
@@ -329,7 +410,7 @@ hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* wor
     return hipGetLastError();
   }
   const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
-  if (n_split > 0) launch_range<256, 256>(a16, a_scale, w, c, m, n, k, 0u, n_split, stream);
+  if (n_split > 0) launch_range<256, 256, 128, 64>(a16, a_scale, w, c, m, n, k, 0u, n_split, stream);
   if (n_split < n) launch_range<128, 64>(a16, a_scale, w, c, m, n, k, n_split, n, stream);
   return hipGetLastError();
 }

@@ -171,7 +171,20 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     nbytes = 2 * n * (k // 256) * 144 + 4 * k + 4 * 2 * n
     out["q4k_gemv_m1_gate_up_as_one_34816x5120"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                                                     "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-    del gu_list, w_gu, w_q1
+    del gu_list, w_gu
+
+    # ---- gate and up as the two GGUF tensors, one fused launch that ends in silu(g) * u (no
+    # concatenated copy, no separate activation launch, the M x 17408 intermediates never stored) ---
+    pairs = [(w_q1.clone(), w_q1.clone()) for _ in range(4)]
+    kffn = backend.LoadKernel("ffn_gate_up_silu_q4k")
+    y = torch.empty(n, dtype=torch.float32, device=dev)
+    launches = [(kffn, KernelLaunch(grid_x=(n + 7) // 8, buffers=[wrap(x), wrap(wg), wrap(wu), wrap(y)], scalars=[1, n, k]))
+                for wg, wu in pairs]
+    us = timed_us(launches, 20) / len(pairs)
+    nbytes = 2 * n * (k // 256) * 144 + 4 * k + 4 * n
+    out["q4k_ffn_gate_up_silu_m1_2x17408x5120"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                                   "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    del pairs, w_q1
 
     # ---- Q6_K and Q5_K (the other block formats of K-quant files), gate/up and down shapes --------
     for fmt, block_bytes, gen, rows in (("q6k", 210, synth.q6k_weights, (1, 2)), ("q5k", 176, synth.q5k_weights, (1,))):

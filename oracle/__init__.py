@@ -66,6 +66,7 @@ def _load() -> C.CDLL:
         "orc_fold_mxfp4_to_fp8": (C.c_int, [u8p, u8p, u8p, u8p, sz, sz]),
         "orc_gemm_mxfp4_fp8_ref": (C.c_int, [u8p, f32p, u8p, u8p, f32p, sz, sz, sz]),
         "orc_gemm_mxfp4_w4a8_ref": (C.c_int, [u8p, f32p, u8p, u8p, f32p, sz, sz, sz]),
+        "orc_silu_mul": (None, [f32p, f32p, f32p, sz]),
         "orc_moe_gate": (None, [f32p, f32p, sz]),
         "orc_top_k_row": (None, [f32p, sz, sz, u32p, f32p]),
         "orc_moe_expert_forward_q4k": (C.c_int, [f32p, u8p, u8p, u8p, sz, sz, f32p]),
@@ -306,6 +307,22 @@ def gemm_mxfp4_w4a8(a8, a_scale, packed, m: int, n: int, k: int) -> np.ndarray:
                                         _p(blob, C.c_uint8), _p(s, C.c_uint8),
                                         _p(c, C.c_float), m, n, k))
     return c
+
+
+# ---- dense feed-forward pieces ------------------------------------------------
+def silu_mul(g, u) -> np.ndarray:
+    g, u = _f32(g).reshape(-1), _f32(u).reshape(-1)
+    out = np.empty_like(g)
+    _lib.orc_silu_mul(_p(g, C.c_float), _p(u, C.c_float), _p(out, C.c_float), g.size)
+    return out
+
+
+def ffn_gate_up_silu_q4k(x, gate, up, m: int, n: int, k: int, threads: bool = False) -> np.ndarray:
+    """silu(x gate^T) * (x up^T): the two Q4_K products and silu_mul, composed as the
+    reference's dense feed-forward block does (src/models/qwen3_5/trunk.cpp:294-304)."""
+    g = gemm_q4k(x, gate, m, n, k, threads)
+    u = gemm_q4k(x, up, m, n, k, threads)
+    return silu_mul(g, u).reshape(m, n)
 
 
 # ---- MoE -------------------------------------------------------------------

@@ -29,6 +29,8 @@
  *                                             tie entries)
  *   MoE expert forward / gate ............... pinned (composition of pinned parts; softmax
  *                                             vs torch)
+ *   silu_mul ................................ pinned (float64 evaluation within 2 ulp, silu(0) = 0,
+ *                                             silu(x) - silu(-x) = x, large |x| limits)
  *
  * Status codes mirror tessera::StatusCode (include/tessera/types.hpp:36-48).
  */
@@ -645,6 +647,15 @@ void orc_top_k_row(const float* logits, size_t n, size_t top_k, uint32_t* ids, f
     }
     ids[p] = (uint32_t)best;
     vals[p] = logits[best];
+  }
+}
+
+/* ---- o = silu(g) * u elementwise (src/core/numerics/norm.cpp:211-226; the device kernel
+ *      src/backends/rocm/rocm_kernels_basic.cpp:1882-1891 is the same expression) ---- */
+void orc_silu_mul(const float* g, const float* u, float* o, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    const float silu = g[i] / (1.0f + expf(-g[i]));
+    o[i] = silu * u[i];
   }
 }
 

@@ -30,6 +30,26 @@ __global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ dst, 
   if (i < count) dst[i] = value;
 }
 
+// "silu_mul": o = silu(g) * u elementwise, the reference's expression
+// (src/backends/rocm/rocm_kernels_basic.cpp:1882-1891).  o may alias g or u.
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* g, const float* u, float* o, uint64_t n) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float gate = g[i];
+  o[i] = (gate / (1.0f + expf(-gate))) * u[i];
+}
+
+// "round_bf16": every fp32 value rounded in place to bfloat16 precision, nearest even, by the
+// reference's integer arithmetic on the bits (src/backends/rocm/rocm_kernels_basic.cpp:885-899;
+// NaN payloads and infinities go through the same add, as there).
+__global__ __launch_bounds__(256) void round_bf16_kernel(uint32_t* __restrict__ x, uint64_t n) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  uint32_t bits = x[i];
+  bits += 0x7FFFu + ((bits >> 16) & 1u);
+  x[i] = bits & 0xFFFF0000u;
+}
+
 // Workgroup-wide max of non-negative values; every thread returns it.
 __device__ __forceinline__ float block_max_256(float v, float* lds) {
   v = wave_max(v);
@@ -350,6 +370,18 @@ hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64
 hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
   hipLaunchKernelGGL(fill_f32_kernel, grid_for(count, 256), dim3(256), 0, stream, dst, value, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(const float* g, const float* u, float* o, uint64_t n, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(silu_mul_kernel, grid_for(n, 256), dim3(256), 0, stream, g, u, o, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(round_bf16_kernel, grid_for(n, 256), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(x), n);
   return hipGetLastError();
 }
 

@@ -419,6 +419,48 @@ struct Q4KPairCodec {
   }
 };
 
+// Gate and up projection of a dense feed-forward block in one pass, ending in
+// silu(G x) * (U x) (the dense analogue of the routed-expert gate/up pass above; the
+// reference runs two GEMVs and the "silu_mul" kernel, src/backends/rocm/rocm_kernels_basic.cpp:1882-1891).
+// The P rows a workgroup lays side by side are P/2 rows of the gate matrix interleaved with
+// the same P/2 rows of the up matrix (slot row p: matrix p & 1, row p / 2), so both dot
+// products of an output element are reduced in the same round and the thread that stores it
+// has both.  The activations are loaded once for the two matrices.
+struct Q4KGateUpCodec : Q4KPairCodec {
+  static constexpr bool kPairRows = true;
+  struct Args {
+    const float* a;
+    const uint8_t* w;      // gate
+    uint32_t k;
+    const uint8_t* up;
+  };
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    Q4KPairCodec::load_x<R>(Q4KPairCodec::Args{p.a, p.w, p.k}, chunk, valid, x, src);
+  }
+  // Bit 0 of off0 (offsets are multiples of 16) carries the matrix of this lane's slot row.
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
+                                                   uint32_t prow) {
+    const uint32_t hdr = (prow >> 1) * (cpr >> 2) * 144u + (chunk >> 2) * 144u;
+    return Lane{hdr | (prow & 1u), hdr + 16u + (chunk & 3u) * 32u};
+  }
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
+                                              uint32_t cpr, Frag& f) {
+    const uint8_t* base = ((ln.off0 & 1u) ? p.up : p.w) + static_cast<size_t>(row) * ((cpr >> 2) * 144u);
+    f.h = load_u4(base + (ln.off0 & ~1u));
+    f.q0 = load_u4(base + ln.off1);
+    f.q1 = load_u4(base + ln.off1 + 16u);
+  }
+  static __device__ __forceinline__ float combine(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
+};
+
+// Whether a codec interleaves two matrices over the slot rows of a group (see Q4KGateUpCodec).
+template <class Codec, class = void>
+struct pair_rows : std::false_type {};
+template <class Codec>
+struct pair_rows<Codec, std::void_t<decltype(Codec::kPairRows)>> : std::bool_constant<Codec::kPairRows> {};
+
 // ----------------------------------------------------------------------------
 // Q5_K: 176-byte super-block = fp16 d, fp16 dmin, 12 bytes of 6-bit scales/mins (packed as in
 // Q4_K), qh[32] fifth bits, qs[128] low nibbles; value = d*sc*(nibble + 16*bit) - dmin*mn
@@ -1015,16 +1057,22 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // last group for the loads (a prefetch must not pull the next workgroup's rows, which would
   // come from HBM a second time through another XCD's L2) and dropped at the store; rows past
   // n inside the last group re-read the group's first row.
-  const uint32_t groups = (n + P - 1) / P;
+  // PR = output rows per group; a paired codec spends two slot rows (one per matrix) on each.
+  constexpr bool kPaired = pair_rows<Codec>::value;
+  constexpr uint32_t PR = kPaired ? P / 2 : P;
+  static_assert(!kPaired || P % 2 == 0, "a paired codec needs an even number of slot rows");
+  const uint32_t groups = (n + PR - 1) / PR;
   const uint32_t g0 = blockIdx.x * groups_per_wg;
   const uint32_t g1 = g0 + groups_per_wg < groups ? g0 + groups_per_wg : groups;
   const Lane ln = Codec::make_lane(args, cpr, chunk, prow);
-  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, (groups - 1u) * P + prow < n ? prow : 0u);
-  const bool ragged = n % P != 0;
+  const uint32_t prow_out = kPaired ? prow >> 1 : prow;      // output row inside the group
+  const uint32_t prow_first = kPaired ? prow & 1u : 0u;      // slot row of the group's first row, same matrix
+  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, (groups - 1u) * PR + prow_out < n ? prow : prow_first);
+  const bool ragged = n % PR != 0;
   auto fetch = [&](uint32_t grp, typename Codec::Frag& f) {
     grp = grp < g1 ? grp : g1 - 1u;
     const bool tail = ragged && grp == groups - 1u;
-    Codec::load(args, tail ? ln_tail : ln, grp * P, cpr, f);
+    Codec::load(args, tail ? ln_tail : ln, grp * PR, cpr, f);
   };
 
   typename Codec::Frag frag[D];
@@ -1110,14 +1158,21 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       }
     }
     lds_barrier();  // LDS only: the prefetched global loads stay in flight across it
-    if (t < D * P * R) {
-      const uint32_t d = t / (P * R), p = (t / R) % P, r = t % R;
-      const uint32_t row = (g + d) * P + p;
+    if (t < D * PR * R) {
+      const uint32_t d = t / (PR * R), po = (t / R) % PR, r = t % R;
+      const uint32_t row = (g + d) * PR + po;
       if (g + d < g1 && row < n) {
-        const uint32_t w_lo = (p * cpr) >> 6, w_hi = ((p + 1u) * cpr - 1u) >> 6;
-        float sum = 0.0f;
-        for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][d][p][r][w];
-        c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, sum);
+        auto slot_sum = [&](uint32_t p) {
+          const uint32_t w_lo = (p * cpr) >> 6, w_hi = ((p + 1u) * cpr - 1u) >> 6;
+          float sum = 0.0f;
+          for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][d][p][r][w];
+          return sum;
+        };
+        if constexpr (kPaired) {
+          c[static_cast<size_t>(r) * ldc + row] = Codec::combine(slot_sum(2u * po), slot_sum(2u * po + 1u));
+        } else {
+          c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, slot_sum(po));
+        }
       }
     }
     buf ^= 1u;
@@ -1192,8 +1247,20 @@ int g_tune_p = 0;  // QMM_GEMV_P: force rows per group (experiments only)
 // to whole wavefronts; picks the P that idles the fewest lanes, larger P on ties
 // (fewer, fuller workgroups share one copy of the activations).
 template <uint32_t kMaxP>
-GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads) {
+GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads, bool even_p = false) {
   GemvPlan g{cpr, 0, 1, false};
+  if (even_p) {
+    // paired codecs: the largest even P that fits, preferring full wavefronts
+    if (cpr < 64) return g;   // p stays 1: the caller rejects it
+    double best = 0.0;
+    for (uint32_t p = 2; p <= kMaxP; p += 2) {
+      const uint32_t t = (p * cpr + 63u) / 64u * 64u;
+      if (t > max_threads) break;
+      const double fill = static_cast<double>(p * cpr) / t;
+      if (fill >= best) best = fill, g.p = p, g.threads = t;
+    }
+    return g;
+  }
   if (cpr == 4 || cpr == 8 || cpr == 16 || cpr == 32) {
     g.smallk = true;
     g.threads = 256;
@@ -1225,7 +1292,8 @@ hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n,
   const uint32_t waves_per_simd = (MAXT / 64u + 3u) / 4u;
   uint32_t per_cu = (4u * waves_per_simd) / waves;
   if (per_cu == 0) per_cu = 1;
-  const uint32_t groups = (n + P - 1) / P;
+  constexpr uint32_t PR = pair_rows<Codec>::value ? P / 2 : P;
+  const uint32_t groups = (n + PR - 1) / PR;
   uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu;
   if (grid > groups) grid = groups;
   uint32_t per_wg = (groups + grid - 1) / grid;
@@ -1250,23 +1318,26 @@ template <class Codec, int R, int MAXT, int D, uint32_t kMaxP = 2>
 hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n, uint32_t k,
                          uint32_t ldc, hipStream_t stream) {
   const uint32_t cpr = Codec::chunks_per_row(k);
-  const GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT);
-  if (g.smallk) {
-    constexpr int U = D > 4 ? 4 : D;
-    const uint32_t rows_per_wave = 64u / cpr;
-    const uint32_t groups = (n + rows_per_wave - 1) / rows_per_wave;
-    uint32_t grid = (groups + 4u * U - 1) / (4u * U);
-    const uint32_t cap = static_cast<uint32_t>(g_num_cus) * 8u;
-    grid = grid > cap ? cap : (grid == 0 ? 1 : grid);
-    hipLaunchKernelGGL((gemv_smallk_kernel<Codec, R, U>), dim3(grid), dim3(256), 0, stream, args, c,
-                       n, cpr, ldc);
-    return hipGetLastError();
+  const GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT, pair_rows<Codec>::value);
+  if (pair_rows<Codec>::value && (g.p % 2u != 0 || g.smallk)) return hipErrorInvalidValue;
+  if constexpr (!pair_rows<Codec>::value) {
+    if (g.smallk) {
+      constexpr int U = D > 4 ? 4 : D;
+      const uint32_t rows_per_wave = 64u / cpr;
+      const uint32_t groups = (n + rows_per_wave - 1) / rows_per_wave;
+      uint32_t grid = (groups + 4u * U - 1) / (4u * U);
+      const uint32_t cap = static_cast<uint32_t>(g_num_cus) * 8u;
+      grid = grid > cap ? cap : (grid == 0 ? 1 : grid);
+      hipLaunchKernelGGL((gemv_smallk_kernel<Codec, R, U>), dim3(grid), dim3(256), 0, stream, args, c,
+                         n, cpr, ldc);
+      return hipGetLastError();
+    }
   }
   if (g.threads > MAXT) return hipErrorInvalidValue;
   switch (g.p) {
 #define QMM_GEMV_CASE(PP)                                                                       \
   case PP:                                                                                      \
-    if constexpr (kMaxP >= PP)                                                                  \
+    if constexpr (kMaxP >= PP && (!pair_rows<Codec>::value || PP % 2 == 0))                     \
       return launch_gemv_p<Codec, R, MAXT, D, PP>(args, c, n, cpr, ldc, g.threads, stream);     \
     break;
     QMM_GEMV_CASE(1) QMM_GEMV_CASE(2) QMM_GEMV_CASE(3) QMM_GEMV_CASE(4) QMM_GEMV_CASE(5) QMM_GEMV_CASE(6)
@@ -1361,6 +1432,16 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     r0 += took;
   }
   return hipSuccess;
+}
+
+// silu(G x) * (U x) for one activation row, one launch: a row of 64 to 384 chunks of 64 weights
+// (two slot rows of it must fit a 768-thread workgroup and a wavefront may span two rows at most).
+bool ffn_gate_up_q4k_supported(uint64_t k) { return k % 256 == 0 && k >= 4096 && k <= 24576; }
+
+hipError_t launch_ffn_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up, float* out,
+                                  uint32_t n, uint32_t k, hipStream_t stream) {
+  Q4KGateUpCodec::Args args{x, gate, k, up};
+  return launch_gemv_r<Q4KGateUpCodec, 1, 768, 3, 8>(args, out, n, k, n, stream);
 }
 
 // Q5_K: one row per weight pass (a lane keeps 64 activations and five 16-byte loads per stage).

@@ -193,6 +193,62 @@ qmm_status run_vec_reduce(const LaunchCtx& c) {
   return map_hip(qmm::launch_vec_reduce(c.ptr<const float>(0), c.ptr<float>(1), total, split, c.stream));
 }
 
+// "silu_mul": buffers G, U, O (fp32, n each); scalar n.  O = silu(G) * U
+// (include/tessera/backend.hpp:257-259,618-625).
+qmm_status run_silu_mul(const LaunchCtx& c) {
+  if (!counts(c, 3, 1)) return bad("silu_mul: expects 3 buffers and 1 scalar");
+  const uint64_t n = c.sc[0];
+  if (n == 0 || n > (1ull << 40)) return bad("silu_mul: n must be non-zero");
+  const u128 bytes = static_cast<u128>(n) * 4;
+  if (!c.fits(0, bytes) || !c.fits(1, bytes) || !c.fits(2, bytes)) return bad("silu_mul: a buffer is smaller than n requires");
+  return map_hip(qmm::launch_silu_mul(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<float>(2), n, c.stream));
+}
+
+// "round_bf16": buffer 0 is the fp32 data rounded in place to bfloat16 precision; scalar n
+// (include/tessera/backend.hpp:337-339,740-747; src/models/qwen3_5/project.cpp:351-364).
+qmm_status run_round_bf16(const LaunchCtx& c) {
+  if (!counts(c, 1, 1)) return bad("round_bf16: expects 1 buffer and 1 scalar");
+  const uint64_t n = c.sc[0];
+  if (n == 0 || n > (1ull << 40)) return bad("round_bf16: n must be non-zero");
+  if (!c.fits(0, static_cast<u128>(n) * 4)) return bad("round_bf16: the buffer is smaller than n requires");
+  return map_hip(qmm::launch_round_bf16(c.ptr<float>(0), n, c.stream));
+}
+
+// "ffn_gate_up_silu_q4k" (not a reference id; the dense analogue of "moe_experts_gate_up_q4k"):
+// buffers X (fp32 m x k), Gate, Up (Q4_K, n rows of k each), Out (fp32 m x n); scalars m, n, k.
+// Out = silu(X Gate^T) * (X Up^T), what the reference computes with two "gemm_q4k*" launches
+// and "silu_mul" (src/models/qwen3_5/trunk.cpp:294-304).  One row of a supported k is a single launch that
+// reads the activations once for both matrices; anything else runs the two products through the
+// Q4_K regimes above (the up product into library scratch) and multiplies.
+qmm_status run_ffn_gate_up_silu_q4k(const LaunchCtx& c) {
+  if (!counts(c, 4, 3)) return bad("ffn_gate_up_silu_q4k: expects 4 buffers and 3 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
+  if (!dims_ok(m, n, k) || k % 256 != 0) return bad("ffn_gate_up_silu_q4k: m, n, k must be non-zero and k a multiple of 256");
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, q4k_bytes(n, k)) || !c.fits(2, q4k_bytes(n, k)) ||
+      !c.fits(3, static_cast<u128>(m) * n * 4)) {
+    return bad("ffn_gate_up_silu_q4k: a buffer is smaller than m, n, k require");
+  }
+  const float* x = c.ptr<const float>(0);
+  const uint8_t* gate = c.ptr<const uint8_t>(1);
+  const uint8_t* up = c.ptr<const uint8_t>(2);
+  float* out = c.ptr<float>(3);
+  if (m == 1 && qmm::ffn_gate_up_q4k_supported(k)) {
+    return map_hip(qmm::launch_ffn_gate_up_q4k(x, gate, up, out, static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
+  }
+  // The up product goes behind whatever the Q4_K GEMM keeps at the start of the workspace; a
+  // request for that smaller size returns the same base, so the two do not overlap.
+  const size_t gemm_ws = (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
+  const size_t up_off = (gemm_ws + 255) & ~size_t{255};
+  void* ws = nullptr;
+  qmm_status st = workspace(up_off + static_cast<size_t>(m) * n * 4, &ws);
+  if (st != QMM_OK) return st;
+  float* u = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + up_off);
+  st = q4k_matmul(x, gate, out, m, n, k, c.stream);
+  if (st == QMM_OK) st = q4k_matmul(x, up, u, m, n, k, c.stream);
+  if (st == QMM_OK) st = map_hip(qmm::launch_silu_mul(out, u, out, m * n, c.stream));
+  return st;
+}
+
 // "dequant_q4k" (not a reference id): buffers W, Out (fp32); scalar nblocks.
 qmm_status run_dequant_q4k(const LaunchCtx& c) {
   if (!counts(c, 2, 1)) return bad("dequant_q4k: expects 2 buffers and 1 scalar");
@@ -646,6 +702,9 @@ const Entry kTable[] = {
     {"gemm_q4k_rows4", run_gemm_q4k_rows4},
     {"gemm_q4k_rows5", run_gemm_q4k_rows5},
     {"gemm_vec_reduce", run_vec_reduce},
+    {"silu_mul", run_silu_mul},
+    {"round_bf16", run_round_bf16},
+    {"ffn_gate_up_silu_q4k", run_ffn_gate_up_silu_q4k},
     {"gemm_mxfp4", run_gemm_mxfp4},
     {"gemm_mxfp4_rows", run_gemm_mxfp4_rows},
     {"gemm_mxfp4_batched", run_gemm_mxfp4},

@@ -97,6 +97,14 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
 hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64_t split,
                              hipStream_t stream);
 hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream);
+hipError_t launch_silu_mul(const float* g, const float* u, float* o, uint64_t n, hipStream_t stream);
+hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
+
+// Dense feed-forward gate and up projections with the activation fused, one activation row:
+// out[j] = silu(G x)[j] * (U x)[j], both matrices n rows of Q4_K.
+bool ffn_gate_up_q4k_supported(uint64_t k);
+hipError_t launch_ffn_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up, float* out,
+                                  uint32_t n, uint32_t k, hipStream_t stream);
 hipError_t launch_quantize_fp8(float* data, float* scale, uint64_t rows, uint64_t cols,
                                hipStream_t stream);
 hipError_t launch_quantize_fp8_pack(const float* in, uint8_t* out, float* scale, uint64_t rows,

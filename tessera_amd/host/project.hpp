@@ -44,6 +44,8 @@ struct ProjectState {
   // The reference splits K to fill a 96-CU card; this backend takes any split (it writes the
   // whole result to region 0) but gains nothing from it, so the default passes split = 1.
   bool honour_reference_split = false;
+  // Take the reference's three launches for the dense gate/up/silu even where the fused id exists.
+  bool no_fused_ffn = false;
 };
 
 inline Expected<const Kernel*> CachedKernel(Backend& backend, ProjectState& h, const std::string& id) {
@@ -188,6 +190,37 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
     return ProjectGemvDevice(backend, h, **vec, a, w, out, m, n, k);
   }
   return unexpected(StatusCode::UnsupportedFeature);
+}
+
+// Front half of the dense feed-forward block: mlp = silu(xn Gate^T) * (xn Up^T)
+// (src/models/qwen3_5/trunk.cpp:294-304: ProjectBatch for gate, ProjectBatch for up,
+// SiluMulDevice).  When both tensors are Q4_K the backend's fused id does it in one launch;
+// a backend without the id (UnsupportedFeature) or other formats take the reference's three
+// launches, with `gate_out` and `up_out` as the intermediates the reference keeps in h.fgate/h.fup.
+inline Expected<void> FfnGateUpSilu(Backend& backend, ProjectState& h, DType gate_dtype, DType up_dtype,
+                                    const Buffer& xn, const Buffer& gate, const Buffer& up, Buffer& gate_out,
+                                    Buffer& up_out, Buffer& mlp, std::size_t m, std::size_t n, std::size_t k) {
+  if (m == 0 || n == 0 || k == 0) return unexpected(StatusCode::InvalidArgument);
+  if (gate_dtype == DType::Q4K && up_dtype == DType::Q4K && !h.no_fused_ffn) {
+    auto fused = CachedKernel(backend, h, "ffn_gate_up_silu_q4k");
+    if (fused) {
+      KernelLaunch l;
+      l.grid_x = static_cast<std::uint32_t>((m * n + 7) / 8);
+      l.buffers = {&xn, &gate, &up, &mlp};
+      l.scalars = {m, n, k};
+      return backend.LaunchKernel(**fused, l);
+    }
+    if (fused.error() != StatusCode::UnsupportedFeature) return unexpected(fused.error());
+  }
+  if (auto st = ProjectBatch(backend, h, gate_dtype, xn, gate, gate_out, m, n, k); !st) return st;
+  if (auto st = ProjectBatch(backend, h, up_dtype, xn, up, up_out, m, n, k); !st) return st;
+  auto silu = CachedKernel(backend, h, "silu_mul");
+  if (!silu) return unexpected(silu.error());
+  KernelLaunch l;
+  l.grid_x = static_cast<std::uint32_t>((m * n + 255) / 256);     // src/core/decode_internal.hpp:976-986
+  l.buffers = {&gate_out, &up_out, &mlp};
+  l.scalars = {m * n};
+  return backend.LaunchKernel(**silu, l);
 }
 
 }  // namespace tessera_amd

@@ -16,6 +16,7 @@ int orc_gemm_q5k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_
 int orc_gemm_q6k_ref(const float* a, const uint8_t* w, float* c, size_t m, size_t n, size_t k, int threads);
 int orc_gemm_mxfp4_ref(const float* a, const uint8_t* w, const uint8_t* s, float* c, size_t m, size_t n, size_t k);
 int orc_quantize_fp8_ref(float* data, float* scale, size_t rows, size_t cols);
+void orc_silu_mul(const float* g, const float* u, float* o, size_t n);
 }
 
 using namespace tessera_amd;
@@ -111,11 +112,55 @@ const Case kCases[] = {
     {"mxfp4 w4a8 m=300 (tiled scaled MFMA)", DType::F4E2M1, 300, 384, 1024, false, 1e-2, 5e-4},
 };
 
+// Front half of the dense feed-forward block through FfnGateUpSilu, fused id or three launches.
+struct FfnCase {
+  const char* name;
+  size_t m, n, k;
+  bool three_launches;
+  double rel_tol;
+};
+const FfnCase kFfnCases[] = {
+    {"ffn gate/up/silu m=1 (ffn_gate_up_silu_q4k, one launch)", 1, 1027, 5120, false, 1e-3},
+    {"ffn gate/up/silu m=1, the reference's three launches", 1, 1027, 5120, true, 1e-3},
+    {"ffn gate/up/silu m=3 (fused id, composed inside the library)", 3, 200, 2048, false, 1e-3},
+};
+
+bool RunFfn(Backend& backend, const FfnCase& c) {
+  ProjectState h;
+  h.no_fused_ffn = c.three_launches;
+  const auto x = Activations(c.m, c.k);
+  const auto gate = Q4KWeights(c.n, c.k), up = Q4KWeights(c.n, c.k);
+  std::vector<float> g(c.m * c.n), u(c.m * c.n), ref(c.m * c.n), got(c.m * c.n);
+  orc_gemm_q4k_ref(x.data(), gate.data(), g.data(), c.m, c.n, c.k);
+  orc_gemm_q4k_ref(x.data(), up.data(), u.data(), c.m, c.n, c.k);
+  orc_silu_mul(g.data(), u.data(), ref.data(), ref.size());
+  auto dx = Upload(backend, x);
+  auto dg = Upload(backend, gate);
+  auto du = Upload(backend, up);
+  auto og = backend.AllocateBuffer(ref.size() * 4), ou = backend.AllocateBuffer(ref.size() * 4);
+  auto out = backend.AllocateBuffer(ref.size() * 4);
+  auto st = FfnGateUpSilu(backend, h, DType::Q4K, DType::Q4K, *dx, *dg, *du, **og, **ou, **out, c.m, c.n, c.k);
+  backend.Synchronize();
+  if (!st) {
+    std::printf("FAIL %s: status %d (%s)\n", c.name, static_cast<int>(st.error()), backend.LastError());
+    return false;
+  }
+  if (!backend.CopyD2H(**out, std::as_writable_bytes(std::span<float>(got)))) std::exit(3);
+  double rel, rms;
+  Errors(got, ref, rel, rms);
+  const bool launches_ok = (h.kernels.count("ffn_gate_up_silu_q4k") == 1) != c.three_launches;
+  const bool ok = rel <= c.rel_tol && launches_ok;
+  std::printf("%s %s: rel %.2e (<= %.0e)%s\n", ok ? "ok  " : "FAIL", c.name, rel, c.rel_tol,
+              launches_ok ? "" : " [wrong launch sequence]");
+  return ok;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
   if (argc > 1 && std::strcmp(argv[1], "--list") == 0) {
     for (const Case& c : kCases) std::printf("%s\n", c.name);
+    for (const FfnCase& c : kFfnCases) std::printf("%s\n", c.name);
     return 0;
   }
   auto backend = CreateBackend();
@@ -176,5 +221,6 @@ int main(int argc, char** argv) {
     std::printf("%s %s: rel %.2e (<= %.0e) rms %.2e (<= %.0e)\n", ok ? "ok  " : "FAIL", c.name, rel, c.rel_tol, rms, c.rms_tol);
     failed += ok ? 0 : 1;
   }
+  for (const FfnCase& c : kFfnCases) failed += RunFfn(*backend, c) ? 0 : 1;
   return failed == 0 ? 0 : 1;
 }

@@ -1470,7 +1470,10 @@ hipError_t launch_q6k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     hipError_t e;
     uint32_t took;
     if (m - r0 >= 2 && row_threads <= 512u) {
-      e = launch_gemv_r<Q6KCodec, 2, 512, 2, 6>(args, out, n, k, n, stream), took = 2;
+      // One fragment in flight per lane: with two, the 256 registers of a 512-thread workgroup
+      // spill a few values, and a kernel with a scratch segment takes microseconds longer to
+      // dispatch (two rows of 17408 x 5120: 38 us with depth 2, 29 us with depth 1).
+      e = launch_gemv_r<Q6KCodec, 2, 512, 1, 6>(args, out, n, k, n, stream), took = 2;
     } else {
       e = launch_gemv_r<Q6KCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
     }

@@ -200,24 +200,26 @@ struct Q4KCodec {
 // kernel.  `batch` moves every per-token pointer to token y (grid.y).
 // ----------------------------------------------------------------------------
 
-// Gate or up projection of the `top_k` selected experts: output row slot*inter + j is row j
-// of expert ids[slot].  With `gate_out` set this is the up pass and the stored value is
-// silu(gate_out[row]) * (U x)[row]: the gate pass wrote gate_out, so two launches leave phi.
-struct Q4KExpertUpCodec : Q4KCodec {
+// Gate and up of the `top_k` selected experts in one pass: output row slot*inter + j is row j of
+// expert ids[slot]; a wavefront loads its activations once, takes that row of both tensors and
+// stores silu(G x) * (U x) (the reference's single "moe_experts_gate_up_q4k" launch,
+// src/backends/rocm/rocm_kernels_moe.cpp:15-49).
+struct Q4KExpertGateUpCodec : Q4KCodec {
+  static constexpr bool kTwoMatrices = true;
   struct Args {
     const float* a;
-    const uint8_t* w;
+    const uint8_t* w;      // gate
     uint32_t k;            // hidden
     const uint32_t* ids;
-    uint64_t stride;
+    uint64_t stride;       // gate expert stride
     uint32_t inter, top_k;
-    uint32_t n_experts;    // ids are clamped below this, so a bad id cannot leave the tensor
-    const float* gate_out;
+    uint32_t n_experts;
+    const uint8_t* up;
+    uint64_t up_stride;
   };
   static __device__ __forceinline__ void batch(Args& p, uint32_t y) {
     p.a += static_cast<size_t>(y) * p.k;
     p.ids += static_cast<size_t>(y) * p.top_k;
-    if (p.gate_out != nullptr) p.gate_out += static_cast<size_t>(y) * p.top_k * p.inter;
   }
   template <int R, class Src>
   static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
@@ -227,20 +229,17 @@ struct Q4KExpertUpCodec : Q4KCodec {
   static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk, uint32_t prow) {
     return Q4KCodec::make_lane(Q4KCodec::Args{}, cpr, chunk, prow);
   }
+  // which = 0: gate, 1: up
   static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row, uint32_t cpr,
-                                              Frag& f) {
+                                              Frag& f, int which = 0) {
     const uint32_t slot = row / p.inter, j = row - slot * p.inter;
     const uint32_t e = p.ids[slot] < p.n_experts ? p.ids[slot] : p.n_experts - 1u;
-    const uint8_t* base = p.w + e * p.stride + static_cast<size_t>(j) * ((cpr >> 3) * 144u);
+    const uint8_t* base = (which ? p.up + e * p.up_stride : p.w + e * p.stride) +
+                          static_cast<size_t>(j) * ((cpr >> 3) * 144u);
     f.h = load_u4(base + ln.off0);
     f.q = load_u4(base + ln.off1);
   }
-  template <int R>
-  static __device__ __forceinline__ float finish(const Args& p, uint32_t row, int, float v) {
-    if (p.gate_out == nullptr) return v;
-    const float g = p.gate_out[row];
-    return (g / (1.0f + expf(-g))) * v;
-  }
+  static __device__ __forceinline__ float combine(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
 };
 
 // Down projection of the selected experts, summed with the routing weights:
@@ -1363,22 +1362,36 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args 
     Codec::batch(args, blockIdx.y);
     c += static_cast<size_t>(blockIdx.y) * ldc;
   }
-  float acc = 0.0f;
+  // A codec over two matrices (kTwoMatrices) takes the same row of both against one copy of the
+  // activations and stores combine(first, second).
+  constexpr bool kTwo = requires { Codec::kTwoMatrices; };
+  float acc = 0.0f, acc2 = 0.0f;
   for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
     typename Codec::template X<1> x;
-    typename Codec::Frag f;
+    typename Codec::Frag f, f2;
+    const Lane ln = Codec::make_lane(args, cpr, chunk, 0u);
+    Codec::load(args, ln, row, cpr, f);
+    if constexpr (kTwo) Codec::load(args, ln, row, cpr, f2, 1);
     if constexpr (Codec::kStageX) {
       Codec::template load_x<1>(args, chunk, true, x, GlobalX{args.a, args.k});
     } else {
       Codec::template load_x<1>(args, chunk, true, x, 0);
     }
-    Codec::load(args, Codec::make_lane(args, cpr, chunk, 0u), row, cpr, f);
     float v[1];
     Codec::template dot<1>(f, x, v);
     acc += v[0];
+    if constexpr (kTwo) {
+      Codec::template dot<1>(f2, x, v);
+      acc2 += v[0];
+    }
   }
   acc = wave_sum(acc);
-  if (lane == 0) c[row] = Codec::template finish<1>(args, row, 0, acc);
+  if constexpr (kTwo) {
+    acc2 = wave_sum(acc2);
+    if (lane == 0) c[row] = Codec::combine(acc, acc2);
+  } else {
+    if (lane == 0) c[row] = Codec::template finish<1>(args, row, 0, acc);
+  }
   (void)ldc;
 }
 
@@ -1560,10 +1573,8 @@ hipError_t launch_moe_gate_up_q4k(const float* x, const uint8_t* gate, const uin
                                   uint32_t n_experts, uint32_t rows, hipStream_t stream) {
   const uint32_t n = top_k * inter, cpr = Q4KCodec::chunks_per_row(hidden);
   const dim3 grid((n + 3u) / 4u, rows);
-  Q4KExpertUpCodec::Args g{x, gate, hidden, ids, gate_stride, inter, top_k, n_experts, nullptr};
-  hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertUpCodec>), grid, dim3(256), 0, stream, g, phi, n, cpr, n);
-  Q4KExpertUpCodec::Args u{x, up, hidden, ids, up_stride, inter, top_k, n_experts, phi};
-  hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertUpCodec>), grid, dim3(256), 0, stream, u, phi, n, cpr, n);
+  Q4KExpertGateUpCodec::Args a{x, gate, hidden, ids, gate_stride, inter, top_k, n_experts, up, up_stride};
+  hipLaunchKernelGGL((gemv_generic_kernel<Q4KExpertGateUpCodec>), grid, dim3(256), 0, stream, a, phi, n, cpr, n);
   return hipGetLastError();
 }
 

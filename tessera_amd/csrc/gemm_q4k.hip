@@ -352,7 +352,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void q4k_gemm_kernel(
 template <int BM, int BN>
 __global__ __launch_bounds__(BN * 2) void q4k_gemm_grouped_kernel(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
-    float* __restrict__ c, const uint32_t* __restrict__ seg, uint64_t w_stride, uint32_t n, uint32_t k) {
+    float* __restrict__ c, const uint32_t* __restrict__ seg, uint64_t w_stride, uint32_t n, uint32_t k,
+    const uint8_t* __restrict__ w2, float* __restrict__ c2, uint64_t w2_stride) {
+  // grid.z = 2 runs a second expert tensor of the same shape against the same rows (gate and up
+  // in one launch: twice the workgroups to fill the tail of the first with).
+  if (blockIdx.z == 1) w = w2, c = c2, w_stride = w2_stride;
   // Expert on grid.x: workgroups are dealt to the eight XCDs by linear index, so with the
   // expert varying fastest all column tiles of an expert land on one XCD and its activation
   // rows are fetched into one L2 instead of eight.
@@ -769,13 +773,11 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
   hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, seg, pos);
   hipLaunchKernelGGL(rows_to_f16_kernel, dim3(pairs), dim3(256), 0, stream, x, a16, x_scale, hidden, pos, top_k);
   constexpr int BM = 32, BN = 64;
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (inter + BN - 1) / BN), dim3(BN * 2), 0, stream,
-                     a16, x_scale, gate, g, seg, gate_stride, inter, hidden);
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (inter + BN - 1) / BN), dim3(BN * 2), 0, stream,
-                     a16, x_scale, up, u, seg, up_stride, inter, hidden);
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (inter + BN - 1) / BN, 2), dim3(BN * 2), 0, stream,
+                     a16, x_scale, gate, g, seg, gate_stride, inter, hidden, up, u, up_stride);
   hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(pairs), dim3(256), 0, stream, g, u, phi16, phi_scale, inter);
   hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (hidden + BN - 1) / BN), dim3(BN * 2), 0, stream,
-                     phi16, phi_scale, down, rows, seg, down_stride, hidden, inter);
+                     phi16, phi_scale, down, rows, seg, down_stride, hidden, inter, nullptr, nullptr, uint64_t{0});
   const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, rows, pos,
                      wts, out, tokens, top_k, hidden, accumulate);

@@ -67,6 +67,8 @@ def _load() -> C.CDLL:
         "orc_gemm_mxfp4_fp8_ref": (C.c_int, [u8p, f32p, u8p, u8p, f32p, sz, sz, sz]),
         "orc_gemm_mxfp4_w4a8_ref": (C.c_int, [u8p, f32p, u8p, u8p, f32p, sz, sz, sz]),
         "orc_silu_mul": (None, [f32p, f32p, f32p, sz]),
+        "orc_rmsnorm": (C.c_int, [f32p, f32p, f32p, sz, sz, C.c_float]),
+        "orc_embedding": (C.c_int, [C.c_int, u32p, C.c_void_p, f32p, sz, sz, sz]),
         "orc_moe_gate": (None, [f32p, f32p, sz]),
         "orc_top_k_row": (None, [f32p, sz, sz, u32p, f32p]),
         "orc_moe_expert_forward_q4k": (C.c_int, [f32p, u8p, u8p, u8p, sz, sz, f32p]),
@@ -314,6 +316,24 @@ def silu_mul(g, u) -> np.ndarray:
     g, u = _f32(g).reshape(-1), _f32(u).reshape(-1)
     out = np.empty_like(g)
     _lib.orc_silu_mul(_p(g, C.c_float), _p(u, C.c_float), _p(out, C.c_float), g.size)
+    return out
+
+
+def rmsnorm(x, w, rows: int, cols: int, eps: float) -> np.ndarray:
+    x, w = _f32(x).reshape(-1), _f32(w).reshape(-1)
+    y = np.empty_like(x)
+    _check(_lib.orc_rmsnorm(_p(x, C.c_float), _p(w, C.c_float), _p(y, C.c_float), rows, cols, eps))
+    return y.reshape(rows, cols)
+
+
+def embedding(kind: str, ids, table, rows: int, cols: int, vocab: int) -> np.ndarray:
+    """kind: "f32", "bf16" (uint16 table) or "q4k" (uint8 blocks)."""
+    ids = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+    table = np.ascontiguousarray(table)
+    out = np.empty((rows, cols), dtype=np.float32)
+    code = {"f32": 0, "bf16": 1, "q4k": 2}[kind]
+    _check(_lib.orc_embedding(code, _p(ids, C.c_uint32), table.ctypes.data_as(C.c_void_p), _p(out, C.c_float),
+                              rows, cols, vocab))
     return out
 
 

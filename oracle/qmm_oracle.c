@@ -29,6 +29,10 @@
  *                                             tie entries)
  *   MoE expert forward / gate ............... pinned (composition of pinned parts; softmax
  *                                             vs torch)
+ *   rmsnorm ................................. pinned (float64 evaluation, scale invariance, unit
+ *                                             rows)
+ *   embedding gather ........................ pinned (composition of the pinned decoders with an
+ *                                             index; out-of-range ids give zero rows)
  *   silu_mul ................................ pinned (float64 evaluation within 2 ulp, silu(0) = 0,
  *                                             silu(x) - silu(-x) = x, large |x| limits)
  *
@@ -648,6 +652,44 @@ void orc_top_k_row(const float* logits, size_t n, size_t top_k, uint32_t* ids, f
     ids[p] = (uint32_t)best;
     vals[p] = logits[best];
   }
+}
+
+/* ---- y = x / sqrt(mean(x^2) + eps) * w per row, the sum of squares one sequential fma chain
+ *      (src/core/numerics/norm.cpp:7-32) ---- */
+int orc_rmsnorm(const float* x, const float* w, float* y, size_t rows, size_t cols, float eps) {
+  if (rows == 0 || cols == 0 || eps < 0.0f) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    const float* xr = x + r * cols;
+    float mean = 0.0f;
+    for (size_t c = 0; c < cols; ++c) mean = fmaf(xr[c], xr[c], mean);
+    mean /= (float)cols;
+    const float gain = 1.0f / sqrtf(mean + eps);
+    for (size_t c = 0; c < cols; ++c) y[r * cols + c] = xr[c] * gain * w[c];
+  }
+  return ORC_OK;
+}
+
+/* ---- out[row] = table[ids[row]], a zero row for an id outside the table; kind 0: fp32 table,
+ *      1: bf16 (the high half of the fp32 bits), 2: Q4_K rows
+ *      (src/backends/rocm/rocm_kernels_embedding.cpp:10-108) ---- */
+int orc_embedding(int kind, const uint32_t* ids, const void* table, float* out, size_t rows, size_t cols,
+                  size_t vocab) {
+  if (rows == 0 || cols == 0 || vocab == 0 || (kind == 2 && cols % 256 != 0)) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    float* o = out + r * cols;
+    const size_t id = ids[r];
+    if (id >= vocab) {
+      memset(o, 0, cols * sizeof(float));
+    } else if (kind == 0) {
+      memcpy(o, (const float*)table + id * cols, cols * sizeof(float));
+    } else if (kind == 1) {
+      const uint16_t* t = (const uint16_t*)table + id * cols;
+      for (size_t c = 0; c < cols; ++c) o[c] = bits_f32((uint32_t)t[c] << 16);
+    } else {
+      orc_dequantize_q4k_rows((const uint8_t*)table + id * (cols / 256) * 144, o, cols / 256);
+    }
+  }
+  return ORC_OK;
 }
 
 /* ---- o = silu(g) * u elementwise (src/core/numerics/norm.cpp:211-226; the device kernel

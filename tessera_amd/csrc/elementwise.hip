@@ -50,6 +50,80 @@ __global__ __launch_bounds__(256) void round_bf16_kernel(uint32_t* __restrict__ 
   x[i] = bits & 0xFFFF0000u;
 }
 
+// "add": o = a + b elementwise (src/backends/rocm/rocm_kernels_basic.cpp:1870-1880).
+__global__ __launch_bounds__(256) void add_kernel(const float* a, const float* b, float* o, uint64_t n) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) o[i] = a[i] + b[i];
+}
+
+// "fill": every int32 element set to the low 32 bits of the value
+// (src/backends/rocm/rocm_kernels_basic.cpp:10-19).
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ out, int32_t value, uint64_t n) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = value;
+}
+
+// "rmsnorm": y = x / sqrt(mean(x^2) + eps) * w per row, one workgroup per row
+// (src/backends/rocm/rocm_kernels_basic.cpp:1586-1616).  The sum of squares is a strided fma chain
+// per thread, a butterfly inside each wavefront and the four wavefront sums in order: the
+// reference's tree adds the same partials in another order, so results agree to rounding.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                      float* __restrict__ y, uint64_t cols, float eps) {
+  __shared__ float part[4];
+  const float* xr = x + static_cast<uint64_t>(blockIdx.x) * cols;
+  float* yr = y + static_cast<uint64_t>(blockIdx.x) * cols;
+  float sum = 0.0f;
+  for (uint64_t c = threadIdx.x; c < cols; c += 256u) sum = fmaf(xr[c], xr[c], sum);
+  sum = wave_sum(sum);
+  if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  const float mean = (((part[0] + part[1]) + part[2]) + part[3]) / static_cast<float>(cols);
+  const float gain = 1.0f / sqrtf(mean + eps);
+  for (uint64_t c = threadIdx.x; c < cols; c += 256u) yr[c] = xr[c] * gain * w[c];
+}
+
+// "embedding_f32" / "embedding_bf16" / "embedding_q4k": out[row] = table[ids[row]], a zero row for
+// an id outside the table (src/backends/rocm/rocm_kernels_embedding.cpp:15-108).  KIND 0: fp32
+// table, 1: bf16 (the high half of the fp32 bits), 2: Q4_K rows of cols/256 super-blocks, decoded
+// as (d*sc)*q - dmin*mn with exact products and one rounding.
+template <int KIND>
+__global__ __launch_bounds__(256) void embedding_kernel(const uint32_t* __restrict__ ids, const void* __restrict__ table,
+                                                        float* __restrict__ out, uint64_t rows, uint64_t cols,
+                                                        uint64_t vocab) {
+  const uint64_t g = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (g >= rows * cols) return;
+  const uint64_t row = g / cols, i = g % cols;
+  const uint64_t id = ids[row];
+  if (id >= vocab) {
+    out[g] = 0.0f;
+    return;
+  }
+  if constexpr (KIND == 0) {
+    out[g] = static_cast<const float*>(table)[id * cols + i];
+  } else if constexpr (KIND == 1) {
+    out[g] = bit_cast<float>(static_cast<uint32_t>(static_cast<const uint16_t*>(table)[id * cols + i]) << 16);
+  } else {
+    const uint64_t b = i / kQ4KBlockElems;
+    const uint32_t e = static_cast<uint32_t>(i % kQ4KBlockElems);
+    const uint8_t* base = static_cast<const uint8_t*>(table) + (id * (cols / kQ4KBlockElems) + b) * kQ4KBlockBytes;
+    const uint32_t grp = e / 64u, half = (e % 64u) / 32u, l = e % 32u, sb = 2u * grp + half;
+    const uint8_t* p = base + 4;
+    uint32_t sc, mn;
+    if (sb < 4) {
+      sc = p[sb] & 63u;
+      mn = p[sb + 4] & 63u;
+    } else {
+      sc = (p[sb + 4] & 15u) | ((p[sb - 4] >> 6) << 4);
+      mn = (p[sb + 4] >> 4) | ((p[sb] >> 6) << 4);
+    }
+    const float d = half_bits_to_float(base[0] | (static_cast<uint32_t>(base[1]) << 8));
+    const float dmin = half_bits_to_float(base[2] | (static_cast<uint32_t>(base[3]) << 8));
+    const uint32_t byte = base[16 + grp * 32u + l];
+    const uint32_t q = half ? byte >> 4 : byte & 15u;
+    out[g] = (d * static_cast<float>(sc)) * static_cast<float>(q) - dmin * static_cast<float>(mn);
+  }
+}
+
 // Workgroup-wide max of non-negative values; every thread returns it.
 __device__ __forceinline__ float block_max_256(float v, float* lds) {
   v = wave_max(v);
@@ -370,6 +444,36 @@ hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64
 hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
   hipLaunchKernelGGL(fill_f32_kernel, grid_for(count, 256), dim3(256), 0, stream, dst, value, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_add(const float* a, const float* b, float* o, uint64_t n, hipStream_t stream) {
+  hipLaunchKernelGGL(add_kernel, grid_for(n, 256), dim3(256), 0, stream, a, b, o, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_i32(int32_t* out, int32_t value, uint64_t n, hipStream_t stream) {
+  hipLaunchKernelGGL(fill_i32_kernel, grid_for(n, 256), dim3(256), 0, stream, out, value, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_rmsnorm(const float* x, const float* w, float* y, uint64_t rows, uint64_t cols, float eps,
+                          hipStream_t stream) {
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, w, y, cols, eps);
+  return hipGetLastError();
+}
+
+// kind 0: fp32 table, 1: bf16, 2: Q4_K
+hipError_t launch_embedding(int kind, const uint32_t* ids, const void* table, float* out, uint64_t rows,
+                            uint64_t cols, uint64_t vocab, hipStream_t stream) {
+  const dim3 grid = grid_for(rows * cols, 256);
+  if (kind == 0) {
+    hipLaunchKernelGGL(embedding_kernel<0>, grid, dim3(256), 0, stream, ids, table, out, rows, cols, vocab);
+  } else if (kind == 1) {
+    hipLaunchKernelGGL(embedding_kernel<1>, grid, dim3(256), 0, stream, ids, table, out, rows, cols, vocab);
+  } else {
+    hipLaunchKernelGGL(embedding_kernel<2>, grid, dim3(256), 0, stream, ids, table, out, rows, cols, vocab);
+  }
   return hipGetLastError();
 }
 

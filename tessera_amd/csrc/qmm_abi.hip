@@ -204,6 +204,63 @@ qmm_status run_silu_mul(const LaunchCtx& c) {
   return map_hip(qmm::launch_silu_mul(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<float>(2), n, c.stream));
 }
 
+// "add": buffers A, B, O (fp32, n each); scalar n (include/tessera/backend.hpp:255-256,618-625).
+qmm_status run_add(const LaunchCtx& c) {
+  if (!counts(c, 3, 1)) return bad("add: expects 3 buffers and 1 scalar");
+  const uint64_t n = c.sc[0];
+  if (n == 0 || n > (1ull << 40)) return bad("add: n must be non-zero");
+  const u128 bytes = static_cast<u128>(n) * 4;
+  if (!c.fits(0, bytes) || !c.fits(1, bytes) || !c.fits(2, bytes)) return bad("add: a buffer is smaller than n requires");
+  return map_hip(qmm::launch_add(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<float>(2), n, c.stream));
+}
+
+// "fill": buffer 0 is an int32 array; scalars value, count (include/tessera/backend.hpp:151-152,393-396).
+qmm_status run_fill(const LaunchCtx& c) {
+  if (!counts(c, 1, 2)) return bad("fill: expects 1 buffer and 2 scalars");
+  const uint64_t n = c.sc[1];
+  if (n > (1ull << 40) || !c.fits(0, static_cast<u128>(n) * 4)) return bad("fill: the buffer is smaller than the count requires");
+  if (n == 0) return QMM_OK;
+  return map_hip(qmm::launch_fill_i32(c.ptr<int32_t>(0), static_cast<int32_t>(c.sc[0]), n, c.stream));
+}
+
+// "rmsnorm": buffers X (rows x cols), W (cols), Y (rows x cols); scalars rows, cols, fp32 bits of
+// epsilon (include/tessera/backend.hpp:212-216,557-564).
+qmm_status run_rmsnorm(const LaunchCtx& c) {
+  if (!counts(c, 3, 3)) return bad("rmsnorm: expects 3 buffers and 3 scalars");
+  const uint64_t rows = c.sc[0], cols = c.sc[1];
+  if (rows == 0 || cols == 0 || rows > (1u << 30) || cols > (1ull << 32)) return bad("rmsnorm: rows and cols must be non-zero");
+  const u128 bytes = static_cast<u128>(rows) * cols * 4;
+  if (!c.fits(0, bytes) || !c.fits(1, static_cast<u128>(cols) * 4) || !c.fits(2, bytes)) {
+    return bad("rmsnorm: a buffer is smaller than rows, cols require");
+  }
+  const uint32_t eps_bits = static_cast<uint32_t>(c.sc[2]);
+  float eps;
+  std::memcpy(&eps, &eps_bits, 4);
+  return map_hip(qmm::launch_rmsnorm(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<float>(2), rows, cols, eps, c.stream));
+}
+
+// "embedding_f32", "embedding_bf16", "embedding_q4k": buffers ids (u32, rows), table (vocab x cols),
+// Out (fp32 rows x cols); scalars rows, cols, vocab (include/tessera/backend.hpp:260-265,827-839).
+qmm_status run_embedding(const LaunchCtx& c, int kind) {
+  if (!counts(c, 3, 3)) return bad("embedding: expects 3 buffers and 3 scalars");
+  const uint64_t rows = c.sc[0], cols = c.sc[1], vocab = c.sc[2];
+  if (rows == 0 || cols == 0 || vocab == 0 || rows > (1u << 30) || cols > (1u << 30) || vocab > (1u << 30)) {
+    return bad("embedding: rows, cols and vocab must be non-zero");
+  }
+  if (kind == 2 && cols % 256 != 0) return bad("embedding_q4k: cols must be a multiple of 256");
+  const u128 table = kind == 0 ? static_cast<u128>(vocab) * cols * 4
+                     : kind == 1 ? static_cast<u128>(vocab) * cols * 2
+                                 : static_cast<u128>(vocab) * (cols / 256) * 144;
+  if (!c.fits(0, static_cast<u128>(rows) * 4) || !c.fits(1, table) || !c.fits(2, static_cast<u128>(rows) * cols * 4)) {
+    return bad("embedding: a buffer is smaller than rows, cols, vocab require");
+  }
+  return map_hip(qmm::launch_embedding(kind, c.ptr<const uint32_t>(0), c.ptr<const void>(1), c.ptr<float>(2), rows, cols,
+                                       vocab, c.stream));
+}
+qmm_status run_embedding_f32(const LaunchCtx& c) { return run_embedding(c, 0); }
+qmm_status run_embedding_bf16(const LaunchCtx& c) { return run_embedding(c, 1); }
+qmm_status run_embedding_q4k(const LaunchCtx& c) { return run_embedding(c, 2); }
+
 // "round_bf16": buffer 0 is the fp32 data rounded in place to bfloat16 precision; scalar n
 // (include/tessera/backend.hpp:337-339,740-747; src/models/qwen3_5/project.cpp:351-364).
 qmm_status run_round_bf16(const LaunchCtx& c) {
@@ -703,6 +760,12 @@ const Entry kTable[] = {
     {"gemm_q4k_rows5", run_gemm_q4k_rows5},
     {"gemm_vec_reduce", run_vec_reduce},
     {"silu_mul", run_silu_mul},
+    {"add", run_add},
+    {"fill", run_fill},
+    {"rmsnorm", run_rmsnorm},
+    {"embedding_f32", run_embedding_f32},
+    {"embedding_bf16", run_embedding_bf16},
+    {"embedding_q4k", run_embedding_q4k},
     {"round_bf16", run_round_bf16},
     {"ffn_gate_up_silu_q4k", run_ffn_gate_up_silu_q4k},
     {"gemm_mxfp4", run_gemm_mxfp4},

@@ -97,6 +97,12 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
 hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64_t split,
                              hipStream_t stream);
 hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream);
+hipError_t launch_add(const float* a, const float* b, float* o, uint64_t n, hipStream_t stream);
+hipError_t launch_fill_i32(int32_t* out, int32_t value, uint64_t n, hipStream_t stream);
+hipError_t launch_rmsnorm(const float* x, const float* w, float* y, uint64_t rows, uint64_t cols, float eps,
+                          hipStream_t stream);
+hipError_t launch_embedding(int kind, const uint32_t* ids, const void* table, float* out, uint64_t rows,
+                            uint64_t cols, uint64_t vocab, hipStream_t stream);
 hipError_t launch_silu_mul(const float* g, const float* u, float* o, uint64_t n, hipStream_t stream);
 hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
 

@@ -23,7 +23,7 @@ REFERENCE_IDS = [
     "top_k_rows", "gemm_q6k", "gemm_q6k_vec", "gemm_q6k_rows2", "gemm_q6k_rows3", "gemm_q6k_rows4",
     "gemm_q6k_rows5", "gemm_q6k_batched", "gemm_q5k", "gemm_q5k_vec", "gemm_q5k_rows2", "gemm_q5k_rows3",
     "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched", "moe_experts_down_q6k", "gemm_q5k_wmma", "gemm_q6k_wmma",
-    "silu_mul", "round_bf16",
+    "silu_mul", "round_bf16", "add", "fill", "rmsnorm", "embedding_f32", "embedding_bf16", "embedding_q4k",
 ]
 
 

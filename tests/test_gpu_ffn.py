@@ -132,3 +132,55 @@ def test_argument_errors(backend):
         run(backend, "silu_mul", [dx, dx, small], [n])
     with pytest.raises(StatusError):
         run(backend, "round_bf16", [small], [n])
+
+
+def test_add_and_fill_bit_exact(backend):
+    g = synth.rng(780)
+    n = 100003
+    a, b = g.standard_normal(n).astype(np.float32), (g.standard_normal(n) * 1e3).astype(np.float32)
+    da, db, do = backend.Upload(a), backend.Upload(b), backend.AllocateBuffer(4 * n)
+    run(backend, "add", [da, db, do], [n], grid=((n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    assert same_bits(backend.CopyD2H(do, dtype=np.float32), a + b)
+    run(backend, "fill", [do], [0xFFFFFFFF, n - 3], grid=((n + 255) // 256, 1, 1))   # value -1, all but the last 3
+    backend.Synchronize()
+    got = backend.CopyD2H(do, dtype=np.int32)
+    assert np.all(got[:n - 3] == -1) and np.array_equal(got[n - 3:].view(np.float32), (a + b)[n - 3:])
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 5120), (7, 2048), (3, 100), (2, 17408), (16, 1)])
+def test_rmsnorm_matches_oracle(backend, rows, cols):
+    g = synth.rng(790 + cols)
+    x = (g.standard_normal((rows, cols)) * 2).astype(np.float32)
+    w = (1 + 0.1 * g.standard_normal(cols)).astype(np.float32)
+    eps = np.float32(1e-6)
+    dx, dw, dy = backend.Upload(x), backend.Upload(w), backend.AllocateBuffer(4 * rows * cols)
+    run(backend, "rmsnorm", [dx, dw, dy], [rows, cols, int(eps.view(np.uint32))], grid=((rows * cols + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dy, dtype=np.float32).reshape(rows, cols)
+    want = oracle.rmsnorm(x, w, rows, cols, float(eps))
+    # the sum of squares is added in another order than the oracle's sequential chain: the gain
+    # differs by about sqrt(cols) * 2^-24 relative, and every output with it
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-12)) < 2e-5
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16", "q4k"])
+def test_embedding_bit_exact(backend, kind):
+    g = synth.rng(800)
+    vocab, cols = 301, 1024
+    ids = np.concatenate([g.integers(0, vocab, 40), [vocab, 2 ** 32 - 1, 0, vocab - 1]]).astype(np.uint32)
+    if kind == "f32":
+        table = g.standard_normal((vocab, cols)).astype(np.float32)
+    elif kind == "bf16":
+        table = (g.standard_normal((vocab, cols)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    else:
+        table = synth.q4k_weights(g, vocab, cols)
+    di, dt = backend.Upload(ids), backend.Upload(table)
+    do = backend.AllocateBuffer(4 * ids.size * cols)
+    run(backend, f"embedding_{kind}", [di, dt, do], [ids.size, cols, vocab], grid=((ids.size * cols + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(do, dtype=np.float32).reshape(ids.size, cols)
+    assert same_bits(got, oracle.embedding(kind, ids, table, ids.size, cols, vocab))
+    if kind == "q4k":
+        with pytest.raises(StatusError):
+            run(backend, "embedding_q4k", [di, dt, do], [ids.size, cols - 1, vocab])

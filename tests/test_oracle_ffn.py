@@ -41,3 +41,44 @@ def test_ffn_gate_up_is_the_composition_of_pinned_parts():
     # a zero gate matrix gives silu(0) * u = 0 everywhere
     zero = np.zeros_like(gate)
     assert np.all(oracle.ffn_gate_up_silu_q4k(x, zero, up, 2, n, k) == 0)
+
+
+def test_rmsnorm_against_float64_and_invariants():
+    g = np.random.default_rng(44)
+    rows, cols, eps = 5, 5120, 1e-6
+    x = (g.standard_normal((rows, cols)) * 3).astype(np.float32)
+    w = (1 + 0.1 * g.standard_normal(cols)).astype(np.float32)
+    got = oracle.rmsnorm(x, w, rows, cols, eps).astype(np.float64)
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps) * w.astype(np.float64)
+    # a sequential fp32 sum of 5120 squares: relative error about sqrt(cols) * 2^-24
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-12)) < 2e-5
+    # a row of equal values c with eps = 0 and unit weights normalises to sign(c) (all ones)
+    ones = oracle.rmsnorm(np.full((1, 256), -3.0, np.float32), np.ones(256, np.float32), 1, 256, 0.0)
+    assert np.allclose(ones, -1.0, rtol=0, atol=1e-6)
+    # scaling the row by a power of two leaves the result unchanged when eps = 0 (exact scaling)
+    a = oracle.rmsnorm(x, w, rows, cols, 0.0)
+    b = oracle.rmsnorm(x * np.float32(8), w, rows, cols, 0.0)
+    assert np.array_equal(a, b)
+    import pytest
+    with pytest.raises(oracle.OracleError):
+        oracle.rmsnorm(x, w, 0, cols, eps)
+
+
+def test_embedding_gathers_decoded_rows_and_zero_fills_bad_ids():
+    from tessera_amd import synth
+    g = synth.rng(45)
+    vocab, cols = 37, 512
+    ids = np.array([0, 36, 5, 37, 4000000000, 5], dtype=np.uint32)
+    f32 = g.standard_normal((vocab, cols)).astype(np.float32)
+    out = oracle.embedding("f32", ids, f32, ids.size, cols, vocab)
+    assert np.array_equal(out[[0, 1, 2, 5]], f32[[0, 36, 5, 5]]) and np.all(out[[3, 4]] == 0)
+    bf16 = (f32.view(np.uint32) >> 16).astype(np.uint16)
+    out = oracle.embedding("bf16", ids, bf16, ids.size, cols, vocab)
+    assert np.array_equal(out[[0, 1, 2]].view(np.uint32), (bf16[[0, 36, 5]].astype(np.uint32) << 16))
+    assert np.all(out[[3, 4]] == 0)
+    q4k = synth.q4k_weights(g, vocab, cols)
+    deq = oracle.dequantize_q4k(q4k).reshape(vocab, cols)
+    out = oracle.embedding("q4k", ids, q4k, ids.size, cols, vocab)
+    assert np.array_equal(out[[0, 1, 2, 5]].view(np.uint32), deq[[0, 36, 5, 5]].view(np.uint32))
+    assert np.all(out[[3, 4]] == 0)

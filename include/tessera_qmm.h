@@ -100,8 +100,9 @@ const char* qmm_kernel_name(size_t index);
  * Validation happens before any device work and returns InvalidArgument: zero grid or
  * block dimensions, more than 16 buffers or scalars (ValidateLaunch,
  * backend.hpp:138-148), the per-id argument counts and shape rules of
- * CheckBuiltInArgs (backend.hpp:391-841), a NULL buffer, and -- when `buf_bytes` is
- * not NULL -- any buffer smaller than the launch's scalars require.  `buf_bytes[i]` is
+ * CheckBuiltInArgs (backend.hpp:391-841), a NULL buffer, a buffer pointer that is not
+ * 16-byte aligned (device allocations are; the kernels use 16-byte vector loads), and --
+ * when `buf_bytes` is not NULL -- any buffer smaller than the launch's scalars require.  `buf_bytes[i]` is
  * Buffer::Size() of buffer i; pass NULL to skip the size check.
  *
  * Geometry: the ids keep the reference's argument contracts, but a gfx950 kernel has

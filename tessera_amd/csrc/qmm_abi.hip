@@ -930,6 +930,9 @@ qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t 
   if ((nbuffers != 0 && buffers == nullptr) || (nscalars != 0 && scalars == nullptr)) return bad("qmm_launch: null argument array");
   for (size_t i = 0; i < nbuffers; ++i) {
     if (buffers[i] == nullptr) return bad("qmm_launch: null buffer");
+    // The kernels use 16-byte vector and direct-to-LDS loads from the start of each operand;
+    // device allocations are aligned far beyond that, a pointer into the middle of one may not be.
+    if (reinterpret_cast<uintptr_t>(buffers[i]) % 16 != 0) return bad("qmm_launch: buffers must be 16-byte aligned");
   }
   if (g_device < 0) {
     g_last_error = "qmm_launch: qmm_init has not succeeded";

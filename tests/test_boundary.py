@@ -105,6 +105,8 @@ def test_per_id_validation_on_device(backend):
         assert e.value.code == StatusCode.InvalidArgument, (name, scalars)
 
     expect_invalid("gemm_q4k", [a, w], [1, n, k])                # buffer count
+    off = backend.WrapBuffer(a.Handle() + 4, a.Size() - 4)          # a pointer into the middle of an allocation
+    expect_invalid("gemm_q4k", [off, w, c], [1, n, k - 256])     # not 16-byte aligned
     expect_invalid("gemm_q4k", [a, w, c], [1, n])                # scalar count
     expect_invalid("gemm_q4k", [a, w, c], [0, n, k])             # zero m
     expect_invalid("gemm_q4k", [a, w, c], [1, n, 500])           # k % 256

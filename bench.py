@@ -186,6 +186,28 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
                                                    "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
     del pairs, w_q1
 
+    # ---- FP8 E4M3 weights with one fp32 scale per row (gemm_fp8), fp32 activations -------------------
+    # random codes (NaN codes avoided) and scales: the generator for parity tests builds a real
+    # distribution on the CPU, which at 89 M weights takes longer than the measurement is worth
+    res = {}
+    kf8 = backend.LoadKernel("gemm_fp8")
+    for label, (nn, kk) in (("17408x5120", (n, k)), ("5120x17408", (k, n))):
+        codes = torch.randint(0, 0x7E, (nn * kk,), dtype=torch.uint8, device=dev) | \
+            (torch.randint(0, 2, (nn * kk,), dtype=torch.uint8, device=dev) << 7)
+        scales = torch.rand(nn, dtype=torch.float32, device=dev) * 1e-4 + 1e-5
+        wl = [codes] + [codes.clone() for _ in range(3)]
+        for m in (1, 4):
+            x = to_dev(synth.activations_f32(g, m, kk))
+            y = torch.empty(m * nn, dtype=torch.float32, device=dev)
+            launches = [(kf8, KernelLaunch(grid_x=(m * nn + 255) // 256, buffers=[wrap(x), wrap(w), wrap(scales), wrap(y)],
+                                           scalars=[m, nn, kk])) for w in wl]
+            us = timed_us(launches, 20) / len(wl)
+            nbytes = nn * kk + 4 * nn + 4 * m * kk + 4 * m * nn
+            res[f"{label}_m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                    "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del wl, codes
+    out["fp8_gemv"] = res
+
     # ---- Q6_K and Q5_K (the other block formats of K-quant files), gate/up and down shapes --------
     for fmt, block_bytes, gen, rows in (("q6k", 210, synth.q6k_weights, (1, 2)), ("q5k", 176, synth.q5k_weights, (1,))):
         res = {}

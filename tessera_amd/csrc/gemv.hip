@@ -947,27 +947,31 @@ struct MxFp4A8Codec {
 // (include/tessera/backend.hpp:191-194; src/core/numerics/gemm.cpp:253-277).
 // A chunk is 16 weights; the row scale multiplies the finished dot product.
 // ----------------------------------------------------------------------------
-struct Fp8Codec {
+// NQ = 16-byte pieces per chunk: a lane takes 16 * NQ consecutive weights of a row.  One piece
+// for rows up to 16384 long, two beyond (a row must fit the 1024 threads of a workgroup).
+template <int NQ>
+struct Fp8CodecT {
   struct Args {
     const float* a;
     const uint8_t* w;
     const float* s;
     uint32_t k;
   };
+  static constexpr uint32_t kChunk = 16u * NQ;
   template <int R>
   struct X {
-    float v[R][16];
+    float v[R][16 * NQ];
   };
   struct Frag {
-    uint4 q;
+    uint4 q[NQ];
   };
 
-  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 16u; }
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / kChunk; }
   // Whether the skeleton stages fp32 activations through LDS for this codec, and the
   // first activation element a chunk needs (its slice stays inside that 64-aligned group
   // or starts there).
   static constexpr bool kStageX = true;
-  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 16u; }
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * kChunk; }
 
   template <int R, class Src>
   static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
@@ -975,8 +979,8 @@ struct Fp8Codec {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
-      for (int i = 0; i < 16; i += 4) {
-        float4 v = src(r, chunk * 16u + i);
+      for (int i = 0; i < 16 * NQ; i += 4) {
+        float4 v = src(r, chunk * kChunk + i);
         if (!valid) v = make_float4(0.f, 0.f, 0.f, 0.f);
         x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
       }
@@ -985,28 +989,33 @@ struct Fp8Codec {
 
   static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
                                                    uint32_t prow) {
-    return Lane{(prow * cpr + chunk) * 16u, 0u};
+    return Lane{(prow * cpr + chunk) * kChunk, 0u};
   }
 
   static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
                                               uint32_t cpr, Frag& f) {
-    f.q = load_u4(p.w + static_cast<size_t>(row) * cpr * 16u + ln.off0);
+    const uint8_t* base = p.w + static_cast<size_t>(row) * cpr * kChunk + ln.off0;
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) f.q[j] = load_u4(base + 16 * j);
   }
 
   template <int R>
   static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
-    const uint32_t qw[4] = {f.q.x, f.q.y, f.q.z, f.q.w};
-    float2_t wv[8];
+    float2_t wv[8 * NQ];
 #pragma unroll
-    for (int wi = 0; wi < 4; ++wi) {
-      wv[2 * wi] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, false);
-      wv[2 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, true);
+    for (int j = 0; j < NQ; ++j) {
+      const uint32_t qw[4] = {f.q[j].x, f.q[j].y, f.q[j].z, f.q[j].w};
+#pragma unroll
+      for (int wi = 0; wi < 4; ++wi) {
+        wv[8 * j + 2 * wi] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, false);
+        wv[8 * j + 2 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, true);
+      }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll
-      for (int b = 0; b < 8; ++b) {
+      for (int b = 0; b < 8 * NQ; ++b) {
         a0 = fmaf(x.v[r][2 * b], wv[b][0], a0);
         a1 = fmaf(x.v[r][2 * b + 1], wv[b][1], a1);
       }
@@ -1019,6 +1028,8 @@ struct Fp8Codec {
     return v * p.s[row];
   }
 };
+using Fp8Codec = Fp8CodecT<1>;
+using Fp8WideCodec = Fp8CodecT<2>;
 
 // ----------------------------------------------------------------------------
 // The skeleton.  A workgroup owns a contiguous range of row groups; a group is P
@@ -1417,7 +1428,7 @@ void set_num_cus(int cus) {
 // 1024 threads per row.
 bool gemv_q4k_supported(uint64_t k) { return k % 256 == 0 && k / 32 <= 1024; }  // multi-row limit
 bool gemv_mxfp4_supported(uint64_t k) { return k % 32 == 0 && k / 32 <= 1024; }
-bool gemv_fp8_supported(uint64_t k) { return k % 16 == 0 && k / 16 <= 1024; }
+bool gemv_fp8_supported(uint64_t k) { return k % 16 == 0 && (k / 16 <= 1024 || (k % 32 == 0 && k / 32 <= 1024)); }
 
 hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                            uint32_t k, hipStream_t stream) {
@@ -1546,6 +1557,23 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream) {
+  if (k / 16u > 1024u) {
+    // rows of 16385..32768 weights: 32 weights a lane, one or two activation rows per weight pass
+    for (uint32_t r0 = 0; r0 < m;) {
+      Fp8WideCodec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
+      float* out = c + static_cast<size_t>(r0) * n;
+      hipError_t e;
+      uint32_t took;
+      if (m - r0 >= 2) {
+        e = launch_gemv_r<Fp8WideCodec, 2, 1024, 2, 1>(args, out, n, k, n, stream), took = 2;
+      } else {
+        e = launch_gemv_r<Fp8WideCodec, 1, 1024, 2, 1>(args, out, n, k, n, stream), took = 1;
+      }
+      if (e != hipSuccess) return e;
+      r0 += took;
+    }
+    return hipSuccess;
+  }
   for (uint32_t r0 = 0; r0 < m;) {
     const uint32_t left = m - r0;
     Fp8Codec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};

@@ -575,7 +575,7 @@ qmm_status run_gemm_fp8(const LaunchCtx& c) {
     return bad("gemm_fp8: a buffer is smaller than m, n, k require");
   }
   if (!qmm::gemv_fp8_supported(k)) {
-    g_last_error = "gemm_fp8: k must be a multiple of 16 and at most 16384";
+    g_last_error = "gemm_fp8: k must be a multiple of 16 up to 16384 or a multiple of 32 up to 32768";
     return QMM_UNSUPPORTED_FEATURE;
   }
   return map_hip(qmm::launch_fp8_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),

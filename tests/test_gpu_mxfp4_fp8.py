@@ -178,7 +178,8 @@ def test_w4a8_wmma_contract(backend, n, k, m, split):
     assert e.value.code == StatusCode.UnsupportedFeature
 
 
-@pytest.mark.parametrize("n,k", [(64, 256), (100, 1008), (130, 5120), (40, 16384)])
+# rows longer than 16384 take the 32-weights-a-lane codec (17408: the dense down projection)
+@pytest.mark.parametrize("n,k", [(64, 256), (100, 1008), (130, 5120), (40, 16384), (67, 17408), (9, 32768), (33, 16416)])
 @pytest.mark.parametrize("m", [1, 2, 5])
 def test_gemm_fp8_matches_oracle(backend, n, k, m):
     g = synth.rng(4000 * m + n + k)
@@ -193,11 +194,12 @@ def test_gemm_fp8_matches_oracle(backend, n, k, m):
     assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
-def test_gemm_fp8_one_hot_bit_exact(backend):
+@pytest.mark.parametrize("k", [512, 17408])
+def test_gemm_fp8_one_hot_bit_exact(backend, k):
     g = synth.rng(77)
-    n, k = 50, 512
+    n = 50
     codes, scales = synth.fp8_weights(g, n, k)
-    pos = [0, 1, 15, 16, 17, 255, 511]
+    pos = [0, 1, 15, 16, 17, 31, 32, 255, k - 1]
     ref = oracle.gemm_fp8(synth.one_hot_rows(k, pos), codes, scales, len(pos), n, k)
     da, dw, ds = backend.Upload(synth.one_hot_rows(k, pos)), backend.Upload(codes), backend.Upload(scales)
     dc = backend.AllocateBuffer(4 * len(pos) * n)

@@ -74,3 +74,16 @@ def test_full_size_prefill_rows(backend):
     shard = synth.mxfp4_column_shard(w, n, k, 0, n // 2)
     got_shard = w4a8(backend, x, shard, m, n // 2, k)
     assert np.array_equal(got_shard, got[:, : n // 2])
+
+
+def test_down_projection_shape_prefill_rows(backend):
+    """The other FFN shape (N=5120, K=17408) at a ragged M: sampled rows against the oracle."""
+    g = synth.rng(31338)
+    m, n, k = 500, 5120, 17408
+    w = synth.mxfp4_weights(g, n, k, -8, -4)
+    x = synth.activations_bf16(g, m, k)
+    got = w4a8(backend, x, w, m, n, k)
+    rows = [0, 255, 256, 499]
+    codes, scale = oracle.quantize_fp8_pack(x[rows], len(rows), k)
+    ref = oracle.gemm_mxfp4_w4a8(codes, scale, w, len(rows), n, k)
+    assert rms_err(got[rows], ref) <= 5e-4, rms_err(got[rows], ref)

@@ -92,3 +92,17 @@ def test_full_size_prefill_rows(backend):
     assert norm_err(got[rows], ref) <= NORM_TOL
     shard = gemm(backend, "gemm_q4k_wmma", a, w[: 8704 * (k // 256) * 144], m, 8704, k)
     assert np.array_equal(shard, got[:, :8704])
+
+
+def test_down_projection_shape_prefill_rows(backend):
+    """The other FFN shape (N=5120, K=17408: 68 super-blocks a row, 544 K-steps a tile) at M=512,
+    with a row count that leaves a ragged last row tile: sampled rows against the oracle."""
+    g = synth.rng(5)
+    m, n, k = 500, 5120, 17408
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_bf16(g, m, k)
+    got = gemm(backend, "gemm_q4k_wmma", a, w, m, n, k)
+    rows = [0, 255, 256, 499]
+    ref = oracle.gemm_q4k(a[rows], w, len(rows), n, k, threads=True)
+    assert rms_err(got[rows], ref) <= RMS_TOL, rms_err(got[rows], ref)
+    assert norm_err(got[rows], ref) <= NORM_TOL

@@ -259,6 +259,24 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
                                     "frac_fp16_peak": round(2 * m * n * k / us / 1e6 / 2500.0, 4)}
         del wf
     out["prefill_gemm_m2048_k5120"] = prefill
+
+    # ---- the same prefill at the down-projection shape (N=5120, K=17408) ---------------------------
+    down = {}
+    a_d = to_dev(synth.activations_bf16(g, m, n))            # m x 17408
+    y = torch.empty(m * k, dtype=torch.float32, device=dev)
+    wq_d = w_q                                               # the same bytes read as 5120 rows of 68 blocks
+    us = timed_us([(kw, KernelLaunch(grid_x=k // 64, grid_y=m // 128, buffers=[wrap(a_d), wrap(wq_d), wrap(y)],
+                                     scalars=[m, k, n]))], 10, graph=False)
+    down["q4k"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * n * k / us / 1e6, 1),
+                   "frac_fp16_peak": round(2 * m * n * k / us / 1e6 / 2500.0, 4)}
+    a8_d = torch.empty(m * n, dtype=torch.uint8, device=dev)
+    backend.LaunchKernel(kq, KernelLaunch(grid_x=m, buffers=[wrap(a_d), wrap(a8_d), wrap(asc)], scalars=[m, n]))
+    wref_d = torch.empty(k, dtype=torch.uint8, device=dev)
+    us = timed_us([(kg, KernelLaunch(grid_x=k // 64, buffers=[wrap(a8_d), wrap(w_mx), wrap(asc), wrap(wref_d), wrap(y)],
+                                     scalars=[m, k, n, 1, 0]))], 10, graph=False)
+    down["mxfp4"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * n * k / us / 1e6, 1),
+                     "frac_fp8_peak": round(2 * m * n * k / us / 1e6 / 5000.0, 4)}
+    out["prefill_gemm_m2048_n5120_k17408"] = down
     del a, w_q, w_mx, a8, y
 
     # ---- configs[4]: routed Q4_K experts ---------------------------------------------------

@@ -139,6 +139,21 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
         w4a8[f"m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                          "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "quantize_us": round(uq, 2)}
     out["mxfp4_w4a8_gemv_17408x5120"] = w4a8
+
+    # ---- the same weights with fp32 activations (gemm_mxfp4, gemm_mxfp4_rows: the reference's
+    # GEMV when no fp8 tensor-core path exists) ---------------------------------------------------
+    f32a = {}
+    for m, kid in ((1, "gemm_mxfp4"), (4, "gemm_mxfp4_rows"), (16, "gemm_mxfp4_rows")):
+        kern = backend.LoadKernel(kid)
+        x = to_dev(synth.activations_f32(g, m, k))
+        y = torch.empty(m * n, dtype=torch.float32, device=dev)
+        launches = [(kern, KernelLaunch(grid_x=(n + 7) // 8, buffers=[wrap(x), wrap(w), wrap(y)], scalars=[m, n, k]))
+                    for w in w_list]
+        us = timed_us(launches, 10) / copies
+        nbytes = n * k // 2 + n * k // 32 + 4 * m * k + 4 * m * n
+        f32a[f"m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                         "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    out["mxfp4_gemv_f32_activations_17408x5120"] = f32a
     del w_list
 
     # ---- configs[1] weights with 2..16 rows (speculative verify), Q4_K -----------------------

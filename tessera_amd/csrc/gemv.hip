@@ -849,6 +849,85 @@ struct MxFp4Codec {
   }
 };
 
+// MXFP4, single activation row: two MX blocks (64 weights, 32 nibble bytes, two scale bytes) per
+// thread, so the reduction, the scale loads and the loop overhead are paid once per 64 weights
+// (as Q4KPairCodec does for Q4_K).  K must be a multiple of 64.
+struct MxFp4PairCodec {
+  using Args = MxFp4Codec::Args;
+  template <int R>
+  struct X {
+    float v[R][64];
+  };
+  struct Frag {
+    uint4 q0, q1;
+    uint32_t s;   // two E8M0 bytes
+  };
+
+  static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / 64u; }
+  static constexpr bool kStageX = true;
+  static __device__ __forceinline__ uint32_t x_elem0(uint32_t chunk) { return chunk * 64u; }
+
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args&, uint32_t chunk, bool valid, X<R>& x, const Src& src) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int i = 0; i < 64; i += 4) {
+        float4 v = src(r, chunk * 64u + i);
+        if (!valid) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        x.v[r][i] = v.x, x.v[r][i + 1] = v.y, x.v[r][i + 2] = v.z, x.v[r][i + 3] = v.w;
+      }
+    }
+  }
+
+  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk, uint32_t prow) {
+    const uint32_t c = prow * cpr + chunk;
+    return Lane{c * 32u, c * 2u};
+  }
+
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row, uint32_t cpr, Frag& f) {
+    const size_t c = static_cast<size_t>(row) * cpr;
+    const uint8_t* base = p.w + c * 32u + ln.off0;
+    f.q0 = load_u4(base);
+    f.q1 = load_u4(base + 16u);
+    f.s = *reinterpret_cast<const uint16_t*>(p.s + c * 2u + ln.off1);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
+    const uint32_t qw[8] = {f.q0.x, f.q0.y, f.q0.z, f.q0.w, f.q1.x, f.q1.y, f.q1.z, f.q1.w};
+    const float scale[2] = {e8m0_to_float(f.s & 0xFFu), e8m0_to_float(f.s >> 8)};
+#pragma unroll
+    for (int r = 0; r < R; ++r) out[r] = 0.0f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float2_t wv[16];
+#pragma unroll
+      for (int wi = 0; wi < 4; ++wi) {
+        wv[4 * wi + 0] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[4 * h + wi], 1.0f, 0);
+        wv[4 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[4 * h + wi], 1.0f, 1);
+        wv[4 * wi + 2] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[4 * h + wi], 1.0f, 2);
+        wv[4 * wi + 3] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(qw[4 * h + wi], 1.0f, 3);
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int b = 0; b < 16; ++b) {
+          a0 = fmaf(x.v[r][32 * h + 2 * b], wv[b][0], a0);
+          a1 = fmaf(x.v[r][32 * h + 2 * b + 1], wv[b][1], a1);
+        }
+        out[r] = fmaf(a0 + a1, scale[h], out[r]);
+      }
+    }
+  }
+
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+
 // ----------------------------------------------------------------------------
 // W4A8: MXFP4 weights, activations already quantized per token to E4M3 codes with
 // one fp32 scale per row (quantize_fp8_pack).  The weight side is lossless:
@@ -1525,7 +1604,14 @@ hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_
     } else if (left >= 2 && row_threads <= 768u) {
       e = launch_gemv_r<MxFp4Codec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<MxFp4Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
+      // one row: 64 weights a lane where K allows (and the row is long enough for the main kernel)
+      e = hipErrorInvalidValue;
+      const uint32_t cpr2 = k / 64u;
+      if (k % 64u == 0 && !(cpr2 == 4 || cpr2 == 8 || cpr2 == 16 || cpr2 == 32)) {
+        e = launch_gemv_r<MxFp4PairCodec, 1, 768, 3, 9>(args, out, n, k, n, stream);
+      }
+      if (e == hipErrorInvalidValue) e = launch_gemv_r<MxFp4Codec, 1, 1024, 4>(args, out, n, k, n, stream);
+      took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;

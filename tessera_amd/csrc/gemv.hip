@@ -1080,26 +1080,29 @@ struct Fp8CodecT {
 
   template <int R>
   static __device__ __forceinline__ void dot(const Frag& f, const X<R>& x, float (&out)[R]) {
-    float2_t wv[8 * NQ];
+    float a0[R], a1[R];
 #pragma unroll
-    for (int j = 0; j < NQ; ++j) {
+    for (int r = 0; r < R; ++r) a0[r] = a1[r] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {           // one 16-byte piece at a time keeps few converted values live
       const uint32_t qw[4] = {f.q[j].x, f.q[j].y, f.q[j].z, f.q[j].w};
+      float2_t wv[8];
 #pragma unroll
       for (int wi = 0; wi < 4; ++wi) {
-        wv[8 * j + 2 * wi] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, false);
-        wv[8 * j + 2 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, true);
+        wv[2 * wi] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, false);
+        wv[2 * wi + 1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(qw[wi], 1.0f, true);
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+          a0[r] = fmaf(x.v[r][16 * j + 2 * b], wv[b][0], a0[r]);
+          a1[r] = fmaf(x.v[r][16 * j + 2 * b + 1], wv[b][1], a1[r]);
+        }
       }
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      float a0 = 0.0f, a1 = 0.0f;
-#pragma unroll
-      for (int b = 0; b < 8 * NQ; ++b) {
-        a0 = fmaf(x.v[r][2 * b], wv[b][0], a0);
-        a1 = fmaf(x.v[r][2 * b + 1], wv[b][1], a1);
-      }
-      out[r] = a0 + a1;
-    }
+    for (int r = 0; r < R; ++r) out[r] = a0[r] + a1[r];
   }
 
   template <int R>
@@ -1109,6 +1112,7 @@ struct Fp8CodecT {
 };
 using Fp8Codec = Fp8CodecT<1>;
 using Fp8WideCodec = Fp8CodecT<2>;
+using Fp8QuadCodec = Fp8CodecT<4>;   // one activation row: 64 weights a lane
 
 // ----------------------------------------------------------------------------
 // The skeleton.  A workgroup owns a contiguous range of row groups; a group is P
@@ -1643,6 +1647,12 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream) {
+  const uint32_t cpr4 = k / 64u;
+  if (m == 1 && k % 64u == 0 && cpr4 >= 64u && cpr4 <= 768u) {
+    // one row: 64 weights a lane, so the reduction and the loop overhead are paid once per 64
+    Fp8QuadCodec::Args args{a, w, s, k};
+    return launch_gemv_r<Fp8QuadCodec, 1, 768, 3, 9>(args, c, n, k, n, stream);
+  }
   if (k / 16u > 1024u) {
     // rows of 16385..32768 weights: 32 weights a lane, one or two activation rows per weight pass
     for (uint32_t r0 = 0; r0 < m;) {

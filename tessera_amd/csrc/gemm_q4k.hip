@@ -346,28 +346,33 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void q4k_gemm_kernel(
                         n_end);
 }
 
-// Grouped form for routed experts: segment e (grid.x) multiplies rows seg[e]..seg[e+1] of a16
+// Grouped form for routed experts: segment e multiplies rows seg[e]..seg[e+1] of a16
 // by expert e's weights (w + e * w_stride) into the same rows of c.  Segment bounds live in
 // device memory (the routing is computed on the device); an empty segment leaves at once.
 template <int BM, int BN>
 __global__ __launch_bounds__(BN * 2) void q4k_gemm_grouped_kernel(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
     float* __restrict__ c, const uint32_t* __restrict__ seg, uint64_t w_stride, uint32_t n, uint32_t k,
-    const uint8_t* __restrict__ w2, float* __restrict__ c2, uint64_t w2_stride) {
-  // grid.z = 2 runs a second expert tensor of the same shape against the same rows (gate and up
-  // in one launch: twice the workgroups to fill the tail of the first with).
-  if (blockIdx.z == 1) w = w2, c = c2, w_stride = w2_stride;
-  // Expert on grid.x: workgroups are dealt to the eight XCDs by linear index, so with the
-  // expert varying fastest all column tiles of an expert land on one XCD and its activation
-  // rows are fetched into one L2 instead of eight.
-  const uint32_t e = blockIdx.x;
+    uint32_t experts, uint32_t tensors, const uint8_t* __restrict__ w2, float* __restrict__ c2, uint64_t w2_stride) {
+  // One-dimensional grid, decoded so that an expert's activation rows are fetched from HBM once:
+  // workgroups are dealt to the eight XCDs (one L2 each) by linear index, so the expert's low three
+  // bits are the index's low three bits (all its tiles on one XCD), and its column tiles of both
+  // tensors follow each other in dispatch order (its rows are still in that L2 when the next tile
+  // asks for them).  `tensors` = 2 runs a second expert tensor of the same shape against the same
+  // rows (gate and up in one launch).
+  const uint32_t tiles = (n + BN - 1) / BN;
+  const uint32_t slot = blockIdx.x / 8u, per_expert = tiles * tensors;
+  const uint32_t e = (slot / per_expert) * 8u + blockIdx.x % 8u;
+  const uint32_t tz = slot % per_expert, tile = tz % tiles;
+  if (e >= experts) return;
+  if (tz >= tiles) w = w2, c = c2, w_stride = w2_stride;
   const uint32_t r0 = seg[e], r1 = seg[e + 1];
   if (r1 <= r0) return;
   const _Float16* a_e = a16 + static_cast<size_t>(r0) * k;
   const uint8_t* w_e = w + e * w_stride;
   float* c_e = c + static_cast<size_t>(r0) * n;
   for (uint32_t m0 = 0; m0 < r1 - r0; m0 += BM) {
-    q4k_gemm_tile<BM, BN, BM, 32>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, blockIdx.y * BN, n);
+    q4k_gemm_tile<BM, BN, BM, 32>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, tile * BN, n);
   }
 }
 
@@ -773,11 +778,13 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
   hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, seg, pos);
   hipLaunchKernelGGL(rows_to_f16_kernel, dim3(pairs), dim3(256), 0, stream, x, a16, x_scale, hidden, pos, top_k);
   constexpr int BM = 32, BN = 64;
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (inter + BN - 1) / BN, 2), dim3(BN * 2), 0, stream,
-                     a16, x_scale, gate, g, seg, gate_stride, inter, hidden, up, u, up_stride);
+  const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((inter + BN - 1) / BN) * 2u), dim3(BN * 2), 0,
+                     stream, a16, x_scale, gate, g, seg, gate_stride, inter, hidden, experts, 2u, up, u, up_stride);
   hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(pairs), dim3(256), 0, stream, g, u, phi16, phi_scale, inter);
-  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(experts, (hidden + BN - 1) / BN), dim3(BN * 2), 0, stream,
-                     phi16, phi_scale, down, rows, seg, down_stride, hidden, inter, nullptr, nullptr, uint64_t{0});
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((hidden + BN - 1) / BN)), dim3(BN * 2), 0,
+                     stream, phi16, phi_scale, down, rows, seg, down_stride, hidden, inter, experts, 1u, nullptr, nullptr,
+                     uint64_t{0});
   const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, rows, pos,
                      wts, out, tokens, top_k, hidden, accumulate);

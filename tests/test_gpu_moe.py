@@ -155,7 +155,7 @@ def forward_grouped(backend, x, ids, wts, gate, up, down, hidden, inter, experts
 
 
 @pytest.mark.parametrize("rows,experts,hidden,inter,top_k", [(1, 8, 256, 256, 2), (40, 16, 512, 256, 4),
-                                                             (130, 6, 256, 512, 3), (64, 3, 768, 256, 1)])
+                                                             (130, 6, 256, 512, 3), (64, 3, 768, 256, 1), (90, 12, 256, 256, 2)])
 def test_grouped_ffn_matches_oracle(backend, rows, experts, hidden, inter, top_k):
     """moe_experts_ffn_q4k_rows: tokens grouped by expert, three grouped fp16-MFMA GEMMs.  The
     operands are rounded to fp16 twice along the way (weights as in the Q4_K prefill GEMM, and

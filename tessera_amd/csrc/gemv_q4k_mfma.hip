@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void q4k_rows_prep_kernel(const float* __restr
   __syncthreads();
   amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   const float s = live ? prep_scale(amax) : 0.0f;
-  if (t == 0 && live) inv_scale[r] = 1.0f / s;
+  if (t == 0 && live && blockIdx.y == 0) inv_scale[r] = 1.0f / s;
 
   constexpr uint32_t kRowsPerChain = XC / 2;
   const uint32_t chain = r / kRowsPerChain, col = 2u * (r % kRowsPerChain);
@@ -97,8 +97,10 @@ __global__ __launch_bounds__(256) void q4k_rows_prep_kernel(const float* __restr
   // share g (consecutive, since 256 is a multiple of 8) add up the two sub-block sums of what the
   // matrix core will see (hi + lo, undivided); the sums are themselves split into hi and lo.
   constexpr uint32_t kOrder[8] = {0, 2, 1, 3, 4, 6, 5, 7};
-  for (uint32_t base = 0; base < sbs * 32u; base += 256u) {
-    const uint32_t i = base + t;
+  // grid.y workgroups share a row: each finds the row's maximum for itself (the row is a few
+  // tens of KB in L2) and converts 256 slots, so the pre-pass is one short wave of work.
+  {
+    const uint32_t i = blockIdx.y * 256u + t;
     const bool in = i < sbs * 32u;
     const uint32_t sb = in ? i / 32u : 0u, dw = i % 32u, g = dw / 8u, e0 = 4u * (dw % 8u);
     const float4 ev = *reinterpret_cast<const float4*>(row + sb * 256u + (2u * g) * 32u + e0);
@@ -721,11 +723,12 @@ hipError_t launch_q4k_gemv_mfma(const float* a, const uint8_t* w, float* c, void
   float* inv = static_cast<float*>(workspace);
   uint8_t* xop = static_cast<uint8_t*>(workspace) + 256;
   const uint32_t prep_rows = p.nc * (p.xc / 2u);
+  const dim3 prep_grid(prep_rows, (k / 256u * 32u + 255u) / 256u);
   if (p.xc == 2) {
-    hipLaunchKernelGGL(q4k_rows_prep_kernel<2>, dim3(prep_rows), dim3(256), 0, stream, a,
+    hipLaunchKernelGGL(q4k_rows_prep_kernel<2>, prep_grid, dim3(256), 0, stream, a,
                        reinterpret_cast<_Float16*>(xop), inv, m, k, p.nc);
   } else {
-    hipLaunchKernelGGL(q4k_rows_prep_kernel<4>, dim3(prep_rows), dim3(256), 0, stream, a,
+    hipLaunchKernelGGL(q4k_rows_prep_kernel<4>, prep_grid, dim3(256), 0, stream, a,
                        reinterpret_cast<_Float16*>(xop), inv, m, k, p.nc);
   }
 #define QMM_MFMA_CASE(KS_, KH_, NC_, XC_, DEPTH_)                                        \

@@ -292,14 +292,28 @@ qmm_status run_ffn_gate_up_silu_q4k(const LaunchCtx& c) {
   if (m == 1 && qmm::ffn_gate_up_q4k_supported(k)) {
     return map_hip(qmm::launch_ffn_gate_up_q4k(x, gate, up, out, static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
   }
-  // The up product goes behind whatever the Q4_K GEMM keeps at the start of the workspace; a
-  // request for that smaller size returns the same base, so the two do not overlap.
-  const size_t gemm_ws = (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
-  const size_t up_off = (gemm_ws + 255) & ~size_t{255};
-  void* ws = nullptr;
-  qmm_status st = workspace(up_off + static_cast<size_t>(m) * n * 4, &ws);
-  if (st != QMM_OK) return st;
-  float* u = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + up_off);
+  const size_t up_bytes = static_cast<size_t>(m) * n * 4;
+  float* u = nullptr;
+  qmm_status st = QMM_OK;
+  if (m < kQ4KGemmMinRows) {
+    // Decode-sized call: the up product goes into the fixed decode scratch, behind the room the
+    // few-row kernels may use for their activation operand, so nothing is allocated (a recorded
+    // decode step stays valid).
+    const size_t up_off = (qmm::gemv_q4k_mfma_workspace_bytes(8, k) + 255) & ~size_t{255};
+    if (g_decode_scratch != nullptr && up_off + up_bytes <= kDecodeScratchBytes) {
+      u = reinterpret_cast<float*>(static_cast<uint8_t*>(g_decode_scratch) + up_off);
+    }
+  }
+  if (u == nullptr) {
+    // The up product goes behind whatever the Q4_K GEMM keeps at the start of the workspace; a
+    // request for that smaller size returns the same base, so the two do not overlap.
+    const size_t gemm_ws = (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
+    const size_t up_off = (gemm_ws + 255) & ~size_t{255};
+    void* ws = nullptr;
+    st = workspace(up_off + up_bytes, &ws);
+    if (st != QMM_OK) return st;
+    u = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + up_off);
+  }
   st = q4k_matmul(x, gate, out, m, n, k, c.stream);
   if (st == QMM_OK) st = q4k_matmul(x, up, u, m, n, k, c.stream);
   if (st == QMM_OK) st = map_hip(qmm::launch_silu_mul(out, u, out, m * n, c.stream));

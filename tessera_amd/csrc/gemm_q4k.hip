@@ -420,7 +420,7 @@ hipError_t launch_q4k_gemm(const float* a, const uint8_t* w, float* c, void* wor
   }
   const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
   if (n_split > 0) launch_range<256, 256, 128, 64>(a16, a_scale, w, c, m, n, k, 0u, n_split, stream);
-  if (n_split < n) launch_range<128, 64>(a16, a_scale, w, c, m, n, k, n_split, n, stream);
+  if (n_split < n) launch_range<128, 64, 64, 32>(a16, a_scale, w, c, m, n, k, n_split, n, stream);
   return hipGetLastError();
 }
 

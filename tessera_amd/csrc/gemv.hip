@@ -16,7 +16,6 @@
 //     (deterministic, no atomics).
 // Codecs plug the block format into this skeleton.
 
-#include <cstdlib>
 #include <type_traits>
 
 #include "qmm_device.hpp"
@@ -1334,7 +1333,6 @@ struct GemvPlan {
 };
 
 int g_num_cus = 256;
-int g_tune_p = 0;  // QMM_GEMV_P: force rows per group (experiments only)
 
 // Workgroup shape: rows per group P in 1..kMaxP and the thread count P*cpr rounded up
 // to whole wavefronts; picks the P that idles the fewest lanes, larger P on ties
@@ -1366,11 +1364,10 @@ GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads, bool even_p = false) {
     const uint32_t t = (p * cpr + 63u) / 64u * 64u;
     if (t > max_threads) break;
     const double fill = static_cast<double>(p * cpr) / t;
-    if (fill >= best || (g_tune_p != 0 && static_cast<int>(p) == g_tune_p)) {
+    if (fill >= best) {
       best = fill;
       g.p = p;
       g.threads = t;
-      if (g_tune_p != 0 && static_cast<int>(p) == g_tune_p) break;
     }
   }
   return g;
@@ -1504,7 +1501,6 @@ int num_cus() { return g_num_cus; }
 
 void set_num_cus(int cus) {
   g_num_cus = cus > 0 ? cus : 256;
-  if (const char* e = std::getenv("QMM_GEMV_P")) g_tune_p = std::atoi(e);
 }
 
 // K limits of the register-resident mapping: one 16-byte chunk per thread, at most

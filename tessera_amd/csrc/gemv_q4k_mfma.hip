@@ -613,10 +613,6 @@ __global__ __launch_bounds__(64 * kResWaves) void q4k_rows_resident_kernel(
   }
 }
 
-#ifdef QMF_TUNE
-} uint32_t g_force_ks = 0, g_force_kh = 0, g_force_depth = 0; namespace {
-#endif
-bool g_use_resident = true;
 struct MfmaPlan {
   uint32_t ks, kh, nc, xc;
 };
@@ -634,10 +630,6 @@ MfmaPlan plan_for(uint32_t m, uint32_t n, uint32_t k) {
   const uint32_t sbs = k / 256u, want = 2u * static_cast<uint32_t>(num_cus());
   const uint32_t ks_max = p.nc > 2 ? 2u : 4u;
   while (p.ks < ks_max && sbs % (2u * p.ks) == 0 && (n * p.ks * p.kh + 63u) / 64u < want) p.ks *= 2u;
-#ifdef QMF_TUNE
-  if (g_force_ks) p.ks = g_force_ks;
-  if (g_force_kh) p.kh = g_force_kh;
-#endif
   return p;
 }
 
@@ -695,10 +687,7 @@ size_t gemv_q4k_mfma_workspace_bytes(uint64_t m, uint64_t k) {
 
 hipError_t launch_q4k_gemv_mfma(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                                 uint32_t n, uint32_t k, hipStream_t stream) {
-#ifdef QMF_TUNE
-  g_use_resident = g_force_depth != 99;
-#endif
-  if (g_use_resident) {
+  {
     uint32_t per = 0, grid = 0;
     constexpr size_t kLdsMax = 160 * 1024;
     for (uint32_t depth = 3; depth >= 2; --depth) {
@@ -736,21 +725,11 @@ hipError_t launch_q4k_gemv_mfma(const float* a, const uint8_t* w, float* c, void
     launch_cfg<KS_, KH_, NC_, XC_, DEPTH_>(w, xop, inv, c, m, n, k, stream);             \
     return hipGetLastError();                                                            \
   }
-#ifdef QMF_TUNE
-  if (g_force_depth == 6) { QMM_MFMA_CASE(1, 2, 1, 4, 6) QMM_MFMA_CASE(2, 2, 1, 4, 6) QMM_MFMA_CASE(1, 2, 2, 4, 6) QMM_MFMA_CASE(1, 2, 1, 2, 6) }
-  if (g_force_depth == 8) { QMM_MFMA_CASE(1, 2, 1, 4, 8) QMM_MFMA_CASE(2, 2, 1, 4, 7) QMM_MFMA_CASE(1, 2, 2, 4, 7) QMM_MFMA_CASE(1, 2, 1, 2, 8) }
-#endif
   QMM_MFMA_CASE(1, 2, 1, 2, 4) QMM_MFMA_CASE(2, 2, 1, 2, 4) QMM_MFMA_CASE(4, 2, 1, 2, 4)
   QMM_MFMA_CASE(1, 2, 1, 4, 4) QMM_MFMA_CASE(2, 2, 1, 4, 4) QMM_MFMA_CASE(4, 2, 1, 4, 3)
   QMM_MFMA_CASE(1, 2, 2, 4, 4) QMM_MFMA_CASE(2, 2, 2, 4, 3) QMM_MFMA_CASE(4, 2, 2, 4, 2)
   QMM_MFMA_CASE(1, 2, 3, 4, 4) QMM_MFMA_CASE(2, 2, 3, 4, 3)
   QMM_MFMA_CASE(1, 2, 4, 4, 4) QMM_MFMA_CASE(2, 2, 4, 4, 2)
-#ifdef QMF_TUNE
-  QMM_MFMA_CASE(1, 1, 4, 4, 3) QMM_MFMA_CASE(2, 1, 4, 4, 2) QMM_MFMA_CASE(4, 1, 4, 4, 2) QMM_MFMA_CASE(4, 2, 4, 4, 2)
-  QMM_MFMA_CASE(1, 1, 3, 4, 3) QMM_MFMA_CASE(2, 1, 3, 4, 2)
-  QMM_MFMA_CASE(1, 1, 2, 4, 3) QMM_MFMA_CASE(2, 1, 2, 4, 3) QMM_MFMA_CASE(4, 1, 2, 4, 2)
-  QMM_MFMA_CASE(1, 1, 1, 4, 4) QMM_MFMA_CASE(2, 1, 1, 4, 3) QMM_MFMA_CASE(4, 1, 1, 4, 2)
-#endif
 #undef QMM_MFMA_CASE
   return hipErrorInvalidValue;
 }

@@ -193,9 +193,13 @@ __global__ __launch_bounds__(256) void quantize_fp8_pack_kernel(const void* __re
   }
   amax = block_max_256(amax, lds);
   const float s = fmaxf(amax / kE4M3Max, kE4M3MinScale);
-  if (threadIdx.x == 0) scale[blockIdx.x] = s;
+  if (threadIdx.x == 0 && blockIdx.y == 0) scale[blockIdx.x] = s;
   uint32_t* dst = reinterpret_cast<uint32_t*>(out + base);
-  for (uint64_t q = threadIdx.x; q < quads; q += 256) {
+  // grid.y workgroups share a row: each finds the row's maximum for itself (a few tens of KB
+  // from L2) and rounds its own interleaved share of the quads, so the divisions and E4M3
+  // roundings of a long row -- most of this kernel's time when only a few rows exist -- are spread
+  // over several CUs.
+  for (uint64_t q = blockIdx.y * 256ull + threadIdx.x; q < quads; q += 256ull * gridDim.y) {
     float v[4];
     load4(q, v);
     uint32_t word = 0;
@@ -496,16 +500,28 @@ hipError_t launch_quantize_fp8(float* data, float* scale, uint64_t rows, uint64_
   return hipGetLastError();
 }
 
+// Workgroups per row of the pack kernel: one per 1024 columns while the rows alone cannot fill
+// the chip, one otherwise.
+static dim3 quantize_pack_grid(uint64_t rows, uint64_t cols) {
+  uint64_t per_row = 1;
+  if (rows < 256) {
+    per_row = (cols + 1023) / 1024;
+    if (per_row > 16) per_row = 16;
+    if (per_row == 0) per_row = 1;
+  }
+  return dim3(static_cast<uint32_t>(rows), static_cast<uint32_t>(per_row));
+}
+
 hipError_t launch_quantize_fp8_pack(const float* in, uint8_t* out, float* scale, uint64_t rows,
                                     uint64_t cols, hipStream_t stream) {
-  hipLaunchKernelGGL(quantize_fp8_pack_kernel<false>, dim3(static_cast<uint32_t>(rows)), dim3(256),
+  hipLaunchKernelGGL(quantize_fp8_pack_kernel<false>, quantize_pack_grid(rows, cols), dim3(256),
                      0, stream, static_cast<const void*>(in), out, scale, cols);
   return hipGetLastError();
 }
 
 hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float* scale,
                                          uint64_t rows, uint64_t cols, hipStream_t stream) {
-  hipLaunchKernelGGL(quantize_fp8_pack_kernel<true>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0,
+  hipLaunchKernelGGL(quantize_fp8_pack_kernel<true>, quantize_pack_grid(rows, cols), dim3(256), 0,
                      stream, static_cast<const void*>(in), out, scale, cols);
   return hipGetLastError();
 }

@@ -101,11 +101,13 @@ qmm_status workspace(size_t bytes, void** out) {
   return QMM_OK;
 }
 
-// From this many rows on, Q4_K goes to the tiled fp16 MFMA GEMM.  Below it, 2 and more rows of
+// From this many rows on, Q4_K goes to the tiled fp16 MFMA GEMM: one more than the largest
+// speculative-verify batch (16), which stays on the exact fp32-accumulate paths as in the
+// reference (its fp16 tensor-core tile starts at 64 rows).  Below it, 2 and more rows of
 // a matrix with at least kQ4KFewRowsMinWeights weights go, eight at a time, to the exact
 // few-row MFMA kernels (weights read once per eight rows); one row and small matrices stay on
 // the VALU GEMV, which needs no activation pre-pass.
-constexpr uint64_t kQ4KGemmMinRows = 24;
+constexpr uint64_t kQ4KGemmMinRows = 17;
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 

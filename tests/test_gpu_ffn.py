@@ -63,17 +63,17 @@ def test_one_row_matches_oracle(backend, n, k):
     assert rel_err(got, want) < TOL
 
 
-@pytest.mark.parametrize("m,n,k", [(2, 300, 5120), (5, 128, 4096), (16, 64, 2048), (24, 96, 1024), (40, 256, 512)])
+@pytest.mark.parametrize("m,n,k", [(2, 300, 5120), (5, 128, 4096), (16, 64, 2048), (17, 96, 1024), (40, 256, 512)])
 def test_several_rows_match_oracle(backend, m, n, k):
     g = synth.rng(730 + m)
     gate, up = synth.q4k_weights(g, n, k), synth.q4k_weights(g, n, k)
     x = synth.activations_f32(g, m, k)
     got = ffn(backend, x, gate, up, m, n, k)
     want = oracle.ffn_gate_up_silu_q4k(x, gate, up, m, n, k)
-    if m < 24:
+    if m < 17:
         assert rel_err(got, want) < TOL
     else:
-        # From 24 rows on the two products come from the fp16 MFMA GEMM, bounded by
+        # From 17 rows on the two products come from the fp16 MFMA GEMM, bounded by
         # max|dg| <= 4e-3 rms(g) (tests/test_gpu_gemm_q4k.py).  With |silu'| <= 1.1,
         # |d out| <= 1.1 |u| |dg| + |silu(g)| |du| <= (1.1 * 4 + 4) * 4e-3 rms(g) rms(u) for
         # operands within 4 rms, and rms(out) is about 0.7 rms(g) rms(u): 5e-2 of rms(out).

@@ -1,4 +1,4 @@
-"""Q4_K prefill GEMM on fp16 MFMA (the Q4_K GEMM ids from 24 rows on) against the CPU oracle.
+"""Q4_K prefill GEMM on fp16 MFMA (the Q4_K GEMM ids from 17 rows on) against the CPU oracle.
 
 The kernel multiplies fp16 activations by fp16 weights decoded in registers as
 w16 = fma(q, RN16(d*sc), -RN16(dmin*mn)) and accumulates in fp32, like the reference's WMMA
@@ -28,7 +28,7 @@ def gemm(backend, name, a, w, m, n, k):
     return backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
 
 
-SHAPES = [(24, 64, 256), (32, 100, 512), (64, 64, 768), (130, 257, 1024), (256, 256, 2048),
+SHAPES = [(17, 96, 512), (24, 64, 256), (32, 100, 512), (64, 64, 768), (130, 257, 1024), (256, 256, 2048),
           (300, 50, 5120), (100, 600, 1280), (513, 320, 256)]
 
 

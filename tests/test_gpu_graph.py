@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 def test_recorded_decode_step_replays_like_eager(backend):
     dev = torch.device("cuda:0")
     g = synth.rng(900)
-    n, k = 4100, 4096                     # 16.8 M weights: 2..23 rows take the few-row MFMA kernels
+    n, k = 4100, 4096                     # 16.8 M weights: 2..16 rows take the few-row MFMA kernels
     to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     wrap = lambda t: backend.WrapBuffer(t.data_ptr(), t.numel() * t.element_size())
     gate_h, up_h = synth.q4k_weights(g, n, k), synth.q4k_weights(g, n, k)

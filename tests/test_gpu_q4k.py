@@ -114,7 +114,7 @@ def test_rows_kernels(backend, rows):
     assert e.value.code == StatusCode.InvalidArgument
 
 
-# Matrices of 16M weights and more take 2..23 rows through the few-row MFMA kernels (eight rows a
+# Matrices of 16M weights and more take 2..16 rows through the few-row MFMA kernels (eight rows a
 # pass, activations as fp16 hi/lo pairs with a per-row power-of-two scale; up to four rows with
 # the activations resident in LDS when n is a multiple of 4, else streamed per stage); the shapes
 # cover k/256 divisible by 4, by 2 only and odd (the tilings), k/256 not a multiple of 8 (ragged
@@ -124,7 +124,7 @@ FEW_ROW_SHAPES = [(4096, 4096), (2060, 8192), (1030, 17408), (8200, 2048), (7400
 
 
 @pytest.mark.parametrize("n,k", FEW_ROW_SHAPES)
-@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 9, 16, 23])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 9, 12, 16])
 def test_few_rows_match_oracle(backend, n, k, m):
     if m > 9 and (n, k) != FEW_ROW_SHAPES[0]:
         pytest.skip("several passes are covered on the first shape")

@@ -101,12 +101,12 @@ def test_full_size_and_linearity(backend):
         assert rel_err(got, ref) <= TOL, (n, k, rel_err(got, ref))
         got2 = gemm(backend, "gemm_q5k_vec", 2 * a, w, 1, n, k, extra=(1,))[0]
         assert np.array_equal(got2, 2 * got)
-# From 24 rows up the weights are decoded once to fp16 and multiplied on the fp16 MFMA: weights
+# From 17 rows up the weights are decoded once to fp16 and multiplied on the fp16 MFMA: weights
 # carry one rounding of 2^-11, activations a second (per-row scaled), accumulation is fp32.
 RMS_TOL, NORM_TOL = 4e-3, 1e-3
 
 
-@pytest.mark.parametrize("m,n,k", [(24, 300, 512), (64, 512, 1024), (100, 257, 2304), (300, 1000, 5120), (256, 256, 256)])
+@pytest.mark.parametrize("m,n,k", [(17, 300, 512), (64, 512, 1024), (100, 257, 2304), (300, 1000, 5120), (256, 256, 256)])
 def test_prefill_fp16_mfma_matches_oracle(backend, m, n, k):
     from util import norm_err, rms_err
     g = synth.rng(5900 + m + n + k)

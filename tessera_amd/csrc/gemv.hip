@@ -1143,7 +1143,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   const uint32_t last_slot = first_slot + 63u < slots ? first_slot + 63u : slots - 1u;
   const uint32_t row_a = first_slot / cpr, row_b = last_slot / cpr;
   const bool two = row_a != row_b;  // wavefront-uniform
-  const float in_a = (prow == row_a) ? 1.0f : 0.0f, in_b = 1.0f - in_a;
+  // Which sum a lane's partial goes into.  Selected, never multiplied by a 0/1 mask: a NaN or an
+  // infinity among one row's weights must not reach its neighbour's sum (0 * inf = NaN), nor may
+  // what an idle lane computed from the chunk it loaded for company.
+  const bool to_a = valid && prow == row_a, to_b = valid && prow != row_a;
 
   // Groups [g0, g1) belong to this workgroup.  A group index past its end is clamped to its
   // last group for the loads (a prefetch must not pull the next workgroup's rows, which would
@@ -1237,14 +1240,14 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (two) {
-          const float sa = wave_sum_last(v[r] * in_a);
-          const float sb = wave_sum_last(v[r] * in_b);
+          const float sa = wave_sum_last(to_a ? v[r] : 0.0f);
+          const float sb = wave_sum_last(to_b ? v[r] : 0.0f);
           if (lane == 63u) {
             red[buf][d][row_a][r][wave] = sa;
             red[buf][d][row_b][r][wave] = sb;
           }
         } else {
-          const float sa = wave_sum_last(v[r]);
+          const float sa = wave_sum_last(valid ? v[r] : 0.0f);
           if (lane == 63u) red[buf][d][row_a][r][wave] = sa;
         }
       }

@@ -208,6 +208,28 @@ def test_gemm_fp8_one_hot_bit_exact(backend, k):
     assert same_bits_zero_sign_free(backend.CopyD2H(dc, dtype=np.float32).reshape(len(pos), n), ref)
 
 
+@pytest.mark.parametrize("k", [64, 512, 17408])
+def test_gemm_fp8_every_weight_code(backend, k):
+    """All 256 E4M3 codes as weights (one per row, the code repeated along the row), a one-hot
+    activation and unit row scales: the device's conversion against Fp8E4M3ToFloat, through the
+    16-, 32- and 64-weights-a-lane codecs (k selects them); 0x7F and 0xFF are NaN."""
+    n = 256
+    codes = np.repeat(np.arange(n, dtype=np.uint8), k)
+    scales = np.ones(n, np.float32)
+    want = np.array([oracle.fp8_e4m3_to_float(c) for c in range(n)], np.float32)
+    for m, pos in ((1, [k - 1]), (2, [0, k // 2]), (5, [1, 15, 16, 33, k - 2])):
+        x = synth.one_hot_rows(k, pos)
+        da, dw, ds = backend.Upload(x), backend.Upload(codes), backend.Upload(scales)
+        dc = backend.AllocateBuffer(4 * m * n)
+        run(backend, "gemm_fp8", [da, dw, ds, dc], [m, n, k])
+        backend.Synchronize()
+        got = backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
+        nan = np.isnan(want)
+        for r in range(m):
+            assert np.array_equal(np.isnan(got[r]), nan)
+            assert same_bits_zero_sign_free(got[r][~nan], want[~nan]), (k, m, r)
+
+
 def test_full_size_config2(backend):
     """BASELINE config 2 at full size: N=17408, K=5120, M in {1, 4, 16}."""
     g = synth.rng(9090)

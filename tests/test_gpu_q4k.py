@@ -44,6 +44,64 @@ def test_dequant_dump_bit_exact_all_blocks(backend):
     assert same_bits(got, oracle.dequantize_q4k(w))
 
 
+def test_every_fp16_header_value_decodes_as_the_oracle(backend):
+    """All 65536 fp16 bit patterns as d (and, mirrored, as dmin): the device's half-to-float
+    conversion (subnormals, signed zeros, infinities, NaNs) against Fp16ToFloat through the dump
+    and through the production GEMV (one-hot rows, k = 256).  Finite results bit for bit;
+    where the oracle gives NaN the device must give NaN."""
+    g = synth.rng(101)
+    nb = 65536
+    w = synth.q4k_weights(g, nb, 256).reshape(nb, 144)
+    bits = np.arange(nb, dtype=np.uint16)
+    w[:, 0:2] = bits.view(np.uint8).reshape(nb, 2)
+    w[:, 2:4] = bits[::-1].copy().view(np.uint8).reshape(nb, 2)
+    w = w.reshape(-1)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle.dequantize_q4k(w).reshape(nb, 256)
+    dw = backend.Upload(w)
+    out = backend.AllocateBuffer(nb * 1024)
+    run(backend, "dequant_q4k", [dw, out], [nb])
+    backend.Synchronize()
+    got = backend.CopyD2H(out, dtype=np.float32).reshape(nb, 256)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    # the GEMV's own decode: column t of deq(W) for a few t (rows = the 65536 blocks)
+    pos = [0, 31, 32, 200, 255]
+    x = synth.one_hot_rows(256, pos)
+    dx, dc = backend.Upload(x), backend.AllocateBuffer(4 * len(pos) * nb)
+    run(backend, "gemm_q4k", [dx, dw, dc], [len(pos), nb, 256])
+    backend.Synchronize()
+    c = backend.CopyD2H(dc, dtype=np.float32).reshape(len(pos), nb)
+    for r, t in enumerate(pos):
+        ok = np.isfinite(want).all(axis=1)      # a NaN or infinity anywhere in the block spreads through 0 * inf
+        assert same_bits_zero_sign_free(c[r][ok], want[ok, t]), t
+
+
+@pytest.mark.parametrize("k", [1280, 5120, 17408])
+def test_non_finite_weight_row_stays_in_its_row(backend, k):
+    """An infinite d in one row: that row's output is not finite (as in the reference), its
+    neighbours', which share wavefronts and workgroups with it, are untouched."""
+    g = synth.rng(102 + k)
+    n = 67
+    w = synth.q4k_weights(g, n, k).reshape(n, -1)
+    bad = [7, 40, 66]
+    for r in bad:
+        w[r, 144 * (r % (k // 256)):144 * (r % (k // 256)) + 2] = np.array([0x00, 0x7C], np.uint8)   # +inf
+    w = w.reshape(-1)
+    good = [r for r in range(n) if r not in bad]
+    for m in (1, 2, 4):
+        a = synth.activations_f32(g, m, k)
+        da, dw, dc = backend.Upload(a), backend.Upload(w), backend.AllocateBuffer(4 * m * n)
+        run(backend, "gemm_q4k", [da, dw, dc], [m, n, k])
+        backend.Synchronize()
+        got = backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
+        with np.errstate(invalid="ignore", over="ignore"):
+            ref = oracle.gemm_q4k(a, w, m, n, k)
+        assert not np.isfinite(got[:, bad]).any() and not np.isfinite(ref[:, bad]).any()
+        assert rel_err(got[:, good], ref[:, good]) < TOL
+
+
 @pytest.mark.parametrize("k", [256, 512, 1024, 768, 2048, 5120])
 def test_gemv_one_hot_reproduces_dequant_bit_exact(backend, k):
     """A one-hot activation makes the production GEMV return one column of deq(W): the

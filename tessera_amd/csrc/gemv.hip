@@ -1506,14 +1506,19 @@ void set_num_cus(int cus) {
   g_num_cus = cus > 0 ? cus : 256;
 }
 
-// K limits of the register-resident mapping: one 16-byte chunk per thread, at most
-// 1024 threads per row.
-bool gemv_q4k_supported(uint64_t k) { return k % 256 == 0 && k / 32 <= 1024; }  // multi-row limit
-bool gemv_mxfp4_supported(uint64_t k) { return k % 32 == 0 && k / 32 <= 1024; }
-bool gemv_fp8_supported(uint64_t k) { return k % 16 == 0 && (k / 16 <= 1024 || (k % 32 == 0 && k / 32 <= 1024)); }
+// Rows longer than the register-resident mapping holds (one chunk per thread, a row inside one
+// workgroup) take the wave-per-row kernel, correct and untuned: any K of a format's granularity works.
 
 hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                            uint32_t k, hipStream_t stream) {
+  if (k / 32u > 1024u) {   // longer rows than a workgroup holds: one wavefront per weight row, row by row
+    for (uint32_t r = 0; r < m; ++r) {
+      const hipError_t e = launch_gemv_generic<Q4KCodec>(Q4KCodec::Args{a + static_cast<size_t>(r) * k, w, k},
+                                                         c + static_cast<size_t>(r) * n, n, k, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   // A lane keeps the 32 activations of its chunk for every row of the pass in registers: 128
   // registers at four rows, which fits only with two wavefronts per SIMD (workgroups of up to
   // 512 threads, k <= 16384); two rows fit 768-thread workgroups (k <= 24576); beyond that the
@@ -1551,10 +1556,17 @@ hipError_t launch_ffn_gate_up_q4k(const float* x, const uint8_t* gate, const uin
 }
 
 // Q5_K: one row per weight pass (a lane keeps 64 activations and five 16-byte loads per stage).
-bool gemv_q5k_supported(uint64_t k) { return k % 256 == 0 && k / 64 <= 768; }
 
 hipError_t launch_q5k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                            uint32_t k, hipStream_t stream) {
+  if (k / 64u > 768u) {
+    for (uint32_t r = 0; r < m; ++r) {
+      const hipError_t e = launch_gemv_generic<Q5KCodec>(Q5KCodec::Args{a + static_cast<size_t>(r) * k, w, k},
+                                                         c + static_cast<size_t>(r) * n, n, k, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   for (uint32_t r0 = 0; r0 < m; ++r0) {
     Q5KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
     const hipError_t e = launch_gemv_r<Q5KCodec, 1, 768, 3, 9>(args, c + static_cast<size_t>(r0) * n, n, k, n, stream);
@@ -1565,10 +1577,17 @@ hipError_t launch_q5k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
 
 // Q6_K: a lane keeps the 64 activations of its chunk per row in registers, so two rows share a
 // weight pass (k <= 32768) and further rows take further passes.
-bool gemv_q6k_supported(uint64_t k) { return k % 256 == 0 && k / 64 <= 768; }
 
 hipError_t launch_q6k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                            uint32_t k, hipStream_t stream) {
+  if (k / 64u > 768u) {
+    for (uint32_t r = 0; r < m; ++r) {
+      const hipError_t e = launch_gemv_generic<Q6KCodec>(Q6KCodec::Args{a + static_cast<size_t>(r) * k, w, k},
+                                                         c + static_cast<size_t>(r) * n, n, k, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   const uint32_t row_threads = (k / 64u + 63u) / 64u * 64u;
   for (uint32_t r0 = 0; r0 < m;) {
     Q6KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
@@ -1592,6 +1611,14 @@ hipError_t launch_q6k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
 hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                              uint32_t k, hipStream_t stream) {
   const uint8_t* s = w + static_cast<size_t>(n) * k / 2;
+  if (k / 32u > 1024u) {
+    for (uint32_t r = 0; r < m; ++r) {
+      const hipError_t e = launch_gemv_generic<MxFp4Codec>(MxFp4Codec::Args{a + static_cast<size_t>(r) * k, w, s, k},
+                                                           c + static_cast<size_t>(r) * n, n, k, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   // Register budgets as for Q4_K: four or three rows need two wavefronts per SIMD, two rows three.
   const uint32_t row_threads = (k / 32u + 63u) / 64u * 64u;
   for (uint32_t r0 = 0; r0 < m;) {
@@ -1625,6 +1652,14 @@ hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_
 hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
   const uint8_t* s = w + static_cast<size_t>(n) * k / 2;
+  if (k / 32u > 1024u) {
+    for (uint32_t r = 0; r < m; ++r) {
+      const hipError_t e = launch_gemv_generic<MxFp4A8Codec>(
+          MxFp4A8Codec::Args{a8 + static_cast<size_t>(r) * k, as + r, w, s, k}, c + static_cast<size_t>(r) * n, n, k, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   for (uint32_t r0 = 0; r0 < m;) {
     const uint32_t left = m - r0;
     MxFp4A8Codec::Args args{a8 + static_cast<size_t>(r0) * k, as + r0, w, s, k};
@@ -1646,6 +1681,14 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream) {
+  if (k / 32u > 1024u || (k / 16u > 1024u && k % 32u != 0)) {
+    for (uint32_t r = 0; r < m; ++r) {
+      const hipError_t e = launch_gemv_generic<Fp8Codec>(Fp8Codec::Args{a + static_cast<size_t>(r) * k, w, s, k},
+                                                         c + static_cast<size_t>(r) * n, n, k, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   const uint32_t cpr4 = k / 64u;
   if (m == 1 && k % 64u == 0 && cpr4 >= 64u && cpr4 <= 768u) {
     // one row: 64 weights a lane, so the reduction and the loop overhead are paid once per 64

@@ -135,10 +135,6 @@ qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, ui
     return map_hip(qmm::launch_q4k_gemm(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                         static_cast<uint32_t>(k), s));
   }
-  if (!qmm::gemv_q4k_supported(k)) {
-    g_last_error = "Q4_K: k above 32768 is not implemented";
-    return QMM_UNSUPPORTED_FEATURE;
-  }
   return map_hip(qmm::launch_q4k_gemv(a, w, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                       static_cast<uint32_t>(k), s));
 }
@@ -363,10 +359,6 @@ qmm_status q5k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, ui
   if (m >= kQ4KGemmMinRows && qmm::gemm_kquant_f16_supported(m, n, k)) {
     return kquant_prefill(c, 176, m, n, k, split);
   }
-  if (!qmm::gemv_q5k_supported(k)) {
-    g_last_error = "Q5_K: k above 49152 is not implemented";
-    return QMM_UNSUPPORTED_FEATURE;
-  }
   qmm_status st = map_hip(qmm::launch_q5k_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out,
                                                static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                                static_cast<uint32_t>(k), c.stream));
@@ -417,10 +409,6 @@ qmm_status q6k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, ui
   if (m >= kQ4KGemmMinRows && qmm::gemm_kquant_f16_supported(m, n, k)) {
     return kquant_prefill(c, 210, m, n, k, split);
   }
-  if (!qmm::gemv_q6k_supported(k)) {
-    g_last_error = "Q6_K: k above 49152 is not implemented";
-    return QMM_UNSUPPORTED_FEATURE;
-  }
   qmm_status st = map_hip(qmm::launch_q6k_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out,
                                                static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                                static_cast<uint32_t>(k), c.stream));
@@ -466,10 +454,6 @@ qmm_status run_gemm_mxfp4(const LaunchCtx& c) {
       !c.fits(2, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_mxfp4: a buffer is smaller than m, n, k require");
   }
-  if (!qmm::gemv_mxfp4_supported(k)) {
-    g_last_error = "MXFP4: k above 32768 is not implemented";
-    return QMM_UNSUPPORTED_FEATURE;
-  }
   return map_hip(qmm::launch_mxfp4_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2),
                                         static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                         static_cast<uint32_t>(k), c.stream));
@@ -510,10 +494,6 @@ qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
   if (!c.fits(0, static_cast<u128>(m) * k) || !c.fits(1, mxfp4_bytes(n, k)) || !c.fits(2, m * 4) ||
       !c.fits(3, n) || !c.fits(4, region * split)) {
     return bad("gemm_mxfp4_wmma: a buffer is smaller than m, n, k, split require");
-  }
-  if (!qmm::gemv_mxfp4_supported(k)) {
-    g_last_error = "MXFP4: k above 32768 is not implemented";
-    return QMM_UNSUPPORTED_FEATURE;
   }
   float* out = c.ptr<float>(4);
   // Regime: a single row stays on the VALU GEMV; from two rows on the scaled MFMA takes over
@@ -589,10 +569,6 @@ qmm_status run_gemm_fp8(const LaunchCtx& c) {
   if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, static_cast<u128>(n) * k) ||
       !c.fits(2, static_cast<u128>(n) * 4) || !c.fits(3, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_fp8: a buffer is smaller than m, n, k require");
-  }
-  if (!qmm::gemv_fp8_supported(k)) {
-    g_last_error = "gemm_fp8: k must be a multiple of 16 up to 16384 or a multiple of 32 up to 32768";
-    return QMM_UNSUPPORTED_FEATURE;
   }
   return map_hip(qmm::launch_fp8_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
                                       c.ptr<float>(3), static_cast<uint32_t>(m), static_cast<uint32_t>(n),

@@ -14,11 +14,6 @@ void set_num_cus(int cus);
 int num_cus();
 
 // ---- decode GEMV family (gemv.hip) -----------------------------------------
-bool gemv_q4k_supported(uint64_t k);
-bool gemv_q5k_supported(uint64_t k);
-bool gemv_q6k_supported(uint64_t k);
-bool gemv_mxfp4_supported(uint64_t k);
-bool gemv_fp8_supported(uint64_t k);
 
 // C (m x n fp32) = A (m x k fp32) . deq(W)^T, W = n rows of k/256 Q4_K blocks.
 hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n,

@@ -179,6 +179,29 @@ def test_grouped_ffn_matches_oracle(backend, rows, experts, hidden, inter, top_k
     assert np.array_equal(again, got)
 
 
+def test_grouped_ffn_skewed_routing(backend):
+    """Every token to the same two experts (segments of 300 rows, ten row tiles each; all other
+    experts empty), then duplicate and out-of-range ids in a token's list (clamped to the last
+    expert, as the per-row ids do)."""
+    g = synth.rng(4321)
+    rows, experts, hidden, inter, top_k = 300, 9, 512, 256, 2
+    gate, up, down = expert_tensors(g, experts, hidden, inter)
+    x = synth.activations_bf16(g, rows, hidden)
+    ids = np.tile(np.array([[6, 2]], np.uint32), (rows, 1))
+    wts = g.uniform(0.1, 0.9, size=(rows, top_k)).astype(np.float32)
+    ref = oracle.moe_batch_forward_q4k(x, ids, wts, gate, up, down, hidden, inter)
+    got = forward_grouped(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
+    assert rms_err(got, ref) <= 8e-3 and norm_err(got, ref) <= 2e-3
+    odd = ids.copy()
+    odd[0] = [4, 4]                      # the same expert twice
+    odd[1] = [experts + 7, 0]            # out of range: clamped to experts - 1
+    clamped = odd.copy()
+    clamped[1, 0] = experts - 1
+    ref = oracle.moe_batch_forward_q4k(x, clamped, wts, gate, up, down, hidden, inter)
+    got = forward_grouped(backend, x, odd, wts, gate, up, down, hidden, inter, experts)
+    assert rms_err(got, ref) <= 8e-3 and norm_err(got, ref) <= 2e-3
+
+
 @pytest.mark.parametrize("experts,hidden,inter,top_k,rows", [(16, 512, 256, 4, 1), (8, 2048, 512, 8, 1),
                                                               (5, 260, 768, 2, 3), (256, 2048, 512, 8, 2)])
 def test_down_q6k_matches_oracle(backend, experts, hidden, inter, top_k, rows):

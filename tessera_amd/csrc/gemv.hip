@@ -306,6 +306,7 @@ struct Q4KExpertDownCodec : Q4KCodec {
 // ----------------------------------------------------------------------------
 struct Q4KPairCodec {
   using Args = Q4KCodec::Args;
+  static constexpr bool kBalanceSimds = true;  // the decode, not the loads, paces the loop
   template <int R>
   struct X {
     float lo[R][32];
@@ -470,6 +471,7 @@ struct pair_rows<Codec, std::void_t<decltype(Codec::kPairRows)>> : std::bool_con
 // activation returns the reference's dequantized weight bit for bit.
 // ----------------------------------------------------------------------------
 struct Q5KCodec {
+  static constexpr bool kBalanceSimds = true;
   using Args = Q4KCodec::Args;
   template <int R>
   struct X {
@@ -602,6 +604,7 @@ struct Q5KCodec {
 // a one-hot activation returns the reference's dequantized weight bit for bit.
 // ----------------------------------------------------------------------------
 struct Q6KCodec {
+  static constexpr bool kBalanceSimds = true;
   struct Args {
     const float* a;
     const uint8_t* w;
@@ -1137,8 +1140,8 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   const uint32_t prow = valid ? t / cpr : 0u;
   const uint32_t chunk = valid ? t - prow * cpr : 0u;
 
-  // Which of the P rows this wavefront's lanes belong to: at most two, because the
-  // launcher only uses this kernel when a row has at least 64 chunks.
+  // Which of the P rows this wavefront's lanes belong to: at most two, which the launcher
+  // guarantees (a row has at least 64 chunks, or the plan checked every wavefront's span).
   const uint32_t first_slot = wave * 64u;
   const uint32_t last_slot = first_slot + 63u < slots ? first_slot + 63u : slots - 1u;
   const uint32_t row_a = first_slot / cpr, row_b = last_slot / cpr;
@@ -1376,6 +1379,56 @@ GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads, bool even_p = false) {
   return g;
 }
 
+// The same choice for a codec whose loop is bound by its vector arithmetic rather than by the
+// loads (kBalanceSimds): a CU runs its wavefronts on four SIMDs, so ten wavefronts put three on
+// two of them and the launch lasts as long as those.  Cost of a candidate = wavefronts on the
+// fullest SIMD x pipeline stages a workgroup runs; ties go to fewer wavefronts per CU (a shorter
+// prologue), then to fuller wavefronts, then to larger P.  At 17408x5120 Q4_K this picks 6 rows
+// (8 wavefronts, 12 stages) over 8 rows (10 wavefronts, 9 stages): 13.3 us against 13.9.
+template <uint32_t kMaxP>
+GemvPlan plan_gemv_balanced(uint32_t cpr, uint32_t max_threads, uint32_t n, bool even_p) {
+  GemvPlan g{cpr, (cpr + 63u) / 64u * 64u, 1, false};
+  const uint32_t waves_per_simd = (max_threads / 64u + 3u) / 4u;
+  const uint32_t cus = static_cast<uint32_t>(g_num_cus);
+  uint64_t best_cost = ~0ull;
+  uint32_t best_waves = 0;
+  double best_fill = 0.0;
+  for (uint32_t p = even_p ? 2u : 1u; p <= kMaxP; p += even_p ? 2u : 1u) {
+    const uint32_t t = (p * cpr + 63u) / 64u * 64u;
+    if (t > max_threads) break;
+    const uint32_t w = t / 64u;
+    // The kernel lets a wavefront's lanes belong to at most two rows of the group.
+    bool spans_ok = true;
+    for (uint32_t i = 0; i < w && cpr < 64u; ++i) {
+      const uint32_t first = i * 64u, last = first + 63u < p * cpr ? first + 63u : p * cpr - 1u;
+      spans_ok = spans_ok && last / cpr - first / cpr <= 1u;
+    }
+    if (!spans_ok) continue;
+    uint32_t per_cu = (4u * waves_per_simd) / w;
+    if (per_cu == 0) per_cu = 1;
+    const uint32_t pr = even_p ? p / 2u : p;
+    const uint32_t groups = (n + pr - 1u) / pr;
+    uint32_t grid = cus * per_cu;
+    if (grid > groups) grid = groups;
+    const uint32_t per_wg = (groups + grid - 1u) / grid;
+    grid = (groups + per_wg - 1u) / per_wg;
+    const uint32_t resident = (grid + cus - 1u) / cus;
+    const uint32_t cu_waves = w * resident;
+    const uint64_t cost = static_cast<uint64_t>((cu_waves + 3u) / 4u) * per_wg;
+    const double fill = static_cast<double>(p * cpr) / t;
+    const bool better = cost < best_cost ||
+                        (cost == best_cost && (cu_waves < best_waves ||
+                                               (cu_waves == best_waves && fill >= best_fill)));
+    if (better) best_cost = cost, best_waves = cu_waves, best_fill = fill, g.p = p, g.threads = t;
+  }
+  return g;
+}
+
+template <class Codec, class = void>
+struct balance_simds : std::false_type {};
+template <class Codec>
+struct balance_simds<Codec, std::void_t<decltype(Codec::kBalanceSimds)>> : std::bool_constant<Codec::kBalanceSimds> {};
+
 template <class Codec, int R, int MAXT, int D, uint32_t P>
 hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n, uint32_t cpr,
                          uint32_t ldc, uint32_t threads, hipStream_t stream) {
@@ -1411,7 +1464,10 @@ template <class Codec, int R, int MAXT, int D, uint32_t kMaxP = 2>
 hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n, uint32_t k,
                          uint32_t ldc, hipStream_t stream) {
   const uint32_t cpr = Codec::chunks_per_row(k);
-  const GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT, pair_rows<Codec>::value);
+  GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT, pair_rows<Codec>::value);
+  if constexpr (balance_simds<Codec>::value && R == 1) {
+    if (!g.smallk) g = plan_gemv_balanced<kMaxP>(cpr, MAXT, n, pair_rows<Codec>::value);
+  }
   if (pair_rows<Codec>::value && (g.p % 2u != 0 || g.smallk)) return hipErrorInvalidValue;
   if constexpr (!pair_rows<Codec>::value) {
     if (g.smallk) {

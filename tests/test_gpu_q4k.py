@@ -78,14 +78,13 @@ def test_every_fp16_header_value_decodes_as_the_oracle(backend):
         assert same_bits_zero_sign_free(c[r][ok], want[ok, t]), t
 
 
-@pytest.mark.parametrize("k", [1280, 5120, 17408])
-def test_non_finite_weight_row_stays_in_its_row(backend, k):
+@pytest.mark.parametrize("k,n", [(1280, 67), (5120, 67), (17408, 67), (3072, 3001), (2560, 3001), (5120, 6007)])
+def test_non_finite_weight_row_stays_in_its_row(backend, k, n):
     """An infinite d in one row: that row's output is not finite (as in the reference), its
     neighbours', which share wavefronts and workgroups with it, are untouched."""
     g = synth.rng(102 + k)
-    n = 67
     w = synth.q4k_weights(g, n, k).reshape(n, -1)
-    bad = [7, 40, 66]
+    bad = [7, 40, 66] if n == 67 else [7, 40, 66, 1001, 1002, n - 2]
     for r in bad:
         w[r, 144 * (r % (k // 256)):144 * (r % (k // 256)) + 2] = np.array([0x00, 0x7C], np.uint8)   # +inf
     w = w.reshape(-1)
@@ -121,6 +120,20 @@ def test_gemv_one_hot_reproduces_dequant_bit_exact(backend, k):
 
 SHAPES = [(64, 256), (33, 512), (100, 1024), (17, 768), (129, 1280), (256, 2048), (130, 5120),
           (67, 17408), (40, 4352), (1, 256), (5, 32768)]
+
+
+@pytest.mark.parametrize("n,k", [(3001, 768), (3003, 1280), (2999, 1536), (3005, 2560), (4099, 3072), (3002, 3584),
+                                 (3001, 4352), (6007, 5120), (2051, 6400), (1027, 8192), (523, 17408)])
+def test_single_row_over_many_output_columns(backend, n, k):
+    """One activation row against enough weight rows that a workgroup takes several rows side by
+    side (which count depends on how K/64 divides into wavefronts, including rows shorter than a
+    wavefront whose lanes then belong to two weight rows); ragged last group."""
+    g = synth.rng(31 * n + k)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, 1, k)
+    ref = oracle.gemm_q4k(a, w, 1, n, k, threads=True)
+    got = gemm(backend, "gemm_q4k", a, w, 1, n, k)[0]
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
 @pytest.mark.parametrize("n,k", SHAPES)

@@ -56,6 +56,20 @@ SHAPES = [(64, 256), (33, 512), (100, 1024), (17, 768), (129, 1280), (256, 2048)
           (67, 17408), (40, 4352), (1, 256), (5, 32768), (3, 49152)]
 
 
+@pytest.mark.parametrize("n,k", [(3001, 768), (3003, 1280), (2999, 1536), (3005, 2560), (4099, 3072), (3002, 3584),
+                                 (3001, 4352), (6007, 5120), (2051, 6400), (1027, 8192), (523, 17408)])
+def test_single_row_over_many_output_columns(backend, n, k):
+    """One activation row against enough weight rows that a workgroup takes several rows side by
+    side (which count depends on how K/64 divides into wavefronts, including rows shorter than a
+    wavefront whose lanes then belong to two weight rows); ragged last group."""
+    g = synth.rng(31 * n + k)
+    w = synth.q5k_weights(g, n, k)
+    a = synth.activations_f32(g, 1, k)
+    ref = oracle.gemm_q5k(a, w, 1, n, k, threads=True)
+    got = gemm(backend, "gemm_q5k", a, w, 1, n, k)[0]
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
 @pytest.mark.parametrize("n,k", SHAPES)
 @pytest.mark.parametrize("m", [1, 2, 3, 5, 16])
 def test_gemm_q5k_matches_oracle(backend, n, k, m):

@@ -1126,12 +1126,17 @@ using Fp8QuadCodec = Fp8CodecT<4>;   // one activation row: 64 weights a lane
 // per-wavefront partial sums; a few threads then add them in wavefront order and
 // store (deterministic, no atomics).
 // ----------------------------------------------------------------------------
-template <class Codec, int R, int P, int D, int MAXT, uint32_t XP>
+template <class Codec, int R, int P, int D, int MAXT, uint32_t XP, bool LR = false>
 __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, float* __restrict__ c,
                                                     uint32_t n, uint32_t cpr, uint32_t ldc,
                                                     uint32_t groups_per_wg) {
+  // LR (rows shorter than a wavefront, whose lanes may then belong to three or more rows): a
+  // lane leaves its partial in LDS and sixteen lanes per output add a row's partials after the
+  // barrier.  Otherwise each wavefront reduces its (at most two) rows itself, which is faster
+  // when rows are long.
   constexpr int kMaxWaves = MAXT / kWave;
-  __shared__ float red[2][D][P][R][kMaxWaves];
+  __shared__ float red[2][D][P][R][LR ? 1 : kMaxWaves];
+  __shared__ float part[2][D][R][LR ? MAXT : 1];
 
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -1140,8 +1145,8 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   const uint32_t prow = valid ? t / cpr : 0u;
   const uint32_t chunk = valid ? t - prow * cpr : 0u;
 
-  // Which of the P rows this wavefront's lanes belong to: at most two, which the launcher
-  // guarantees (a row has at least 64 chunks, or the plan checked every wavefront's span).
+  // Which of the P rows this wavefront's lanes belong to: at most two when a row has at least
+  // 64 chunks (shorter rows take the LR path, which does not use these).
   const uint32_t first_slot = wave * 64u;
   const uint32_t last_slot = first_slot + 63u < slots ? first_slot + 63u : slots - 1u;
   const uint32_t row_a = first_slot / cpr, row_b = last_slot / cpr;
@@ -1233,7 +1238,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // fragment they consume (unconditionally, so the compiler can count outstanding loads
   // exactly and never waits for more than the one fragment it needs); the last round
   // loads nothing and skips stages past the range.
-  auto round = [&](uint32_t g, auto refill) {
+  auto round_wave = [&](uint32_t g, auto refill) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       if (!decltype(refill)::value && g + d >= g1) break;
@@ -1274,6 +1279,45 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       }
     }
     buf ^= 1u;
+  };
+
+  auto round_lds = [&](uint32_t g, auto refill) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      if (!decltype(refill)::value && g + d >= g1) break;
+      float v[R];
+      Codec::template dot<R>(frag[d], x, v);
+      if constexpr (decltype(refill)::value) fetch(g + D + d, frag[d]);
+      // Selected, never multiplied by a 0/1 mask (see to_a above).
+#pragma unroll
+      for (int r = 0; r < R; ++r) part[buf][d][r][t] = valid ? v[r] : 0.0f;
+    }
+    lds_barrier();  // LDS only: the prefetched global loads stay in flight across it
+    for (uint32_t o = t >> 4; o < D * PR * R; o += blockDim.x >> 4) {
+      const uint32_t d = o / (PR * R), po = (o / R) % PR, r = o % R;
+      const uint32_t row = (g + d) * PR + po;
+      const bool live = g + d < g1 && row < n;
+      auto slot_sum = [&](uint32_t p) {
+        const float* src = &part[buf][d][r][p * cpr];
+        float sum = 0.0f;
+        if (live) {
+          for (uint32_t i = t & 15u; i < cpr; i += 16u) sum += src[i];
+        }
+        return row16_sum(sum);
+      };
+      float res;
+      if constexpr (kPaired) {
+        const float first = slot_sum(2u * po), second = slot_sum(2u * po + 1u);
+        res = Codec::combine(first, second);
+      } else {
+        res = Codec::template finish<R>(args, live ? row : 0u, r, slot_sum(po));
+      }
+      if (live && (t & 15u) == 0u) c[static_cast<size_t>(r) * ldc + row] = res;
+    }
+    buf ^= 1u;
+  };
+  auto round = [&](uint32_t g, auto refill) {
+    if constexpr (LR) round_lds(g, refill); else round_wave(g, refill);
   };
 
   uint32_t g = g0;
@@ -1397,13 +1441,6 @@ GemvPlan plan_gemv_balanced(uint32_t cpr, uint32_t max_threads, uint32_t n, bool
     const uint32_t t = (p * cpr + 63u) / 64u * 64u;
     if (t > max_threads) break;
     const uint32_t w = t / 64u;
-    // The kernel lets a wavefront's lanes belong to at most two rows of the group.
-    bool spans_ok = true;
-    for (uint32_t i = 0; i < w && cpr < 64u; ++i) {
-      const uint32_t first = i * 64u, last = first + 63u < p * cpr ? first + 63u : p * cpr - 1u;
-      spans_ok = spans_ok && last / cpr - first / cpr <= 1u;
-    }
-    if (!spans_ok) continue;
     uint32_t per_cu = (4u * waves_per_simd) / w;
     if (per_cu == 0) per_cu = 1;
     const uint32_t pr = even_p ? p / 2u : p;
@@ -1455,6 +1492,11 @@ hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n,
       return hipGetLastError();
     }
   }
+  if (cpr < 64u) {
+    hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall, true>), dim3(grid), dim3(threads), 0,
+                       stream, args, c, n, cpr, ldc, per_wg);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall>), dim3(grid), dim3(threads), 0, stream,
                      args, c, n, cpr, ldc, per_wg);
   return hipGetLastError();
@@ -1465,8 +1507,10 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
                          uint32_t ldc, hipStream_t stream) {
   const uint32_t cpr = Codec::chunks_per_row(k);
   GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT, pair_rows<Codec>::value);
-  if constexpr (balance_simds<Codec>::value && R == 1) {
-    if (!g.smallk) g = plan_gemv_balanced<kMaxP>(cpr, MAXT, n, pair_rows<Codec>::value);
+  // Rows shorter than a wavefront (and not of the small-K kernel's lengths) also go side by
+  // side in a workgroup: plan_gemv would give each a workgroup of one partly idle wavefront.
+  if (!g.smallk && ((balance_simds<Codec>::value && R == 1) || cpr < 64u)) {
+    g = plan_gemv_balanced<kMaxP>(cpr, MAXT, n, pair_rows<Codec>::value);
   }
   if (pair_rows<Codec>::value && (g.p % 2u != 0 || g.smallk)) return hipErrorInvalidValue;
   if constexpr (!pair_rows<Codec>::value) {

@@ -111,6 +111,16 @@ __device__ __forceinline__ float wave_sum_last(float v) {
   return v;
 }
 
+// Sum over each aligned run of 16 lanes (a DPP row); every lane of the run returns its total.
+// A run must be active or idle as a whole.
+__device__ __forceinline__ float row16_sum(float v) {
+  v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_add<0x140, 0xF>(v);  // row_mirror
+  return v;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {

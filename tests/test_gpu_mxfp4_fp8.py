@@ -68,6 +68,36 @@ def test_gemm_mxfp4_matches_oracle(backend, n, k, m):
     assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
+@pytest.mark.parametrize("n,k", [(3001, 96), (3003, 352), (2999, 768), (3001, 1280), (3005, 2560), (4099, 3072),
+                                 (3002, 3584), (6007, 5120), (1027, 8192)])
+@pytest.mark.parametrize("m", [1, 2, 4])
+def test_mxfp4_many_output_columns(backend, n, k, m):
+    """Enough weight rows that a workgroup takes several side by side, including rows shorter than
+    a wavefront (lanes of one wavefront then belong to several weight rows); ragged last group."""
+    g = synth.rng(37 * n + k + m)
+    w = synth.mxfp4_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_mxfp4(a, w, m, n, k)
+    got = mx_gemm(backend, "gemm_mxfp4" if m == 1 else "gemm_mxfp4_rows", a, w, m, n, k)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
+@pytest.mark.parametrize("n,k", [(3001, 80), (3003, 352), (2999, 768), (3001, 1280), (3005, 2560), (4099, 3072),
+                                 (3002, 3584), (6007, 5120), (1027, 8192)])
+@pytest.mark.parametrize("m", [1, 2, 4])
+def test_fp8_many_output_columns(backend, n, k, m):
+    g = synth.rng(41 * n + k + m)
+    codes, scales = synth.fp8_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_fp8(a, codes, scales, m, n, k)
+    da, dw, ds = backend.Upload(a), backend.Upload(codes), backend.Upload(scales)
+    dc = backend.AllocateBuffer(4 * m * n)
+    run(backend, "gemm_fp8", [da, dw, ds, dc], [m, n, k], grid=((m * n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
 def quant_inputs(g, rows, cols):
     x = synth.activations_bf16_outliers(g, rows, cols)
     if rows > 2:

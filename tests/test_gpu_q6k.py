@@ -71,6 +71,17 @@ def test_single_row_over_many_output_columns(backend, n, k):
     assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
+@pytest.mark.parametrize("n,k", [(3001, 768), (2999, 1536), (3005, 2560), (4099, 3072), (3002, 3584), (1030, 5120)])
+@pytest.mark.parametrize("m", [2, 3, 4])
+def test_few_rows_over_many_output_columns(backend, n, k, m):
+    g = synth.rng(43 * n + k + m)
+    w = synth.q6k_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_q6k(a, w, m, n, k, threads=True)
+    got = gemm(backend, "gemm_q6k", a, w, m, n, k)[0]
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
 @pytest.mark.parametrize("n,k", SHAPES)
 @pytest.mark.parametrize("m", [1, 2, 3, 5, 16])
 def test_gemm_q6k_matches_oracle(backend, n, k, m):

@@ -1191,21 +1191,26 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
     if (R == 1 && k <= kPiece && k <= kXPer * 4u * blockDim.x) {   // uniform
       // Short single row: its loads are requested BEFORE the weight prefetch.  Loads return in
       // order, so requested after it they would sit behind D fragments per lane (over 100 KB
-      // per workgroup) and the first dot product would start microseconds later.
+      // per workgroup) and the first dot product would start microseconds later.  Only the
+      // first stage of weights is requested before the barrier, the others right after it: with
+      // all D requested up front, the slowest wavefront's activations arrive behind everybody
+      // else's burst (a third of a 50 MB matrix), the barrier opens when the burst has drained
+      // and the memory system idles while the first stage is computed (3-4 % per launch).
       float4 xr[kXPer];
 #pragma unroll
       for (int i = 0; i < kXPer; ++i) {
         const uint32_t e = (t + i * blockDim.x) * 4u;
         xr[i] = *reinterpret_cast<const float4*>(args.a + (e < k ? e : k - 4u));
       }
-#pragma unroll
-      for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
+      fetch(g0, frag[0]);
 #pragma unroll
       for (int i = 0; i < kXPer; ++i) {
         const uint32_t e = (t + i * blockDim.x) * 4u;
         if (e < k) *reinterpret_cast<float4*>(&xs[StagedX::pad(e)]) = xr[i];
       }
       lds_barrier();
+#pragma unroll
+      for (int d = 1; d < D; ++d) fetch(g0 + d, frag[d]);
       Codec::template load_x<R>(args, chunk, valid, x, StagedX{xs, 0u, kStride});
     } else {
       // Weight loads first, activations second: both are in flight before anything waits.

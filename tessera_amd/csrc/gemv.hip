@@ -1642,7 +1642,9 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     } else if (left >= 2 && row_threads <= 768u) {
       e = launch_gemv_r<Q4KCodec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<Q4KPairCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
+      // Two fragments in flight per lane: a third makes the opening burst larger and the
+      // launch longer (5120x17408 16.3 us against 15.1; 17408x5120 the same within noise).
+      e = launch_gemv_r<Q4KPairCodec, 1, 768, 2, 9>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;
@@ -1657,7 +1659,7 @@ bool ffn_gate_up_q4k_supported(uint64_t k) { return k % 256 == 0 && k >= 4096 &&
 hipError_t launch_ffn_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up, float* out,
                                   uint32_t n, uint32_t k, hipStream_t stream) {
   Q4KGateUpCodec::Args args{x, gate, k, up};
-  return launch_gemv_r<Q4KGateUpCodec, 1, 768, 3, 8>(args, out, n, k, n, stream);
+  return launch_gemv_r<Q4KGateUpCodec, 1, 768, 2, 8>(args, out, n, k, n, stream);
 }
 
 // Q5_K: one row per weight pass (a lane keeps 64 activations and five 16-byte loads per stage).
@@ -1674,7 +1676,7 @@ hipError_t launch_q5k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
   }
   for (uint32_t r0 = 0; r0 < m; ++r0) {
     Q5KCodec::Args args{a + static_cast<size_t>(r0) * k, w, k};
-    const hipError_t e = launch_gemv_r<Q5KCodec, 1, 768, 3, 9>(args, c + static_cast<size_t>(r0) * n, n, k, n, stream);
+    const hipError_t e = launch_gemv_r<Q5KCodec, 1, 768, 2, 9>(args, c + static_cast<size_t>(r0) * n, n, k, n, stream);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
@@ -1705,7 +1707,7 @@ hipError_t launch_q6k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
       // dispatch (two rows of 17408 x 5120: 38 us with depth 2, 29 us with depth 1).
       e = launch_gemv_r<Q6KCodec, 2, 512, 1, 6>(args, out, n, k, n, stream), took = 2;
     } else {
-      e = launch_gemv_r<Q6KCodec, 1, 768, 3, 9>(args, out, n, k, n, stream), took = 1;
+      e = launch_gemv_r<Q6KCodec, 1, 768, 2, 9>(args, out, n, k, n, stream), took = 1;
     }
     if (e != hipSuccess) return e;
     r0 += took;
@@ -1743,7 +1745,7 @@ hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_
       e = hipErrorInvalidValue;
       const uint32_t cpr2 = k / 64u;
       if (k % 64u == 0 && !(cpr2 == 4 || cpr2 == 8 || cpr2 == 16 || cpr2 == 32)) {
-        e = launch_gemv_r<MxFp4PairCodec, 1, 768, 3, 9>(args, out, n, k, n, stream);
+        e = launch_gemv_r<MxFp4PairCodec, 1, 768, 2, 9>(args, out, n, k, n, stream);
       }
       if (e == hipErrorInvalidValue) e = launch_gemv_r<MxFp4Codec, 1, 1024, 4>(args, out, n, k, n, stream);
       took = 1;
@@ -1798,7 +1800,7 @@ hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, flo
   if (m == 1 && k % 64u == 0 && cpr4 >= 64u && cpr4 <= 768u) {
     // one row: 64 weights a lane, so the reduction and the loop overhead are paid once per 64
     Fp8QuadCodec::Args args{a, w, s, k};
-    return launch_gemv_r<Fp8QuadCodec, 1, 768, 3, 9>(args, c, n, k, n, stream);
+    return launch_gemv_r<Fp8QuadCodec, 1, 768, 2, 9>(args, c, n, k, n, stream);
   }
   if (k / 16u > 1024u) {
     // rows of 16385..32768 weights: 32 weights a lane, one or two activation rows per weight pass

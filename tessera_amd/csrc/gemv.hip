@@ -855,6 +855,7 @@ struct MxFp4Codec {
 // thread, so the reduction, the scale loads and the loop overhead are paid once per 64 weights
 // (as Q4KPairCodec does for Q4_K).  K must be a multiple of 64.
 struct MxFp4PairCodec {
+  static constexpr bool kBalanceSimds = true;
   using Args = MxFp4Codec::Args;
   template <int R>
   struct X {
@@ -1431,16 +1432,16 @@ GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads, bool even_p = false) {
 // The same choice for a codec whose loop is bound by its vector arithmetic rather than by the
 // loads (kBalanceSimds): a CU runs its wavefronts on four SIMDs, so ten wavefronts put three on
 // two of them and the launch lasts as long as those.  Cost of a candidate = wavefronts on the
-// fullest SIMD x pipeline stages a workgroup runs; ties go to fewer wavefronts per CU (a shorter
-// prologue), then to fuller wavefronts, then to larger P.  At 17408x5120 Q4_K this picks 6 rows
-// (8 wavefronts, 12 stages) over 8 rows (10 wavefronts, 9 stages): 13.3 us against 13.9.
+// fullest SIMD x pipeline stages a workgroup runs; ties are ranked in the loop below, then go
+// to fuller wavefronts, then to larger P.  At 17408x5120 Q4_K this picks 9 rows (12 wavefronts,
+// 8 stages) over 8 rows (10 wavefronts, 9 stages).
 template <uint32_t kMaxP>
 GemvPlan plan_gemv_balanced(uint32_t cpr, uint32_t max_threads, uint32_t n, bool even_p) {
   GemvPlan g{cpr, (cpr + 63u) / 64u * 64u, 1, false};
   const uint32_t waves_per_simd = (max_threads / 64u + 3u) / 4u;
   const uint32_t cus = static_cast<uint32_t>(g_num_cus);
   uint64_t best_cost = ~0ull;
-  uint32_t best_waves = 0;
+  uint32_t best_rank = 0;
   double best_fill = 0.0;
   for (uint32_t p = even_p ? 2u : 1u; p <= kMaxP; p += even_p ? 2u : 1u) {
     const uint32_t t = (p * cpr + 63u) / 64u * 64u;
@@ -1458,10 +1459,14 @@ GemvPlan plan_gemv_balanced(uint32_t cpr, uint32_t max_threads, uint32_t n, bool
     const uint32_t cu_waves = w * resident;
     const uint64_t cost = static_cast<uint64_t>((cu_waves + 3u) / 4u) * per_wg;
     const double fill = static_cast<double>(p * cpr) / t;
+    // Among equal costs: a long loop (four stages or more) likes one workgroup per CU with as
+    // many wavefronts as fit (17408x5120: 9 rows, 12 wavefronts, 12.3 us; 6 rows, 8 wavefronts,
+    // 12.9); a short one is mostly prologue and likes few wavefronts.
+    const uint32_t rank = per_wg >= 4u ? (resident == 1u ? 100u : 0u) + cu_waves : 1000u - cu_waves;
     const bool better = cost < best_cost ||
-                        (cost == best_cost && (cu_waves < best_waves ||
-                                               (cu_waves == best_waves && fill >= best_fill)));
-    if (better) best_cost = cost, best_waves = cu_waves, best_fill = fill, g.p = p, g.threads = t;
+                        (cost == best_cost && (rank > best_rank ||
+                                               (rank == best_rank && fill >= best_fill)));
+    if (better) best_cost = cost, best_rank = rank, best_fill = fill, g.p = p, g.threads = t;
   }
   return g;
 }

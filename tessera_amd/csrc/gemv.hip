@@ -1522,7 +1522,10 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
   GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT, pair_rows<Codec>::value);
   // Rows shorter than a wavefront (and not of the small-K kernel's lengths) also go side by
   // side in a workgroup: plan_gemv would give each a workgroup of one partly idle wavefront.
-  if (!g.smallk && ((balance_simds<Codec>::value && R == 1) || cpr < 64u)) {
+  // Several activation rows make every codec's loop arithmetic-bound (a multiply-add per weight
+  // and row), so those are planned by SIMD load as well: MXFP4 with four fp32 rows went from 2
+  // rows a workgroup (5 wavefronts: 2,1,1,1 on the SIMDs) to 3 (8 wavefronts), 42.5 -> 32.4 us.
+  if (!g.smallk && ((balance_simds<Codec>::value && R == 1) || cpr < 64u || R > 1)) {
     g = plan_gemv_balanced<kMaxP>(cpr, MAXT, n, pair_rows<Codec>::value);
   }
   if (pair_rows<Codec>::value && (g.p % 2u != 0 || g.smallk)) return hipErrorInvalidValue;
@@ -1644,11 +1647,11 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
     hipError_t e;
     uint32_t took;
     if (left >= 4 && row_threads <= 512u) {
-      e = launch_gemv_r<Q4KCodec, 4, 512, 2>(args, out, n, k, n, stream), took = 4;
+      e = launch_gemv_r<Q4KCodec, 4, 512, 2, 6>(args, out, n, k, n, stream), took = 4;
     } else if (left == 3 && row_threads <= 512u) {
-      e = launch_gemv_r<Q4KCodec, 3, 512, 2>(args, out, n, k, n, stream), took = 3;
+      e = launch_gemv_r<Q4KCodec, 3, 512, 2, 6>(args, out, n, k, n, stream), took = 3;
     } else if (left >= 2 && row_threads <= 768u) {
-      e = launch_gemv_r<Q4KCodec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
+      e = launch_gemv_r<Q4KCodec, 2, 768, 2, 6>(args, out, n, k, n, stream), took = 2;
     } else {
       // Two fragments in flight per lane: a third makes the opening burst larger and the
       // launch longer (5120x17408 16.3 us against 15.1; 17408x5120 the same within noise).
@@ -1743,11 +1746,11 @@ hipError_t launch_mxfp4_gemv(const float* a, const uint8_t* w, float* c, uint32_
     hipError_t e;
     uint32_t took;
     if (left >= 4 && row_threads <= 512u) {
-      e = launch_gemv_r<MxFp4Codec, 4, 512, 2>(args, out, n, k, n, stream), took = 4;
+      e = launch_gemv_r<MxFp4Codec, 4, 512, 2, 6>(args, out, n, k, n, stream), took = 4;
     } else if (left == 3 && row_threads <= 512u) {
-      e = launch_gemv_r<MxFp4Codec, 3, 512, 2>(args, out, n, k, n, stream), took = 3;
+      e = launch_gemv_r<MxFp4Codec, 3, 512, 2, 6>(args, out, n, k, n, stream), took = 3;
     } else if (left >= 2 && row_threads <= 768u) {
-      e = launch_gemv_r<MxFp4Codec, 2, 768, 2>(args, out, n, k, n, stream), took = 2;
+      e = launch_gemv_r<MxFp4Codec, 2, 768, 2, 6>(args, out, n, k, n, stream), took = 2;
     } else {
       // one row: 64 weights a lane where K allows (and the row is long enough for the main kernel)
       e = hipErrorInvalidValue;
@@ -1782,9 +1785,9 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
     hipError_t e;
     uint32_t took;
     if (left >= 4) {
-      e = launch_gemv_r<MxFp4A8Codec, 4, 1024, 2>(args, out, n, k, n, stream), took = 4;
+      e = launch_gemv_r<MxFp4A8Codec, 4, 1024, 2, 6>(args, out, n, k, n, stream), took = 4;
     } else if (left >= 2) {
-      e = launch_gemv_r<MxFp4A8Codec, 2, 1024, 4>(args, out, n, k, n, stream), took = 2;
+      e = launch_gemv_r<MxFp4A8Codec, 2, 1024, 4, 6>(args, out, n, k, n, stream), took = 2;
     } else {
       e = launch_gemv_r<MxFp4A8Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
     }
@@ -1834,9 +1837,9 @@ hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, flo
     hipError_t e;
     uint32_t took;
     if (left >= 4) {
-      e = launch_gemv_r<Fp8Codec, 4, 1024, 2>(args, out, n, k, n, stream), took = 4;
+      e = launch_gemv_r<Fp8Codec, 4, 1024, 2, 6>(args, out, n, k, n, stream), took = 4;
     } else if (left >= 2) {
-      e = launch_gemv_r<Fp8Codec, 2, 1024, 4>(args, out, n, k, n, stream), took = 2;
+      e = launch_gemv_r<Fp8Codec, 2, 1024, 4, 6>(args, out, n, k, n, stream), took = 2;
     } else {
       e = launch_gemv_r<Fp8Codec, 1, 1024, 4>(args, out, n, k, n, stream), took = 1;
     }

@@ -721,6 +721,22 @@ __global__ __launch_bounds__(256) void moe_silu_mul_kernel(const float* __restri
   if (threadIdx.x == 0) scale[blockIdx.x] = s;
 }
 
+// phi[p][j] = silu(g[pos[p]][j]) * u[pos[p]][j]: the grouped gate and up products of (token,
+// slot) pair p, which sit at sorted row pos[p], back in the caller's pair order as fp32.
+__global__ __launch_bounds__(256) void moe_silu_scatter_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                               const uint32_t* __restrict__ pos,
+                                                               float* __restrict__ phi, uint32_t inter) {
+  const size_t src = static_cast<size_t>(pos[blockIdx.x]) * inter, dst = static_cast<size_t>(blockIdx.x) * inter;
+  const float4* gp = reinterpret_cast<const float4*>(g + src);
+  const float4* up = reinterpret_cast<const float4*>(u + src);
+  float4* out = reinterpret_cast<float4*>(phi + dst);
+  auto f = [](float gv, float uv) { return (gv / (1.0f + expf(-gv))) * uv; };
+  for (uint32_t q = threadIdx.x; q < inter / 4u; q += 256u) {
+    const float4 a = gp[q], b = up[q];
+    out[q] = make_float4(f(a.x, b.x), f(a.y, b.y), f(a.z, b.z), f(a.w, b.w));
+  }
+}
+
 // out[t][j] (+)= sum_slot wts[t][slot] * rows[pos[t*top_k + slot]][j], slots in order.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, const uint32_t* __restrict__ pos,
                                                           const float* __restrict__ wts, float* __restrict__ out,
@@ -782,6 +798,70 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
   hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((inter + BN - 1) / BN) * 2u), dim3(BN * 2), 0,
                      stream, a16, x_scale, gate, g, seg, gate_stride, inter, hidden, experts, 2u, up, u, up_stride);
   hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(pairs), dim3(256), 0, stream, g, u, phi16, phi_scale, inter);
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((hidden + BN - 1) / BN)), dim3(BN * 2), 0,
+                     stream, phi16, phi_scale, down, rows, seg, down_stride, hidden, inter, experts, 1u, nullptr, nullptr,
+                     uint64_t{0});
+  const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, rows, pos,
+                     wts, out, tokens, top_k, hidden, accumulate);
+  return hipGetLastError();
+}
+
+// The two halves of launch_moe_ffn_q4k behind the reference's own pair of ids
+// ("moe_experts_gate_up_q4k_rows" then "moe_experts_down_q4k_rows",
+// src/backends/rocm/rocm_kernels_moe.cpp:15-79) for a chunk of tokens: each sorts the pairs by
+// expert, gathers its operand as fp16 rows and runs the grouped GEMM, so an expert's weights are
+// read once per launch instead of once per token that chose it.  phi keeps the caller's layout
+// (tokens x top_k x inter, fp32) between the two.  Workspace as for launch_moe_ffn_q4k.
+hipError_t launch_moe_gate_up_q4k_grouped(const float* x, const uint8_t* gate, const uint8_t* up, const uint32_t* ids,
+                                          float* phi, void* workspace, uint32_t hidden, uint32_t inter, uint32_t top_k,
+                                          uint64_t gate_stride, uint64_t up_stride, uint32_t experts, uint32_t tokens,
+                                          hipStream_t stream) {
+  const uint32_t pairs = tokens * top_k;
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  uint32_t* seg = reinterpret_cast<uint32_t*>(ws);
+  ws += align256((static_cast<size_t>(experts) + 1) * 4);
+  uint32_t* pos = reinterpret_cast<uint32_t*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * 4);
+  float* x_scale = reinterpret_cast<float*>(ws);
+  ws += align256((static_cast<size_t>(pairs) + 256) * 4);
+  _Float16* a16 = reinterpret_cast<_Float16*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * hidden * 2);
+  float* g = reinterpret_cast<float*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * inter * 4);
+  float* u = reinterpret_cast<float*>(ws);
+
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, seg, pos);
+  hipLaunchKernelGGL(rows_to_f16_kernel, dim3(pairs), dim3(256), 0, stream, x, a16, x_scale, hidden, pos, top_k);
+  constexpr int BM = 32, BN = 64;
+  const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((inter + BN - 1) / BN) * 2u), dim3(BN * 2), 0,
+                     stream, a16, x_scale, gate, g, seg, gate_stride, inter, hidden, experts, 2u, up, u, up_stride);
+  hipLaunchKernelGGL(moe_silu_scatter_kernel, dim3(pairs), dim3(256), 0, stream, g, u, pos, phi, inter);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_down_q4k_grouped(const float* phi, const uint8_t* down, const uint32_t* ids, const float* wts,
+                                       float* out, void* workspace, uint32_t hidden, uint32_t inter, uint32_t top_k,
+                                       uint64_t down_stride, uint32_t experts, uint32_t tokens, bool accumulate,
+                                       hipStream_t stream) {
+  const uint32_t pairs = tokens * top_k;
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  uint32_t* seg = reinterpret_cast<uint32_t*>(ws);
+  ws += align256((static_cast<size_t>(experts) + 1) * 4);
+  uint32_t* pos = reinterpret_cast<uint32_t*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * 4);
+  float* phi_scale = reinterpret_cast<float*>(ws);
+  ws += align256((static_cast<size_t>(pairs) + 256) * 4);
+  _Float16* phi16 = reinterpret_cast<_Float16*>(ws);
+  ws += align256(static_cast<size_t>(pairs) * inter * 2);
+  float* rows = reinterpret_cast<float*>(ws);
+
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, seg, pos);
+  // source row of pair p is p itself (phi is pair-major): top_k = 1 in the gather
+  hipLaunchKernelGGL(rows_to_f16_kernel, dim3(pairs), dim3(256), 0, stream, phi, phi16, phi_scale, inter, pos, 1u);
+  constexpr int BM = 32, BN = 64;
+  const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
   hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((hidden + BN - 1) / BN)), dim3(BN * 2), 0,
                      stream, phi16, phi_scale, down, rows, seg, down_stride, hidden, inter, experts, 1u, nullptr, nullptr,
                      uint64_t{0});

@@ -595,6 +595,8 @@ qmm_status run_moe_scale_add(const LaunchCtx& c) {
 // src/models/qwen3_5/moe.cpp:396-404).  "..._rows" (not a reference id) adds a trailing
 // scalar `rows`: x is rows x hidden, ids rows x top_k, phi rows x top_k x inter, one token
 // per row in a single launch.
+constexpr uint64_t kMoeGroupedMinRows = 48;
+
 qmm_status run_moe_gate_up_n(const LaunchCtx& c, bool batched) {
   if (!counts(c, 5, batched ? 6 : 5)) return bad("moe_experts_gate_up_q4k: expects 5 buffers and 5 (6) scalars");
   const uint64_t hidden = c.sc[0], inter = c.sc[1], top_k = c.sc[2], gs = c.sc[3], us = c.sc[4];
@@ -615,6 +617,18 @@ qmm_status run_moe_gate_up_n(const LaunchCtx& c, bool batched) {
     const uint64_t eg = (c.bytes[1] - static_cast<uint64_t>(expert)) / gs + 1, eu = (c.bytes[2] - static_cast<uint64_t>(expert)) / us + 1;
     experts = eg < eu ? eg : eu;
     if (experts > 0xFFFFFFFFull) experts = 0xFFFFFFFFull;
+  }
+  // A chunk of tokens (prefill): grouped by expert on the MFMA path, each expert's weights read
+  // once per launch; 48 tokens is about where that overtakes one exact pass per token.
+  if (batched && rows >= kMoeGroupedMinRows && c.bytes != nullptr && rows * top_k <= (1u << 20) &&
+      qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
+    void* ws = nullptr;
+    const qmm_status st = workspace(qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
+    if (st != QMM_OK) return st;
+    return map_hip(qmm::launch_moe_gate_up_q4k_grouped(
+        c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint8_t>(2), c.ptr<const uint32_t>(3), c.ptr<float>(4),
+        ws, static_cast<uint32_t>(hidden), static_cast<uint32_t>(inter), static_cast<uint32_t>(top_k), gs, us,
+        static_cast<uint32_t>(experts), static_cast<uint32_t>(rows), c.stream));
   }
   return map_hip(qmm::launch_moe_gate_up_q4k(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint8_t>(2),
                                              c.ptr<const uint32_t>(3), c.ptr<float>(4), static_cast<uint32_t>(hidden),
@@ -649,6 +663,16 @@ qmm_status run_moe_down_n(const LaunchCtx& c, bool batched, bool q6k) {
   }
   uint64_t experts = 0xFFFFFFFFull;
   if (c.bytes != nullptr) experts = (c.bytes[1] - static_cast<uint64_t>(expert_bytes)) / ds + 1;
+  if (!q6k && batched && rows >= kMoeGroupedMinRows && c.bytes != nullptr && rows * top_k <= (1u << 20) &&
+      qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
+    void* ws = nullptr;
+    const qmm_status st = workspace(qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
+    if (st != QMM_OK) return st;
+    return map_hip(qmm::launch_moe_down_q4k_grouped(
+        c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint32_t>(2), c.ptr<const float>(3), c.ptr<float>(4), ws,
+        static_cast<uint32_t>(hidden), static_cast<uint32_t>(inter), static_cast<uint32_t>(top_k), ds,
+        static_cast<uint32_t>(experts), static_cast<uint32_t>(rows), acc != 0, c.stream));
+  }
   const auto launch = q6k ? qmm::launch_moe_down_q6k : qmm::launch_moe_down_q4k;
   return map_hip(launch(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint32_t>(2),
                         c.ptr<const float>(3), c.ptr<float>(4), static_cast<uint32_t>(hidden),

@@ -82,6 +82,14 @@ hipError_t launch_kquant_f16_gemm(const float* a, const uint8_t* w, uint32_t blo
 // the token's top_k experts of wts * down_e(silu(gate_e x) * up_e x), as grouped MFMA GEMMs.
 bool moe_ffn_q4k_supported(uint64_t hidden, uint64_t inter, uint64_t experts);
 size_t moe_ffn_q4k_workspace_bytes(uint64_t pairs, uint64_t hidden, uint64_t inter, uint64_t experts);
+hipError_t launch_moe_gate_up_q4k_grouped(const float* x, const uint8_t* gate, const uint8_t* up, const uint32_t* ids,
+                                          float* phi, void* workspace, uint32_t hidden, uint32_t inter, uint32_t top_k,
+                                          uint64_t gate_stride, uint64_t up_stride, uint32_t experts, uint32_t tokens,
+                                          hipStream_t stream);
+hipError_t launch_moe_down_q4k_grouped(const float* phi, const uint8_t* down, const uint32_t* ids, const float* wts,
+                                       float* out, void* workspace, uint32_t hidden, uint32_t inter, uint32_t top_k,
+                                       uint64_t down_stride, uint32_t experts, uint32_t tokens, bool accumulate,
+                                       hipStream_t stream);
 hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                               const uint32_t* ids, const float* wts, float* out, void* workspace,
                               uint32_t hidden, uint32_t inter, uint32_t top_k, uint64_t gate_stride,

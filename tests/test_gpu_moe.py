@@ -106,6 +106,29 @@ def test_rows_match_oracle(backend, rows, experts, hidden, inter, top_k):
     assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
+@pytest.mark.parametrize("rows,experts,hidden,inter,top_k", [(47, 16, 512, 256, 4), (48, 16, 512, 256, 4),
+                                                             (130, 6, 256, 512, 3), (300, 9, 512, 256, 2)])
+def test_rows_ids_around_the_grouping_threshold(backend, rows, experts, hidden, inter, top_k):
+    """moe_experts_gate_up_q4k_rows + moe_experts_down_q4k_rows: 47 tokens run one exact pass per
+    token, 48 and more are grouped by expert on the fp16 MFMA path (bound as for
+    moe_experts_ffn_q4k_rows); accumulate adds to what the output held."""
+    g = synth.rng(rows * 5 + experts + hidden)
+    gate, up, down = expert_tensors(g, experts, hidden, inter)
+    x = synth.activations_bf16(g, rows, hidden)
+    ids, vals = synth.moe_routing(g, rows, experts, top_k)
+    ids[0, 0] = experts + 3              # out of range: clamped to the last expert in both regimes
+    wts = np.stack([oracle.moe_gate(v) for v in vals])
+    clamped = np.minimum(ids, experts - 1)
+    ref = oracle.moe_batch_forward_q4k(x, clamped, wts, gate, up, down, hidden, inter)
+    got = forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
+    if rows < 48:
+        assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    else:
+        assert rms_err(got, ref) <= 8e-3 and norm_err(got, ref) <= 2e-3, (rms_err(got, ref), norm_err(got, ref))
+    again = forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
+    assert np.array_equal(again, got)
+
+
 def test_config4_shapes(backend):
     """BASELINE configs[4]: 256 experts, hidden 2048, expert FFN 512, softmax top-8; M = 1
     (decode) and M = 512 (prefill chunk) in one launch each.  The M = 512 result is checked on
@@ -129,17 +152,23 @@ def test_config4_shapes(backend):
     x = synth.activations_bf16(g, rows, hidden)
     ids, vals = synth.moe_routing(g, rows, experts, top_k)
     wts = np.stack([oracle.moe_gate(v) for v in vals])
-    got = forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
     sample = [0, 1, 100, 255, 256, 511]
     ref = oracle.moe_batch_forward_q4k(x[sample], ids[sample], wts[sample], gate, up, down, hidden, inter)
-    assert rel_err(got[sample], ref) <= TOL, rel_err(got[sample], ref)
+    # Below 48 tokens the two row-batched ids take one exact fp32 pass per token.
+    few = forward_rows(backend, x[:40], ids[:40], wts[:40], gate, up, down, hidden, inter, experts)
+    assert rel_err(few[:2], ref[:2]) <= TOL, rel_err(few[:2], ref[:2])
     alone = forward_rows(backend, x[:1], ids[:1], wts[:1], gate, up, down, hidden, inter, experts)
-    assert np.array_equal(alone[0], got[0])
+    assert np.array_equal(alone[0], few[0])
+    # The whole chunk: the same two ids now group the tokens by expert (fp16 MFMA), as the
+    # one-call form does; both within the grouped path's bound of the oracle, and of each other
+    # to rounding (they share every kernel but the one that applies silu).
+    got = forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
     assert np.all(np.isfinite(got))
-    # the grouped form (tokens sorted by expert, fp16 MFMA) on the same chunk
+    assert rms_err(got[sample], ref) <= 8e-3, rms_err(got[sample], ref)
+    assert rms_err(got[:40], few) <= 8e-3 and norm_err(got[:40], few) <= 2e-3
     grouped = forward_grouped(backend, x, ids, wts, gate, up, down, hidden, inter, experts)
     assert rms_err(grouped[sample], ref) <= 8e-3, rms_err(grouped[sample], ref)
-    assert rms_err(grouped, got) <= 8e-3 and norm_err(grouped, got) <= 2e-3
+    assert rms_err(grouped, got) <= 1e-5, rms_err(grouped, got)
 
 
 def forward_grouped(backend, x, ids, wts, gate, up, down, hidden, inter, experts, accumulate=0, out0=None):

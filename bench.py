@@ -302,9 +302,9 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     gs, ds = inter * (hidden // 256) * 144, hidden * (inter // 256) * 144
     kgu, kdn = backend.LoadKernel("moe_experts_gate_up_q4k_rows"), backend.LoadKernel("moe_experts_down_q4k_rows")
     moe = {}
-    # m1 and m32: one exact pass per token; m512: the same two ids group the tokens by expert (from
-    # 48 tokens), m512_grouped: the one-call form of that.
-    for rows in (1, 32, 512):
+    # m1 and m16: one exact pass per token; m512: the same two ids group the tokens by expert (from
+    # 17 tokens), m512_grouped: the one-call form of that.
+    for rows in (1, 16, 512):
         x = to_dev(synth.activations_bf16(g, rows, hidden))
         ids, vals = synth.moe_routing(g, rows, experts, top_k)
         e = np.exp(vals - vals.max(axis=1, keepdims=True))
@@ -321,7 +321,7 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
         us = timed_us(launches, 20 if rows == 1 else 5, graph=rows == 1)
         touched = (min(rows * top_k, experts) if rows > 1 else top_k) * 3 * gs
         moe[f"m{rows}"] = {"us": round(us, 2), "weight_GBps": round(touched / us / 1e3, 1)}
-        if rows > 32:
+        if rows > 16:
             # the same chunk with the tokens grouped by expert (one weight pass per expert, MFMA)
             kff = backend.LoadKernel("moe_experts_ffn_q4k_rows")
             grouped = [(kff, KernelLaunch(grid_x=1, buffers=[wrap(x), wrap(gate), wrap(up), wrap(down), wrap(ids),

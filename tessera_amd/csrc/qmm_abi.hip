@@ -595,7 +595,7 @@ qmm_status run_moe_scale_add(const LaunchCtx& c) {
 // src/models/qwen3_5/moe.cpp:396-404).  "..._rows" (not a reference id) adds a trailing
 // scalar `rows`: x is rows x hidden, ids rows x top_k, phi rows x top_k x inter, one token
 // per row in a single launch.
-constexpr uint64_t kMoeGroupedMinRows = 48;
+constexpr uint64_t kMoeGroupedMinRows = 17;   // as kQ4KGemmMinRows: past the largest speculative-verify batch
 
 qmm_status run_moe_gate_up_n(const LaunchCtx& c, bool batched) {
   if (!counts(c, 5, batched ? 6 : 5)) return bad("moe_experts_gate_up_q4k: expects 5 buffers and 5 (6) scalars");
@@ -619,7 +619,8 @@ qmm_status run_moe_gate_up_n(const LaunchCtx& c, bool batched) {
     if (experts > 0xFFFFFFFFull) experts = 0xFFFFFFFFull;
   }
   // A chunk of tokens (prefill): grouped by expert on the MFMA path, each expert's weights read
-  // once per launch; 48 tokens is about where that overtakes one exact pass per token.
+  // once per launch; that overtakes one exact pass per token at about 16 tokens (256 experts,
+  // top-8: 89 against 81 us).
   if (batched && rows >= kMoeGroupedMinRows && c.bytes != nullptr && rows * top_k <= (1u << 20) &&
       qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
     void* ws = nullptr;

@@ -117,6 +117,24 @@ qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t 
                       void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
                       const uint64_t* scalars, size_t nscalars, void* stream);
 
+/* qmm_launch for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its
+ * scratch lives in the caller's arch state).  Same arguments, validation and results as
+ * qmm_launch, but every kernel that needs scratch beyond its inputs and outputs (the Q4_K
+ * few-row operand, the fp16 copies of the MFMA GEMMs, the fused feed-forward's up product, the
+ * grouped routed-expert tables) takes it from one device array of QMM_STATIC_SCRATCH_BYTES that
+ * is part of the library's code object: it calls no hipMalloc or hipFree, and a launch that
+ * needs more returns InvalidArgument with the two sizes in qmm_last_error.  Each device the
+ * library is loaded on holds that array until the process ends.  All calls on a device share
+ * it and it keeps the last call's contents (no kernel here needs it zeroed): launches through
+ * this entry point on one device must be ordered (one stream, or events); overlapping ones
+ * race on the scratch. */
+#define QMM_STATIC_SCRATCH_BYTES (32u << 20)
+qmm_status qmm_launch_static(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                             void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
+                             const uint64_t* scalars, size_t nscalars, void* stream);
+size_t qmm_static_scratch_bytes(void);
+
 /* Backend::Synchronize (backend.hpp:1028-1029; rocm_backend.cpp:731-739). */
 qmm_status qmm_sync(void* stream);
 

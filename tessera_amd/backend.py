@@ -70,6 +70,9 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
         "qmm_kernel_name": (C.c_char_p, [sz]),
         "qmm_launch": (C.c_int32, [C.c_size_t, u32p, u32p, C.POINTER(vp), C.POINTER(sz), sz, u64p,
                                    sz, vp]),
+        "qmm_launch_static": (C.c_int32, [C.c_size_t, u32p, u32p, C.POINTER(vp), C.POINTER(sz), sz, u64p,
+                                          sz, vp]),
+        "qmm_static_scratch_bytes": (sz, []),
         "qmm_sync": (C.c_int32, [vp]),
         "qmm_last_error": (C.c_char_p, []),
     }
@@ -233,15 +236,22 @@ class Backend:
     def KernelNames(self) -> list[str]:
         return [self._lib.qmm_kernel_name(i).decode() for i in range(self._lib.qmm_kernel_count())]
 
-    def LaunchKernel(self, kernel: Kernel, launch: KernelLaunch) -> None:
+    def LaunchKernel(self, kernel: Kernel, launch: KernelLaunch, no_alloc: bool = False) -> None:
+        """``no_alloc=True`` goes through ``qmm_launch_static`` (not in the reference): the same
+        launch with every kernel's scratch taken from the library's static device array, for
+        callers that may not allocate device memory."""
         nb, ns = len(launch.buffers), len(launch.scalars)
         grid = (C.c_uint32 * 3)(launch.grid_x, launch.grid_y, launch.grid_z)
         block = (C.c_uint32 * 3)(launch.block_x, launch.block_y, launch.block_z)
         bufs = (C.c_void_p * max(nb, 1))(*[b.Handle() for b in launch.buffers])
         sizes = (C.c_size_t * max(nb, 1))(*[b.Size() for b in launch.buffers])
         scal = (C.c_uint64 * max(ns, 1))(*[int(s) & 0xFFFFFFFFFFFFFFFF for s in launch.scalars])
-        self._check(self._lib.qmm_launch(kernel.Handle(), grid, block, bufs, sizes, nb, scal, ns,
-                                         self._stream), f"LaunchKernel({kernel.Id()})")
+        entry = self._lib.qmm_launch_static if no_alloc else self._lib.qmm_launch
+        self._check(entry(kernel.Handle(), grid, block, bufs, sizes, nb, scal, ns, self._stream),
+                    f"LaunchKernel({kernel.Id()})")
+
+    def StaticScratchBytes(self) -> int:
+        return int(self._lib.qmm_static_scratch_bytes())
 
     def Synchronize(self) -> None:
         self._check(self._lib.qmm_sync(self._stream), "Synchronize")

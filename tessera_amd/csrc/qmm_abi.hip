@@ -22,6 +22,7 @@ struct LaunchCtx {
   const uint64_t* sc;
   size_t nsc;
   hipStream_t stream;
+  bool no_alloc = false;  // qmm_launch_static: scratch comes from the static device array only
 
   template <class T>
   T* ptr(size_t i) const { return static_cast<T*>(buf[i]); }
@@ -83,7 +84,26 @@ constexpr size_t kDecodeScratchBytes = size_t{16} << 20;
 void* g_decode_scratch = nullptr;
 std::mutex g_workspace_mutex;
 
-qmm_status workspace(size_t bytes, void** out) {
+// Scratch of qmm_launch_static, the entry point that allocates nothing: a device array that is
+// part of the code object, so it exists on every device the library is loaded on from load time
+// to process end.  In host code the array's name is only a handle for hipGetSymbolAddress;
+// g_static_scratch[device] holds the device address (resolved by qmm_init with that device
+// current) and is what every launch uses.
+constexpr size_t kStaticScratchBytes = QMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};
+
+qmm_status workspace(const LaunchCtx& c, size_t bytes, void** out) {
+  if (c.no_alloc) {
+    if (bytes > kStaticScratchBytes) {
+      g_last_error = "qmm_launch_static: this launch needs " + std::to_string(bytes) +
+                     " bytes of scratch, the static scratch holds " + std::to_string(kStaticScratchBytes);
+      return QMM_INVALID_ARGUMENT;
+    }
+    *out = g_static_scratch[g_device];
+    return QMM_OK;
+  }
   std::lock_guard<std::mutex> lock(g_workspace_mutex);
   if (bytes > g_workspace_bytes) {
     if (g_workspace != nullptr) (void)hipFree(g_workspace);
@@ -101,6 +121,13 @@ qmm_status workspace(size_t bytes, void** out) {
   return QMM_OK;
 }
 
+// The fixed-address scratch of the decode-sized kernels: qmm_init's allocation, or the first
+// kDecodeScratchBytes of the static array for qmm_launch_static.
+void* decode_scratch(const LaunchCtx& c) {
+  static_assert(kDecodeScratchBytes <= kStaticScratchBytes, "the static scratch holds the decode scratch");
+  return c.no_alloc ? g_static_scratch[g_device] : g_decode_scratch;
+}
+
 // From this many rows on, Q4_K goes to the tiled fp16 MFMA GEMM: one more than the largest
 // speculative-verify batch (16), which stays on the exact fp32-accumulate paths as in the
 // reference (its fp16 tensor-core tile starts at 64 rows).  Below it, 2 and more rows of
@@ -111,11 +138,12 @@ constexpr uint64_t kQ4KGemmMinRows = 17;
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 
-qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
-                      uint64_t k, hipStream_t s) {
+qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
+                      uint64_t k) {
+  const hipStream_t s = ctx.stream;
   if (m >= 2 && m < kQ4KGemmMinRows && n * k >= kQ4KFewRowsMinWeights && k <= kQ4KFewRowsMaxK &&
       qmm::gemv_q4k_mfma_supported(1, n, k)) {
-    void* ws = g_decode_scratch;   // fixed address: a recorded decode step stays valid
+    void* ws = decode_scratch(ctx);   // fixed address: a recorded decode step stays valid
     if (ws == nullptr || qmm::gemv_q4k_mfma_workspace_bytes(8, k) > kDecodeScratchBytes) {
       g_last_error = "Q4_K: decode scratch missing or too small for this k";
       return QMM_DEVICE_ERROR;
@@ -130,7 +158,7 @@ qmm_status q4k_matmul(const float* a, const uint8_t* w, float* c, uint64_t m, ui
   }
   if (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) {
     void* ws = nullptr;
-    const qmm_status st = workspace(qmm::gemm_q4k_workspace_bytes(m, k), &ws);
+    const qmm_status st = workspace(ctx, qmm::gemm_q4k_workspace_bytes(m, k), &ws);
     if (st != QMM_OK) return st;
     return map_hip(qmm::launch_q4k_gemm(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                         static_cast<uint32_t>(k), s));
@@ -150,7 +178,7 @@ qmm_status run_gemm_q4k(const LaunchCtx& c) {
       !c.fits(2, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_q4k: a buffer is smaller than m, n, k require");
   }
-  return q4k_matmul(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k, c.stream);
+  return q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k);
 }
 
 // "gemm_q4k_vec" and "gemm_q4k_rows{R}": buffers A, W, C; scalars m, n, k, split
@@ -168,7 +196,7 @@ qmm_status run_gemm_q4k_split(const LaunchCtx& c, uint64_t rows_required) {
     return bad("gemm_q4k_vec/rows: a buffer is smaller than m, n, k, split require");
   }
   float* out = c.ptr<float>(2);
-  qmm_status st = q4k_matmul(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, m, n, k, c.stream);
+  qmm_status st = q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, m, n, k);
   if (st == QMM_OK && split > 1) {
     st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
   }
@@ -298,8 +326,8 @@ qmm_status run_ffn_gate_up_silu_q4k(const LaunchCtx& c) {
     // few-row kernels may use for their activation operand, so nothing is allocated (a recorded
     // decode step stays valid).
     const size_t up_off = (qmm::gemv_q4k_mfma_workspace_bytes(8, k) + 255) & ~size_t{255};
-    if (g_decode_scratch != nullptr && up_off + up_bytes <= kDecodeScratchBytes) {
-      u = reinterpret_cast<float*>(static_cast<uint8_t*>(g_decode_scratch) + up_off);
+    if (decode_scratch(c) != nullptr && up_off + up_bytes <= kDecodeScratchBytes) {
+      u = reinterpret_cast<float*>(static_cast<uint8_t*>(decode_scratch(c)) + up_off);
     }
   }
   if (u == nullptr) {
@@ -308,12 +336,12 @@ qmm_status run_ffn_gate_up_silu_q4k(const LaunchCtx& c) {
     const size_t gemm_ws = (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
     const size_t up_off = (gemm_ws + 255) & ~size_t{255};
     void* ws = nullptr;
-    st = workspace(up_off + up_bytes, &ws);
+    st = workspace(c, up_off + up_bytes, &ws);
     if (st != QMM_OK) return st;
     u = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + up_off);
   }
-  st = q4k_matmul(x, gate, out, m, n, k, c.stream);
-  if (st == QMM_OK) st = q4k_matmul(x, up, u, m, n, k, c.stream);
+  st = q4k_matmul(c, x, gate, out, m, n, k);
+  if (st == QMM_OK) st = q4k_matmul(c, x, up, u, m, n, k);
   if (st == QMM_OK) st = map_hip(qmm::launch_silu_mul(out, u, out, m * n, c.stream));
   return st;
 }
@@ -334,7 +362,7 @@ qmm_status run_dequant_q4k(const LaunchCtx& c) {
 qmm_status kquant_prefill(const LaunchCtx& c, uint32_t block_bytes, uint64_t m, uint64_t n, uint64_t k,
                           uint64_t split) {
   void* ws = nullptr;
-  qmm_status st = workspace(qmm::gemm_kquant_f16_workspace_bytes(m, n, k), &ws);
+  qmm_status st = workspace(c, qmm::gemm_kquant_f16_workspace_bytes(m, n, k), &ws);
   if (st != QMM_OK) return st;
   float* out = c.ptr<float>(2);
   st = map_hip(qmm::launch_kquant_f16_gemm(c.ptr<const float>(0), c.ptr<const uint8_t>(1), block_bytes, out, ws,
@@ -624,7 +652,7 @@ qmm_status run_moe_gate_up_n(const LaunchCtx& c, bool batched) {
   if (batched && rows >= kMoeGroupedMinRows && c.bytes != nullptr && rows * top_k <= (1u << 20) &&
       qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
     void* ws = nullptr;
-    const qmm_status st = workspace(qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
+    const qmm_status st = workspace(c, qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
     if (st != QMM_OK) return st;
     return map_hip(qmm::launch_moe_gate_up_q4k_grouped(
         c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint8_t>(2), c.ptr<const uint32_t>(3), c.ptr<float>(4),
@@ -667,7 +695,7 @@ qmm_status run_moe_down_n(const LaunchCtx& c, bool batched, bool q6k) {
   if (!q6k && batched && rows >= kMoeGroupedMinRows && c.bytes != nullptr && rows * top_k <= (1u << 20) &&
       qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
     void* ws = nullptr;
-    const qmm_status st = workspace(qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
+    const qmm_status st = workspace(c, qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
     if (st != QMM_OK) return st;
     return map_hip(qmm::launch_moe_down_q4k_grouped(
         c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint32_t>(2), c.ptr<const float>(3), c.ptr<float>(4), ws,
@@ -751,7 +779,7 @@ qmm_status run_moe_ffn_rows(const LaunchCtx& c) {
     return QMM_UNSUPPORTED_FEATURE;
   }
   void* ws = nullptr;
-  const qmm_status st = workspace(qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
+  const qmm_status st = workspace(c, qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
   if (st != QMM_OK) return st;
   return map_hip(qmm::launch_moe_ffn_q4k(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const uint8_t>(2),
                                          c.ptr<const uint8_t>(3), c.ptr<const uint32_t>(4), c.ptr<const float>(5),
@@ -850,6 +878,15 @@ qmm_status qmm_init(int device) {
   g_device_name = prop.name[0] != '\0' ? prop.name : prop.gcnArchName;   // some hosts report no marketing name
   qmm::set_num_cus(prop.multiProcessorCount);
   g_device = device;
+  if (device < kMaxDevices && g_static_scratch[device] == nullptr) {
+    // Each device holds its own copy of the array at its own address; `device` is current here.
+    void* p = nullptr;
+    if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) != hipSuccess) {
+      g_device = -1;
+      return map_hip(e);
+    }
+    g_static_scratch[device] = p;
+  }
   if (g_decode_scratch == nullptr) {
     if ((e = hipMalloc(&g_decode_scratch, kDecodeScratchBytes)) != hipSuccess) {
       g_decode_scratch = nullptr;
@@ -935,9 +972,11 @@ size_t qmm_kernel_count(void) { return kTableSize; }
 
 const char* qmm_kernel_name(size_t index) { return index < kTableSize ? kTable[index].id : nullptr; }
 
-qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
-                      void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
-                      const uint64_t* scalars, size_t nscalars, void* stream) {
+namespace {
+
+qmm_status launch_checked(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                          void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
+                          const uint64_t* scalars, size_t nscalars, void* stream, bool no_alloc) {
   if (kernel == 0 || kernel > kTableSize) return bad("qmm_launch: bad kernel handle");
   if (grid == nullptr || block == nullptr) return bad("qmm_launch: null grid or block");
   for (int i = 0; i < 3; ++i) {
@@ -955,14 +994,34 @@ qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t 
     g_last_error = "qmm_launch: qmm_init has not succeeded";
     return QMM_DEVICE_ERROR;
   }
+  if (no_alloc && (g_device >= kMaxDevices || g_static_scratch[g_device] == nullptr)) {
+    g_last_error = "qmm_launch_static: the static scratch was not resolved on this device";
+    return QMM_DEVICE_ERROR;
+  }
   if (t_device != g_device) {  // callers may hop threads; HIP's current device is per thread
     const hipError_t e = hipSetDevice(g_device);
     if (e != hipSuccess) return map_hip(e);
     t_device = g_device;
   }
-  const LaunchCtx ctx{buffers, buf_bytes, nbuffers, scalars, nscalars, static_cast<hipStream_t>(stream)};
+  const LaunchCtx ctx{buffers, buf_bytes, nbuffers, scalars, nscalars, static_cast<hipStream_t>(stream), no_alloc};
   return kTable[kernel - 1].fn(ctx);
 }
+
+}  // namespace
+
+qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                      void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
+                      const uint64_t* scalars, size_t nscalars, void* stream) {
+  return launch_checked(kernel, grid, block, buffers, buf_bytes, nbuffers, scalars, nscalars, stream, false);
+}
+
+qmm_status qmm_launch_static(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                             void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
+                             const uint64_t* scalars, size_t nscalars, void* stream) {
+  return launch_checked(kernel, grid, block, buffers, buf_bytes, nbuffers, scalars, nscalars, stream, true);
+}
+
+size_t qmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 qmm_status qmm_sync(void* stream) { return map_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
 

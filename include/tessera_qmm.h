@@ -15,8 +15,13 @@
  *     (src/backends/rocm/rocm_backend.cpp:311-330,716-722);
  *   - every function returns a qmm_status whose integer values are identical to
  *     tessera::StatusCode (include/tessera/types.hpp:36-48);
- *   - no exceptions cross the boundary and nothing here allocates device memory
- *     except qmm_alloc.
+ *   - no exceptions cross the boundary;
+ *   - device memory: qmm_alloc allocates what the caller asks for; qmm_init allocates the 16 MB
+ *     scratch of the decode-sized kernels once; prefill-sized launches (Q4_K/Q5_K/Q6_K from 17
+ *     rows, the grouped routed-expert ids) need a workspace, which is the caller's when one was
+ *     set with qmm_set_workspace and otherwise a library-owned block that qmm_launch grows on
+ *     demand (hipFree + hipMalloc, which synchronises the device and must not happen under stream
+ *     capture).  qmm_launch_static never allocates.
  */
 #ifndef TESSERA_QMM_H_
 #define TESSERA_QMM_H_
@@ -103,7 +108,9 @@ const char* qmm_kernel_name(size_t index);
  * CheckBuiltInArgs (backend.hpp:391-841), a NULL buffer, a buffer pointer that is not
  * 16-byte aligned (device allocations are; the kernels use 16-byte vector loads), and --
  * when `buf_bytes` is not NULL -- any buffer smaller than the launch's scalars require.  `buf_bytes[i]` is
- * Buffer::Size() of buffer i; pass NULL to skip the size check.
+ * Buffer::Size() of buffer i; pass NULL to skip the size check (the routed-expert ids that clamp
+ * expert ids to their tensor -- "moe_experts_down_*", "moe_experts_ffn_q4k_rows" -- need the sizes
+ * and return InvalidArgument without them).
  *
  * Geometry: the ids keep the reference's argument contracts, but a gfx950 kernel has
  * its own natural launch shape, so `grid` and `block` are validated and otherwise
@@ -134,6 +141,18 @@ qmm_status qmm_launch_static(qmm_kernel kernel, const uint32_t grid[3], const ui
                              void* const* buffers, const size_t* buf_bytes, size_t nbuffers,
                              const uint64_t* scalars, size_t nscalars, void* stream);
 size_t qmm_static_scratch_bytes(void);
+
+/* Caller-owned scratch, as the reference keeps it in the arch state and grows it on demand
+ * (src/models/qwen3_5/project.cpp:127-155,198-206: gemv_part, wmma_a, wmma_as, wmma_part).
+ * qmm_workspace_bytes returns what a launch of `kernel` with these scalars needs (0 for
+ * decode-sized launches and ids without scratch; for the grouped routed-expert ids an upper bound
+ * over the expert count).  qmm_set_workspace hands the library a device block of that size
+ * (256-byte aligned) to use for every later qmm_launch on any stream, in stream order, until it
+ * is replaced or cleared with (NULL, 0); while one is set, qmm_launch allocates nothing and a
+ * launch that needs more returns InvalidArgument.  The caller must not free or replace the
+ * block while launches that use it are in flight. */
+qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_t nscalars, size_t* out_bytes);
+qmm_status qmm_set_workspace(void* device_ptr, size_t bytes);
 
 /* Backend::Synchronize (backend.hpp:1028-1029; rocm_backend.cpp:731-739). */
 qmm_status qmm_sync(void* stream);

@@ -73,6 +73,8 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
         "qmm_launch_static": (C.c_int32, [C.c_size_t, u32p, u32p, C.POINTER(vp), C.POINTER(sz), sz, u64p,
                                           sz, vp]),
         "qmm_static_scratch_bytes": (sz, []),
+        "qmm_workspace_bytes": (C.c_int32, [C.c_size_t, u64p, sz, C.POINTER(sz)]),
+        "qmm_set_workspace": (C.c_int32, [vp, sz]),
         "qmm_sync": (C.c_int32, [vp]),
         "qmm_last_error": (C.c_char_p, []),
     }
@@ -249,6 +251,22 @@ class Backend:
         entry = self._lib.qmm_launch_static if no_alloc else self._lib.qmm_launch
         self._check(entry(kernel.Handle(), grid, block, bufs, sizes, nb, scal, ns, self._stream),
                     f"LaunchKernel({kernel.Id()})")
+
+    def WorkspaceBytes(self, kernel: Kernel, scalars: Sequence[int]) -> int:
+        """Scratch a launch of ``kernel`` with these scalars needs (``qmm_workspace_bytes``)."""
+        ns = len(scalars)
+        scal = (C.c_uint64 * max(ns, 1))(*[int(s) & 0xFFFFFFFFFFFFFFFF for s in scalars])
+        out = C.c_size_t()
+        self._check(self._lib.qmm_workspace_bytes(kernel.Handle(), scal, ns, C.byref(out)), "WorkspaceBytes")
+        return int(out.value)
+
+    def SetWorkspace(self, buffer: "Buffer | None") -> None:
+        """Hand the library a caller-owned workspace (``qmm_set_workspace``); ``None`` clears it.
+        Mirrors the scratch the reference's arch state owns (project.cpp:127-155)."""
+        if buffer is None:
+            self._check(self._lib.qmm_set_workspace(None, 0), "SetWorkspace")
+        else:
+            self._check(self._lib.qmm_set_workspace(C.c_void_p(buffer.Handle()), buffer.Size()), "SetWorkspace")
 
     def StaticScratchBytes(self) -> int:
         return int(self._lib.qmm_static_scratch_bytes())

@@ -350,30 +350,33 @@ __global__ __launch_bounds__(256) void moe_scale_add_kernel(const float* __restr
 }
 
 // "moe_gate" (src/backends/rocm/rocm_kernels_basic.cpp:1896-1929): softmax over the top_k
-// selected router logits, and the shared expert's sigmoid gate sig = sigmoid(x . w).
-// One workgroup; same summation tree as the reference (strided partials, then halving).
+// selected router logits (wts), and the shared expert's sigmoid gate sig = sigmoid(x . w).
+// One workgroup of four wavefronts: the dot product is summed per wavefront with cross-lane
+// adds and the four partials in order; the softmax (top_k is a handful of values) runs in the
+// first wavefront, one value per lane, with wavefront-wide max and sum.  Sums are taken in
+// another order than the reference's halving tree, so sig agrees to fp32 rounding, not bitwise.
 __global__ __launch_bounds__(256) void moe_gate_kernel(const float* __restrict__ vals,
                                                        const float* __restrict__ x,
                                                        const float* __restrict__ w,
                                                        float* __restrict__ wts, float* __restrict__ sig,
                                                        uint32_t top_k, uint32_t hidden) {
-  __shared__ float red[256];
-  const uint32_t tid = threadIdx.x;
+  __shared__ float part[4];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
   float dot = 0.0f;
-  for (uint32_t t = tid; t < hidden; t += 256u) dot += x[t] * w[t];
-  red[tid] = dot;
+  for (uint32_t t = tid; t < hidden; t += 256u) dot = fmaf(x[t], w[t], dot);
+  dot = wave_sum(dot);
+  if (lane == 0u) part[tid >> 6] = dot;
   __syncthreads();
-  for (uint32_t s = 128u; s > 0u; s >>= 1) {
-    if (tid < s) red[tid] += red[tid + s];
-    __syncthreads();
-  }
-  if (tid == 0u) {
+  if (tid < 64u) {
+    // softmax over the selected logits, 64 at a time
     float m = -3.402823466e+38f;
-    for (uint32_t p = 0; p < top_k; ++p) m = fmaxf(m, vals[p]);
+    for (uint32_t p = lane; p < top_k; p += 64u) m = fmaxf(m, vals[p]);
+    m = wave_max(m);
     float sum = 0.0f;
-    for (uint32_t p = 0; p < top_k; ++p) sum += expf(vals[p] - m);
-    for (uint32_t p = 0; p < top_k; ++p) wts[p] = expf(vals[p] - m) / sum;
-    sig[0] = 1.0f / (1.0f + expf(-red[0]));
+    for (uint32_t p = lane; p < top_k; p += 64u) sum += expf(vals[p] - m);
+    sum = wave_sum(sum);
+    for (uint32_t p = lane; p < top_k; p += 64u) wts[p] = expf(vals[p] - m) / sum;
+    if (lane == 0u) sig[0] = 1.0f / (1.0f + expf(-(((part[0] + part[1]) + part[2]) + part[3])));
   }
 }
 

@@ -77,6 +77,10 @@ u128 mxfp4_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * k / 2 +
 // Launches that use it are ordered by the caller's stream, as everything else here.
 void* g_workspace = nullptr;
 size_t g_workspace_bytes = 0;
+// A workspace the caller owns (qmm_set_workspace): while one is set the library neither grows nor
+// frees anything in qmm_launch; a launch that needs more than it holds is refused.
+void* g_user_workspace = nullptr;
+size_t g_user_workspace_bytes = 0;
 // Scratch of the decode-sized kernels (the few-row Q4_K path's activation operand): allocated
 // once by qmm_init and never moved or freed, so a decode step recorded into a HIP graph keeps
 // pointing at live memory whatever the prefill-sized workspace above does later.
@@ -105,6 +109,15 @@ qmm_status workspace(const LaunchCtx& c, size_t bytes, void** out) {
     return QMM_OK;
   }
   std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  if (g_user_workspace != nullptr) {
+    if (bytes > g_user_workspace_bytes) {
+      g_last_error = "qmm_launch: this launch needs " + std::to_string(bytes) + " bytes of workspace, the one set with "
+                     "qmm_set_workspace holds " + std::to_string(g_user_workspace_bytes);
+      return QMM_INVALID_ARGUMENT;
+    }
+    *out = g_user_workspace;
+    return QMM_OK;
+  }
   if (bytes > g_workspace_bytes) {
     if (g_workspace != nullptr) (void)hipFree(g_workspace);
     g_workspace = nullptr;
@@ -686,13 +699,15 @@ qmm_status run_moe_down_n(const LaunchCtx& c, bool batched, bool q6k) {
       !c.fits(4, static_cast<u128>(rows) * hidden * 4)) {
     return bad(std::string(who) + ": a buffer is smaller than the shape requires");
   }
-  if (c.bytes != nullptr && c.bytes[1] >= (1ull << 32)) {
+  // The expert ids are clamped to the tensor and the kernels address it with 32-bit offsets, so
+  // the tensor's size must be known and below 4 GB.
+  if (c.bytes == nullptr) return bad(std::string(who) + ": buffer sizes are required (they bound the expert ids)");
+  if (c.bytes[1] >= (1ull << 32)) {
     g_last_error = std::string(who) + ": expert tensors of 4 GB and more are not implemented";
     return QMM_UNSUPPORTED_FEATURE;
   }
-  uint64_t experts = 0xFFFFFFFFull;
-  if (c.bytes != nullptr) experts = (c.bytes[1] - static_cast<uint64_t>(expert_bytes)) / ds + 1;
-  if (!q6k && batched && rows >= kMoeGroupedMinRows && c.bytes != nullptr && rows * top_k <= (1u << 20) &&
+  const uint64_t experts = (c.bytes[1] - static_cast<uint64_t>(expert_bytes)) / ds + 1;
+  if (!q6k && batched && rows >= kMoeGroupedMinRows && rows * top_k <= (1u << 20) &&
       qmm::moe_ffn_q4k_supported(hidden, inter, experts)) {
     void* ws = nullptr;
     const qmm_status st = workspace(c, qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, experts), &ws);
@@ -1022,6 +1037,45 @@ qmm_status qmm_launch_static(qmm_kernel kernel, const uint32_t grid[3], const ui
 }
 
 size_t qmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_t nscalars, size_t* out_bytes) {
+  if (kernel == 0 || kernel > kTableSize || out_bytes == nullptr || (nscalars != 0 && scalars == nullptr)) {
+    return bad("qmm_workspace_bytes: bad kernel handle or null argument");
+  }
+  *out_bytes = 0;
+  const std::string id = kTable[kernel - 1].id;
+  auto sc = [&](size_t i) { return i < nscalars ? scalars[i] : uint64_t{0}; };
+  auto starts = [&](const char* prefix) { return id.rfind(prefix, 0) == 0; };
+  if (starts("gemm_q4k")) {
+    const uint64_t m = sc(0), k = sc(2);
+    if (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) *out_bytes = qmm::gemm_q4k_workspace_bytes(m, k);
+  } else if (id == "ffn_gate_up_silu_q4k") {
+    const uint64_t m = sc(0), n = sc(1), k = sc(2);
+    if (m >= kQ4KGemmMinRows) {
+      const size_t gemm_ws = qmm::gemm_q4k_supported(m, k) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
+      *out_bytes = ((gemm_ws + 255) & ~size_t{255}) + static_cast<size_t>(m) * n * 4;
+    }
+  } else if (starts("gemm_q5k") || starts("gemm_q6k")) {
+    const uint64_t m = sc(0), n = sc(1), k = sc(2);
+    if (m >= kQ4KGemmMinRows && qmm::gemm_kquant_f16_supported(m, n, k)) *out_bytes = qmm::gemm_kquant_f16_workspace_bytes(m, n, k);
+  } else if (id == "moe_experts_gate_up_q4k_rows" || id == "moe_experts_down_q4k_rows") {
+    const uint64_t hidden = sc(0), inter = sc(1), top_k = sc(2), rows = sc(5);
+    if (rows >= kMoeGroupedMinRows) *out_bytes = qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, 1024);
+  } else if (id == "moe_experts_ffn_q4k_rows") {
+    const uint64_t hidden = sc(0), inter = sc(1), top_k = sc(2), rows = sc(6);
+    *out_bytes = qmm::moe_ffn_q4k_workspace_bytes(rows * top_k, hidden, inter, 1024);
+  }
+  return QMM_OK;
+}
+
+qmm_status qmm_set_workspace(void* device_ptr, size_t bytes) {
+  if ((device_ptr == nullptr) != (bytes == 0)) return bad("qmm_set_workspace: pointer and size must both be set or both be zero");
+  if (reinterpret_cast<uintptr_t>(device_ptr) % 256 != 0) return bad("qmm_set_workspace: the workspace must be 256-byte aligned");
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  g_user_workspace = device_ptr;
+  g_user_workspace_bytes = bytes;
+  return QMM_OK;
+}
 
 qmm_status qmm_sync(void* stream) { return map_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
 

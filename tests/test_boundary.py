@@ -129,3 +129,31 @@ def test_per_id_validation_on_device(backend):
     with pytest.raises(StatusError) as e:
         backend.CopyD2HAt(c, 8, 4 * n)
     assert e.value.code == StatusCode.InvalidArgument
+
+
+@pytest.mark.gpu
+def test_routed_expert_down_ids_need_buffer_sizes(backend):
+    """The expert ids are clamped to the tensor, whose size only the buffer sizes tell: without
+    them (buf_bytes = NULL, which other ids accept) the call is refused before any device work."""
+    import ctypes as C
+    g = synth.rng(2)
+    experts, hidden, inter, top_k = 4, 256, 256, 2
+    down = backend.Upload(synth.q4k_weights(g, experts * hidden, inter))
+    phi = backend.Upload(np.zeros(top_k * inter, np.float32))
+    ids = backend.Upload(np.array([1, 3], np.uint32))
+    wts = backend.Upload(np.array([0.5, 0.5], np.float32))
+    out = backend.AllocateBuffer(4 * hidden)
+    backend.CopyH2D(out, np.full(hidden, 7.0, np.float32))
+    ds = hidden * (inter // 256) * 144
+    lib = backend._lib
+    grid, block = (C.c_uint32 * 3)(1, 1, 1), (C.c_uint32 * 3)(256, 1, 1)
+    bufs = (C.c_void_p * 5)(phi.Handle(), down.Handle(), ids.Handle(), wts.Handle(), out.Handle())
+    for name, scalars in (("moe_experts_down_q4k", [hidden, inter, top_k, ds, 0]),
+                          ("moe_experts_down_q4k_rows", [hidden, inter, top_k, ds, 0, 1])):
+        scal = (C.c_uint64 * len(scalars))(*scalars)
+        kern = backend.LoadKernel(name)
+        rc = lib.qmm_launch(kern.Handle(), grid, block, bufs, None, 5, scal, len(scalars), None)
+        assert rc == StatusCode.InvalidArgument, name
+        assert b"sizes" in lib.qmm_last_error()
+    backend.Synchronize()
+    assert np.all(backend.CopyD2H(out, dtype=np.float32) == 7.0)

@@ -76,3 +76,65 @@ def test_recorded_decode_step_replays_like_eager(backend):
         backend.LaunchKernel(kw, KernelLaunch(grid_x=n // 64 + 1, grid_y=1, buffers=[wrap(xb), wrap(gate), wrap(yb)],
                                               scalars=[big_m, n, k]))
         torch.cuda.synchronize()
+
+
+def test_prefill_call_recorded_with_a_caller_owned_workspace(backend):
+    """A prefill-sized Q4_K call (64 rows: fp16 MFMA path, which needs scratch) recorded into a HIP
+    graph with a workspace the caller set beforehand: nothing is allocated while recording, every
+    replay equals the eager result, a launch that needs more than the workspace holds is refused,
+    and clearing the workspace restores the library-owned one."""
+    from tessera_amd import StatusCode, StatusError
+    dev = torch.device("cuda:0")
+    g = synth.rng(901)
+    m, n, k = 64, 1030, 4096
+    to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    wrap = lambda t: backend.WrapBuffer(t.data_ptr(), t.numel() * t.element_size())
+    w_h = synth.q4k_weights(g, n, k)
+    w = to_dev(w_h)
+    x = torch.empty(m * k, device=dev)
+    y = torch.empty(m * n, device=dev)
+    kern = backend.LoadKernel("gemm_q4k_wmma")
+    need = backend.WorkspaceBytes(kern, [m, n, k])
+    assert need >= m * k * 2                                   # the fp16 copy of the activations at least
+    assert backend.WorkspaceBytes(backend.LoadKernel("gemm_q4k_vec"), [1, n, k, 1]) == 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    launch = KernelLaunch(grid_x=n // 64 + 1, buffers=[wrap(x), wrap(w), wrap(y)], scalars=[m, n, k])
+    cur = torch.cuda.current_stream()
+    backend.SetStream(cur.cuda_stream)
+    backend.SetWorkspace(wrap(ws))
+    try:
+        a = synth.activations_f32(synth.rng(11), m, k)
+        x.copy_(to_dev(a.reshape(-1)))
+        backend.LaunchKernel(kern, launch)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            backend.SetStream(torch.cuda.current_stream().cuda_stream)
+            backend.LaunchKernel(kern, launch)
+        backend.SetStream(cur.cuda_stream)
+        for seed in (11, 12, 13):
+            a = synth.activations_f32(synth.rng(seed), m, k)
+            x.copy_(to_dev(a.reshape(-1)))
+            y.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = y.cpu().numpy().copy()
+            y.fill_(float("nan"))
+            backend.LaunchKernel(kern, launch)
+            torch.cuda.synchronize()
+            eager = y.cpu().numpy().copy()
+            assert np.array_equal(got.view(np.uint32), eager.view(np.uint32)), seed
+            if seed == 11:
+                ref = oracle.gemm_q4k(a, w_h, m, n, k, threads=True)
+                rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+                assert float(np.max(np.abs(eager.reshape(m, n) - ref))) <= 4e-3 * rms
+        # twice the rows need twice the scratch: refused, nothing launched, nothing allocated
+        xb = torch.empty(2 * m * k, device=dev)
+        yb = torch.empty(2 * m * n, device=dev)
+        with pytest.raises(StatusError) as err:
+            backend.LaunchKernel(kern, KernelLaunch(grid_x=1, buffers=[wrap(xb), wrap(w), wrap(yb)], scalars=[2 * m, n, k]))
+        assert err.value.code == StatusCode.InvalidArgument and "workspace" in str(err.value)
+    finally:
+        backend.SetWorkspace(None)
+    backend.LaunchKernel(kern, KernelLaunch(grid_x=1, buffers=[wrap(xb), wrap(w), wrap(yb)], scalars=[2 * m, n, k]))
+    torch.cuda.synchronize()

@@ -265,3 +265,22 @@ def test_down_q6k_matches_oracle(backend, experts, hidden, inter, top_k, rows):
         ref = want + (prev.astype(np.float64) if accumulate else 0.0)
         base = want      # the bound is relative to the routed sum, not to what it is added to
         assert rel_err(got - (prev if accumulate else 0), base) <= TOL, (accumulate, rel_err(got, ref))
+
+
+@pytest.mark.parametrize("n,idx", [(1, 0), (2048, 3), (5000, 7)])
+def test_moe_scale_add_matches_reference_formula(backend, n, idx):
+    """o = a + f[idx] * b (src/backends/rocm/rocm_kernels_basic.cpp:1932-1942): the shared expert's
+    output scaled by its gate and added to the routed sum.  One multiply and one add per element;
+    the device may contract them into a fused multiply-add, so the result is one of the two."""
+    g = synth.rng(7000 + n)
+    a = g.standard_normal(n).astype(np.float32)
+    b = g.standard_normal(n).astype(np.float32)
+    f = g.standard_normal(8).astype(np.float32)
+    da, db, df = backend.Upload(a), backend.Upload(b), backend.Upload(f)
+    do = backend.AllocateBuffer(4 * n)
+    run(backend, "moe_scale_add", [da, db, df, do], [n, idx], grid=((n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(do, dtype=np.float32)
+    separate = a + f[idx] * b                                                     # rounded product, then the sum
+    fused = (a.astype(np.float64) + np.float64(f[idx]) * b.astype(np.float64)).astype(np.float32)
+    assert np.all((got == separate) | (got == fused))

@@ -68,6 +68,18 @@ def test_gemm_mxfp4_matches_oracle(backend, n, k, m):
     assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 200, 1024), (20, 131, 5120), (33, 64, 2048), (64, 515, 1280), (100, 96, 4096)])
+def test_gemm_mxfp4_batched_matches_oracle(backend, m, n, k):
+    """The id ProjectBatch issues for MXFP4 with more than 16 rows
+    (src/core/decode_internal.hpp:1494-1504): fp32 activations, no activation quantization."""
+    g = synth.rng(2100 * m + n + k)
+    w = synth.mxfp4_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_mxfp4(a, w, m, n, k)
+    got = mx_gemm(backend, "gemm_mxfp4_batched", a, w, m, n, k)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+
+
 @pytest.mark.parametrize("n,k", [(3001, 96), (3003, 352), (2999, 768), (3001, 1280), (3005, 2560), (4099, 3072),
                                  (3002, 3584), (6007, 5120), (1027, 8192)])
 @pytest.mark.parametrize("m", [1, 2, 4])

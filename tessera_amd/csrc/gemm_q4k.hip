@@ -11,11 +11,13 @@
 //
 // Weights never exist dequantized in memory: the raw 144-byte super-blocks travel
 // HBM -> LDS by direct loads, and each wavefront decodes the eight weights a lane owes the
-// B operand of one MFMA straight from those bytes into registers -- a nibble pair is masked
-// into the mantissa of an fp16 constant in one v_and_or_b32 (1024.0 for low nibbles, 64.0 for
-// high ones, so neither needs a shift), the constant subtracted, then one packed fma with the
-// sub-block's (d*sc, dmin*mn) pair, i.e. w16 = fma(q, RN16(d*sc), -RN16(dmin*mn)): three VALU
-// instructions per two weights.  The nibble pairs come out of a dword in the order
+// B operand of one MFMA straight from those bytes into registers.  The decode is the reference's:
+// the fp32 value fma(q, d*sc, -(dmin*mn)) -- d*sc, dmin*mn and q*(d*sc) are exact in fp32, so this
+// is DequantizeQ4K's value bit for bit -- rounded ONCE to fp16 (round to nearest even), which is
+// what the reference's tensor-core tile stages (rocm_kernels_wmma.cpp:73-77).  A masked nibble
+// pair masked in place is a pair of fp16 subnormals (q * 2^-24) that the mixed-precision
+// multiply-add consumes directly, so two weights cost one mask and two multiply-adds that also
+// round to fp16.  The nibble pairs come out of a dword in the order
 // (k0,k2),(k1,k3); instead of un-shuffling them, the fp16 copy of A is written with the same
 // order inside every group of 8, which a dot product cannot see.
 //
@@ -100,38 +102,16 @@ __device__ __forceinline__ void unrolled(F&& body) {
   }
 }
 
-// (x & mask) | magic in one instruction.  With the two constants in registers the three-operand
-// form applies; as literals they would cost an AND and an OR (one literal an instruction).
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(mask), "v"(magic));
-  return r;
-}
-
-// Nibble decode constants, kept in registers for and_or.  Low nibbles (bits [3:0] and [19:16])
-// are or-ed into the mantissa of 1024.0, high nibbles (bits [7:4] and [23:20]) into that of 64.0,
-// where the same four bits weigh 1: no shift is needed for either, and subtracting the base
-// leaves the exact integer 0..15.
-struct NibbleConsts {
-  uint32_t mask[2], magic[2];
-  half2_t base[2];
-};
-__device__ __forceinline__ NibbleConsts nibble_consts() {
-  NibbleConsts c;
-  c.mask[0] = 0x000F000Fu, c.mask[1] = 0x00F000F0u;
-  c.magic[0] = 0x64006400u, c.magic[1] = 0x54005400u;
-  asm volatile("" : "+v"(c.mask[0]), "+v"(c.mask[1]), "+v"(c.magic[0]), "+v"(c.magic[1]));  // not literals
-  c.base[0] = half2_t{1024, 1024}, c.base[1] = half2_t{64, 64};
-  return c;
-}
-
-// Two packed fp16 weights q * scale - min from the nibbles (low: HI = 0, high: HI = 1) of bytes 0
-// and 2 of `x`; `sm` holds the sub-block's fp16 scale in its low half and minus its min in the
-// high half.
+// Two packed fp16 weights RN16(fma(q, dsc, ndmm)) from the nibbles (low: HI = 0, high: HI = 1) of
+// bytes 0 and 2 of `x`.  A nibble masked in place inside a 16-bit half is the fp16 subnormal
+// q * 2^-24 (16 q * 2^-24 for a high nibble), which the mixed-precision multiply-add reads as it
+// is: `dsc24` is d*sc * 2^24 (d*sc * 2^20 for high nibbles), so the fp32 result is exactly
+// DequantizeQ4K's and one instruction per weight forms it and rounds it to fp16.
 template <int HI>
-__device__ __forceinline__ half2_t decode_pair(uint32_t x, const NibbleConsts& c, half2_t sm) {
-  const half2_t q = bit_cast<half2_t>(and_or(x, c.mask[HI], c.magic[HI])) - c.base[HI];   // exact 0..15
-  return __builtin_elementwise_fma(q, half2_t{sm[0], sm[0]}, half2_t{sm[1], sm[1]});
+__device__ __forceinline__ half2_t decode_pair(uint32_t x, float dsc24, float ndmm) {
+  const half2_t q = bit_cast<half2_t>(x & (HI ? 0x00F000F0u : 0x000F000Fu));
+  return half2_t{static_cast<_Float16>(fmaf(static_cast<float>(q[0]), dsc24, ndmm)),
+                 static_cast<_Float16>(fmaf(static_cast<float>(q[1]), dsc24, ndmm))};
 }
 
 // The 6-bit scales and mins of a super-block, one byte each (src/core/numerics/quant.cpp:58-70):
@@ -148,15 +128,17 @@ __device__ __forceinline__ ScaleBytes unpack_scales(uint32_t s0, uint32_t s1, ui
   return r;
 }
 
-// (d * sc, -(dmin * mn)) of sub-block SB as packed fp16, each product rounded once to nearest
-// even (the 6-bit integers are exact in fp16).  `d_negdmin` is the block header with the sign of
-// its high half flipped.
+// (d * sc * 2^24, -(dmin * mn)) of sub-block SB in fp32, both exact (11-bit header times 6-bit
+// integer; the 2^24 undoes the subnormal reading of the nibbles in decode_pair).  Odd sub-blocks
+// live in the high nibbles, which read as 16 q: their factor is 2^20.
+struct ScaleMin {
+  float dsc, ndmm;
+};
 template <int SB>
-__device__ __forceinline__ half2_t scale_min_f16(const ScaleBytes& sbytes, half2_t d_negdmin) {
-  constexpr uint32_t kSel = 0x0C000C00u | ((4u + (SB & 3)) << 16) | (SB & 3);   // bytes: sc, 0, mn, 0
-  const uint32_t pair = __builtin_amdgcn_perm(sbytes.mn[SB >> 2], sbytes.sc[SB >> 2], kSel);
-  const half2_t ints = bit_cast<half2_t>(pair | 0x64006400u) - half2_t{1024, 1024};
-  return ints * d_negdmin;
+__device__ __forceinline__ ScaleMin scale_min_f32(const ScaleBytes& sbytes, float d, float ndmin) {
+  const float sc = static_cast<float>((sbytes.sc[SB >> 2] >> (8 * (SB & 3))) & 0xFFu);
+  const float mn = static_cast<float>((sbytes.mn[SB >> 2] >> (8 * (SB & 3))) & 0xFFu);
+  return ScaleMin{d * sc * ((SB & 1) ? 0x1p20f : 0x1p24f), ndmin * mn};
 }
 
 // Wavefronts of a BM x BN tile whose wavefronts each own WM rows x WN columns.
@@ -238,7 +220,6 @@ __device__ __forceinline__ void q4k_gemm_tile(
   for (int tt = 0; tt < 2; ++tt) a_fr[tt] = (wave_m * WM + l32) * 64u + (((tt * 2u + kg) ^ ((l32 >> 2) & 3u)) * 16u);
 
   const uint32_t slices = k / 32;
-  const NibbleConsts nc = nibble_consts();
 
   // Prologue: first super-block and three activation slices in flight, then the first of each
   // is waited for.
@@ -251,12 +232,13 @@ __device__ __forceinline__ void q4k_gemm_tile(
   for (uint32_t blk = 0; blk < row_blocks; ++blk) {
     const uint8_t* raw = lds + 4 * kAStage + (blk & 1u) * kWStage + w_row;
     const bool more = blk + 1 < row_blocks;        // uniform
-    half2_t d_negdmin[kTJ];                        // block header, sign of dmin flipped
+    float hd[kTJ], hndmin[kTJ];                    // block header: d and -dmin
     ScaleBytes sbytes[kTJ];
 #pragma unroll
     for (int j = 0; j < kTJ; ++j) {
       const uint4 head = *reinterpret_cast<const uint4*>(raw + j * 32 * 144);
-      d_negdmin[j] = bit_cast<half2_t>(head.x ^ 0x80000000u);
+      hd[j] = half_bits_to_float(head.x & 0xFFFFu);
+      hndmin[j] = -half_bits_to_float(head.x >> 16);
       sbytes[j] = unpack_scales(head.y, head.z, head.w);
     }
     uint32_t qw[kTJ][4], qs8[kTJ][4];
@@ -274,7 +256,7 @@ __device__ __forceinline__ void q4k_gemm_tile(
       half8_t b[kTJ][2];
 #pragma unroll
       for (int j = 0; j < kTJ; ++j) {
-        const half2_t sm = scale_min_f16<sb>(sbytes[j], d_negdmin[j]);
+        const ScaleMin sm = scale_min_f32<sb>(sbytes[j], hd[j], hndmin[j]);
         if (kHi == 0) {
           const uint8_t* qp = raw + j * 32 * 144 + 16 + (sb >> 1) * 32 + kg * 8u;
           const uint2 q0 = *reinterpret_cast<const uint2*>(qp);
@@ -285,8 +267,8 @@ __device__ __forceinline__ void q4k_gemm_tile(
         }
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
-          const half2_t p0 = decode_pair<kHi>(qw[j][2 * tt], nc, sm), p1 = decode_pair<kHi>(qs8[j][2 * tt], nc, sm);
-          const half2_t p2 = decode_pair<kHi>(qw[j][2 * tt + 1], nc, sm), p3 = decode_pair<kHi>(qs8[j][2 * tt + 1], nc, sm);
+          const half2_t p0 = decode_pair<kHi>(qw[j][2 * tt], sm.dsc, sm.ndmm), p1 = decode_pair<kHi>(qs8[j][2 * tt], sm.dsc, sm.ndmm);
+          const half2_t p2 = decode_pair<kHi>(qw[j][2 * tt + 1], sm.dsc, sm.ndmm), p3 = decode_pair<kHi>(qs8[j][2 * tt + 1], sm.dsc, sm.ndmm);
           b[j][tt] = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
         }
       }

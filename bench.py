@@ -248,6 +248,7 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     a = to_dev(synth.activations_bf16(g, m, k))
     w_q = to_dev(synth.q4k_weights(g, n, k))
     kw = backend.LoadKernel("gemm_q4k_wmma")
+    kmb = backend.LoadKernel("gemm_mxfp4_batched")
     a8 = torch.empty(m * k, dtype=torch.uint8, device=dev)
     asc = torch.empty(m, dtype=torch.float32, device=dev)
     backend.LaunchKernel(kq, KernelLaunch(grid_x=m, buffers=[wrap(a), wrap(a8), wrap(asc)], scalars=[m, k]))
@@ -263,6 +264,19 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
                                          scalars=[m, nn, k, 1, 0]))], 10, graph=False)
         prefill[f"mxfp4_{label}"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * nn * k / us / 1e6, 1),
                                      "frac_fp8_peak": round(2 * m * nn * k / us / 1e6 / 5000.0, 4)}
+        # the same with the per-token quantization of the activation inside the timed region
+        us = timed_us([(kq, KernelLaunch(grid_x=m, buffers=[wrap(a), wrap(a8), wrap(asc)], scalars=[m, k])),
+                       (kg, KernelLaunch(grid_x=nn // 64, buffers=[wrap(a8), wrap(wm), wrap(asc), wrap(wref), wrap(y)],
+                                         scalars=[m, nn, k, 1, 0]))], 10, graph=False)
+        prefill[f"mxfp4_{label}"].update({"ms_with_quantize": round(us / 1e3, 4),
+                                          "TFLOPs_with_quantize": round(2 * m * nn * k / us / 1e6, 1)})
+        # fp32 activation rows, not quantized ("gemm_mxfp4_batched", the reference's prefill id): bf16-valued
+        # rows are two E4M3 terms, so the matrix cores do twice the E4M3 x E2M1 work counted here
+        us = timed_us([(kmb, KernelLaunch(grid_x=(nn + 7) // 8, buffers=[wrap(a), wrap(wm), wrap(y)], scalars=[m, nn, k]))],
+                      10, graph=False)
+        prefill[f"mxfp4_f32rows_{label}"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * nn * k / us / 1e6, 1),
+                                             "frac_bf16_peak": round(2 * m * nn * k / us / 1e6 / 2500.0, 4),
+                                             "e4m3_terms": 2}
     # Q6_K and Q5_K prefill: weights decoded to fp16 per call, then the dense fp16 MFMA GEMM
     for fmt, gen in (("q6k", synth.q6k_weights), ("q5k", synth.q5k_weights)):
         wf = to_dev(gen(g, n, k))

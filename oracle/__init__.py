@@ -59,6 +59,7 @@ def _load() -> C.CDLL:
         "orc_dequantize_q6k_rows": (None, [u8p, f32p, sz]),
         "orc_gemm_q6k_ref": (C.c_int, [f32p, u8p, f32p, sz, sz, sz, C.c_int]),
         "orc_gemm_mxfp4_ref": (C.c_int, [f32p, u8p, u8p, f32p, sz, sz, sz]),
+        "orc_gemm_mxfp4_ref_omp": (C.c_int, [f32p, u8p, u8p, f32p, sz, sz, sz]),
         "orc_dequantize_mxfp4": (C.c_int, [u8p, f32p, sz, sz]),
         "orc_gemm_fp8_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
         "orc_fold_entry": (C.c_uint8, [C.c_uint, C.c_uint]),
@@ -240,12 +241,12 @@ def split_mxfp4(packed, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:
     return packed[: n * k // 2], packed[n * k // 2:]
 
 
-def gemm_mxfp4(a, packed, m: int, n: int, k: int) -> np.ndarray:
+def gemm_mxfp4(a, packed, m: int, n: int, k: int, threads: bool = False) -> np.ndarray:
     a = _f32(a)
     blob, s = split_mxfp4(packed, n, k)
     c = np.empty((m, n), dtype=np.float32)
-    _check(_lib.orc_gemm_mxfp4_ref(_p(a, C.c_float), _p(blob, C.c_uint8), _p(s, C.c_uint8),
-                                   _p(c, C.c_float), m, n, k))
+    fn = _lib.orc_gemm_mxfp4_ref_omp if threads else _lib.orc_gemm_mxfp4_ref
+    _check(fn(_p(a, C.c_float), _p(blob, C.c_uint8), _p(s, C.c_uint8), _p(c, C.c_float), m, n, k))
     return c
 
 

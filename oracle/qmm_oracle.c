@@ -511,6 +511,41 @@ int orc_gemm_mxfp4_ref(const float* a, const uint8_t* w, const uint8_t* s, float
   return ORC_OK;
 }
 
+/* Same arithmetic with the weight rows spread over OpenMP threads: a row is decoded once (the
+ * same product sc * e2m1 as above), every output keeps its sequential fma chain, so the result
+ * equals orc_gemm_mxfp4_ref bit for bit (checked in tests/test_oracle_gemm.py). */
+int orc_gemm_mxfp4_ref_omp(const float* a, const uint8_t* w, const uint8_t* s, float* c, size_t m,
+                           size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0 || k % MX_BLOCK != 0) return ORC_INVALID_ARGUMENT;
+  const size_t nb = k / MX_BLOCK;
+  int failed = 0;
+#pragma omp parallel
+  {
+    float* row = (float*)malloc(k * sizeof(float));
+    if (!row) {
+#pragma omp atomic write
+      failed = 1;
+    }
+#pragma omp for schedule(static)
+    for (long long j = 0; j < (long long)n; ++j) {
+      if (!row) continue;
+      for (size_t t = 0; t < k; ++t) {
+        const uint8_t byte = w[((size_t)j * k + t) / 2];
+        const uint8_t nib = (t % 2 == 0) ? (byte & 15u) : (byte >> 4);
+        row[t] = orc_e8m0_to_float(s[(size_t)j * nb + t / MX_BLOCK]) * orc_f4e2m1_to_float(nib);
+      }
+      for (size_t i = 0; i < m; ++i) {
+        const float* ar = a + i * k;
+        float acc = 0.0f;
+        for (size_t t = 0; t < k; ++t) acc = fmaf(ar[t], row[t], acc);
+        c[i * n + (size_t)j] = acc;
+      }
+    }
+    free(row);
+  }
+  return failed ? ORC_OOM : ORC_OK;
+}
+
 /* MXFP4 weights -> fp32, n x k, from the packed device layout (blob then scales,
  * include/tessera/backend.hpp:195-201). */
 int orc_dequantize_mxfp4(const uint8_t* packed, float* out, size_t n, size_t k) {

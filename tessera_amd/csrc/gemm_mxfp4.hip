@@ -30,6 +30,7 @@
 namespace qmm {
 namespace {
 
+constexpr int kMaxTerms = 4;                // E4M3 terms an fp32 activation is split into at most
 constexpr int kKS = 128;                    // K per step: one 32-bit word of E8M0 bytes per weight row
 constexpr int kDmaPerStage = 13;            // direct loads a wavefront issues per stage (8 A, 4 B, 1 scales)
 
@@ -47,10 +48,15 @@ __device__ __forceinline__ void direct_load4(const void* base, uint32_t voff, ui
                :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
-template <int BM, int BN, int WM, int WN>
+// SPLIT: the activation is a sum of E4M3 terms (see split_rows_kernel): a8 holds kMaxTerms
+// planes of m x k codes, term t weighing 2^(-4t); `need` says how many terms each row has.  A
+// tile walks K once per term it needs, all into the same accumulators, the term's weight being
+// the E8M0 scale of the A operand.
+template <int BM, int BN, int WM, int WN, bool SPLIT>
 __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
     const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
-    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end) {
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end,
+    const uint8_t* __restrict__ need) {
   constexpr int kWaves = WM * WN;
   static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BN % 64 == 0, "tile shape");
   static_assert((BM / 8) % kWaves == 0 && (BN / 16) % kWaves == 0, "direct-load blocks divide among the wavefronts");
@@ -79,9 +85,24 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   struct Source {
     const uint8_t *a, *b, *s;           // tile origins (wave-uniform)
     uint32_t a_off[kABlk], b_off[kBBlk], s_off;
+    uint32_t terms;                     // passes over K (SPLIT)
+  };
+  const size_t plane = static_cast<size_t>(m) * k;
+  // Terms the rows m0 .. m0 + BM - 1 need: the largest of their `need` bytes (wave-uniform).
+  auto tile_terms = [&](uint32_t m0) -> uint32_t {
+    if (!SPLIT) return 1u;
+    float most = 1.0f;
+#pragma unroll
+    for (int i = 0; i < (BM + 63) / 64; ++i) {
+      const uint32_t row = m0 + i * 64u + lane;
+      if (i * 64u + lane < BM && row < m) most = fmaxf(most, static_cast<float>(need[row]));
+    }
+    const uint32_t terms = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(wave_max(most)));
+    return terms < static_cast<uint32_t>(kMaxTerms) ? terms : static_cast<uint32_t>(kMaxTerms);
   };
   auto locate = [&](uint32_t tile, Source& src) {
     const uint32_t m0 = (tile / tiles_n) * BM, n0 = n_begin + (tile % tiles_n) * BN;
+    src.terms = tile_terms(m0);
     src.a = a8 + static_cast<size_t>(m0) * k;
     src.b = w + static_cast<size_t>(n0) * row_bytes;
     src.s = w + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(n0) * row_blocks;
@@ -100,9 +121,9 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
     const uint32_t row = 64u * (wave % (BN / 64)) + lane;
     src.s_off = (n0 + row < n ? row : n - 1u - n0) * row_blocks;
   };
-  auto issue_stage = [&](uint32_t stage_off, const Source& src, uint32_t k0) {
+  auto issue_stage = [&](uint32_t stage_off, const Source& src, uint32_t k0, uint32_t term) {
     const uint32_t stage = lds_base + stage_off;
-    const uint8_t* ga = src.a + k0;
+    const uint8_t* ga = src.a + (SPLIT ? term * plane : 0) + k0;
     const uint8_t* gb = src.b + k0 / 2;
     const uint8_t* gs = src.s + k0 / 32;
 #pragma unroll
@@ -158,18 +179,20 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   };
 
   float16_t acc[kTI][kTJ];
-  auto mfmas = [&](const Frag& f, int ks, const int (&sv)[kTJ]) {
+  auto mfmas = [&](const Frag& f, int ks, const int (&sv)[kTJ], int sa) {
 #pragma unroll
     for (int j = 0; j < kTJ; ++j) {
       const int8v_t bf = int8v_t{static_cast<int>(f.b[j].x), static_cast<int>(f.b[j].y),
                                  static_cast<int>(f.b[j].z), static_cast<int>(f.b[j].w), 0, 0, 0, 0};
 #pragma unroll
       for (int i = 0; i < kTI; ++i) {
-        // A: E4M3 (cbsz 0) with unit scale (E8M0 127); B: E2M1 (blgp 4) with the block scale.
+        // A: E4M3 (cbsz 0) with unit scale (E8M0 127), or the term's weight; B: E2M1 (blgp 4)
+        // with the block scale.
+        const int a_scale = SPLIT ? sa : 0x7F7F7F7F;
         if (ks == 0) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 0, sv[j]);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], bf, acc[i][j], 0, 4, 0, a_scale, 0, sv[j]);
         } else {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], bf, acc[i][j], 0, 4, 0, 0x7F7F7F7F, 2, sv[j]);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], bf, acc[i][j], 0, 4, 0, a_scale, 2, sv[j]);
         }
       }
     }
@@ -199,18 +222,20 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   const uint32_t my_tiles = (tiles - tile + gridDim.x - 1) / gridDim.x;
   Source src;
   locate(tile, src);
-  uint32_t load_tile = tile, load_step = 0;
+  uint32_t load_tile = tile, load_step = 0, load_term = 0;
   auto advance_load = [&]() {
     if (++load_step == steps) {          // uniform
       asm volatile("" ::: "memory");     // keeps this rare block a branch, not a chain of selects
       load_step = 0;
+      if (SPLIT && ++load_term < src.terms) return;
+      load_term = 0;
       load_tile += gridDim.x;
       if (load_tile < tiles) locate(load_tile, src);
     }
   };
-  issue_stage(0, src, 0);
+  issue_stage(0, src, 0, 0);
   advance_load();
-  issue_stage(kStage, src, load_step * kKS);
+  issue_stage(kStage, src, load_step * kKS, load_term);
   advance_load();
   publish();
 #pragma unroll
@@ -221,24 +246,28 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   for (uint32_t done_tiles = 0; done_tiles < my_tiles; ++done_tiles) {
-    for (uint32_t cur = 0; cur < steps; ++cur) {
-      // One step of K: `rd` is the stage being multiplied, `nx` the stage of the step after
-      // it and `fill` the one the load cursor's step goes into.  Two wavefronts share each
-      // SIMD, so one's fragment reads run under the other's MFMAs.
-      issue_stage(fill, src, load_step * kKS);
-      read_scales(rd, sv_raw);
+    const uint32_t terms = tile_terms((tile / tiles_n) * BM);
+    for (uint32_t term = 0; term < terms; ++term) {
+      const int sa = 0x7F - 4 * static_cast<int>(term);      // E8M0 of 2^(-4 term), byte 0 is the one used
+      for (uint32_t cur = 0; cur < steps; ++cur) {
+        // One step of K: `rd` is the stage being multiplied, `nx` the stage of the step after
+        // it and `fill` the one the load cursor's step goes into.  Two wavefronts share each
+        // SIMD, so one's fragment reads run under the other's MFMAs.
+        issue_stage(fill, src, load_step * kKS, load_term);
+        read_scales(rd, sv_raw);
 #pragma unroll
-      for (int j = 0; j < kTJ; ++j) sv[j] = static_cast<int>(sv_raw[j] >> (kg * 8u));
-      read_frags(rd, 0, f0);
-      read_frags(rd, 1, f1);
-      mfmas(f0, 0, sv);
-      mfmas(f1, 1, sv);
-      publish();
-      const uint32_t done = rd;
-      rd = nx;
-      nx = fill;
-      fill = done;
-      advance_load();
+        for (int j = 0; j < kTJ; ++j) sv[j] = static_cast<int>(sv_raw[j] >> (kg * 8u));
+        read_frags(rd, 0, f0);
+        read_frags(rd, 1, f1);
+        mfmas(f0, 0, sv, sa);
+        mfmas(f1, 1, sv, sa);
+        publish();
+        const uint32_t done = rd;
+        rd = nx;
+        nx = fill;
+        fill = done;
+        advance_load();
+      }
     }
 
     // Epilogue: lane holds column l32 and rows (e/4)*8 + kg*4 + e%4 of each 32 x 32 tile.
@@ -532,6 +561,103 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void mxfp4_a8_stream_kernel(
   }
 }
 
+
+// ---- fp32 activations as a sum of E4M3 terms (for the ids whose contract is fp32 rows) -------
+// A row is written as  a = s0 * (h0 + h1/16 + h2/256 + h3/4096),  s0 = 2^(floor(log2 rowmax) - 7),
+// every h an E4M3 number: h0 is a/s0 (below 256) cut to its four leading significant bits, h1
+// the same of 16 * (a/s0 - h0), and so on; the last term rounds instead of cutting.  All of it is
+// exact fp32 arithmetic, so a value of 4T significant bits is reproduced exactly by T terms as
+// long as its last bit is not below the E4M3 grid of the last term (2^-9 * 16^-(T-1) * s0, i.e.
+// rowmax * 2^-(12+4T) at the least); what lies below is dropped.  `need` = terms the row's
+// widest significand asks for: 2 for bf16-valued rows, 3 up to 12 bits, else 4 (16 bits kept).
+// A non-finite element becomes the E4M3 NaN, which spoils its row of C.
+__device__ __forceinline__ uint32_t e4m3_cut(float x, float& val) {        // |x| < 256
+  const uint32_t b = bit_cast<uint32_t>(x), sign = (b >> 24) & 0x80u;
+  if (fabsf(x) >= 0x1p-6f) {
+    const uint32_t tb = b & 0xFFF00000u;                                  // sign, exponent, three mantissa bits
+    val = bit_cast<float>(tb);
+    return sign | ((((tb >> 23) & 0xFFu) - 120u) << 3) | ((tb >> 20) & 7u);
+  }
+  const uint32_t q = static_cast<uint32_t>(fabsf(x) * 512.0f);           // the subnormal grid, 2^-9
+  val = copysignf(static_cast<float>(q) * 0x1p-9f, x);
+  return sign | q;
+}
+__device__ __forceinline__ uint32_t e4m3_near(float x) {                  // |x| < 256, to nearest
+  const uint32_t b = bit_cast<uint32_t>(x), sign = (b >> 24) & 0x80u, mag = b & 0x7FFFFFFFu;
+  if (fabsf(x) >= 0x1p-6f) {
+    const uint32_t r = mag + 0x7FFFFu + ((mag >> 20) & 1u);               // carry may reach the exponent (256 = 0x78)
+    return sign | ((r >> 20) - (120u << 3));
+  }
+  return sign | static_cast<uint32_t>(rintf(fabsf(x) * 512.0f));         // 8 = 2^-6, the first normal code
+}
+
+__global__ __launch_bounds__(256) void split_rows_kernel(const float* __restrict__ a, uint8_t* __restrict__ planes,
+                                                         float* __restrict__ as, uint8_t* __restrict__ need,
+                                                         uint32_t m, uint32_t k) {
+  __shared__ float s_max[4];
+  __shared__ uint32_t s_or[4];
+  const uint32_t row = blockIdx.x, t = threadIdx.x;
+  const float* ar = a + static_cast<size_t>(row) * k;
+  float amax = 0.0f;
+  uint32_t low = 0;
+  for (uint32_t i = t * 4u; i < k; i += 1024u) {                          // k is a multiple of 128
+    const uint4 v = load_u4(ar + i);
+    const uint32_t b[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t mag = b[e] & 0x7FFFFFFFu;
+      if (mag < 0x7F800000u) {
+        amax = fmaxf(amax, bit_cast<float>(mag));
+        if (mag != 0) low |= mag & 0x7FFFFFu;
+      }
+    }
+  }
+  amax = wave_max(amax);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) low |= __shfl_xor(low, off, kWave);
+  if ((t & 63u) == 0) {
+    s_max[t >> 6] = amax;
+    s_or[t >> 6] = low;
+  }
+  __syncthreads();
+  amax = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+  low = s_or[0] | s_or[1] | s_or[2] | s_or[3];
+  // floor(log2 amax), kept where both s0 and 1/s0 are normal numbers
+  int e = static_cast<int>(bit_cast<uint32_t>(amax) >> 23) - 127;
+  e = amax == 0.0f ? 7 : (e < -112 ? -112 : e);
+  const float s0 = bit_cast<float>(static_cast<uint32_t>(e - 7 + 127) << 23);
+  const float inv = bit_cast<float>(static_cast<uint32_t>(7 - e + 127) << 23);
+  if (t == 0) {
+    as[row] = s0;
+    const uint32_t bits = 24u - static_cast<uint32_t>(__builtin_ctz(low | 0x800000u));
+    need[row] = static_cast<uint8_t>(bits <= 8 ? 2 : (bits <= 12 ? 3 : 4));
+  }
+  const size_t plane = static_cast<size_t>(m) * k;
+  uint8_t* out = planes + static_cast<size_t>(row) * k;
+  for (uint32_t i = t * 4u; i < k; i += 1024u) {
+    const uint4 v = load_u4(ar + i);
+    const uint32_t b[4] = {v.x, v.y, v.z, v.w};
+    uint32_t code[kMaxTerms] = {0, 0, 0, 0};
+#pragma unroll
+    for (int el = 0; el < 4; ++el) {
+      if ((b[el] & 0x7FFFFFFFu) >= 0x7F800000u) {
+        code[0] |= 0x7Fu << (8 * el);
+        continue;
+      }
+      float r = bit_cast<float>(b[el]) * inv;
+#pragma unroll
+      for (int term = 0; term < kMaxTerms - 1; ++term) {
+        float val;
+        code[term] |= e4m3_cut(r, val) << (8 * el);
+        r = (r - val) * 16.0f;
+      }
+      code[kMaxTerms - 1] |= e4m3_near(r) << (8 * el);
+    }
+#pragma unroll
+    for (int term = 0; term < kMaxTerms; ++term) *reinterpret_cast<uint32_t*>(out + term * plane + i) = code[term];
+  }
+}
+
 }  // namespace
 
 bool gemm_mxfp4_a8_supported(uint64_t k) { return k % 128 == 0 && k <= (1u << 24); }
@@ -540,11 +666,34 @@ namespace {
 
 template <int BM, int BN, int WM, int WN>
 void launch_range(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m, uint32_t n,
-                  uint32_t k, uint32_t n_begin, uint32_t n_end, uint32_t max_groups, hipStream_t stream) {
+                  uint32_t k, uint32_t n_begin, uint32_t n_end, uint32_t max_groups, const uint8_t* need,
+                  hipStream_t stream) {
   const uint32_t tiles = ((m + BM - 1) / BM) * ((n_end - n_begin + BN - 1) / BN);
   const uint32_t grid = tiles < max_groups ? tiles : max_groups;
-  hipLaunchKernelGGL((mxfp4_a8_gemm_kernel<BM, BN, WM, WN>), dim3(grid), dim3(64 * WM * WN), 0, stream,
-                     a8, as, w, c, m, n, k, n_begin, n_end);
+  if (need != nullptr) {
+    hipLaunchKernelGGL((mxfp4_a8_gemm_kernel<BM, BN, WM, WN, true>), dim3(grid), dim3(64 * WM * WN), 0, stream,
+                       a8, as, w, c, m, n, k, n_begin, n_end, need);
+  } else {
+    hipLaunchKernelGGL((mxfp4_a8_gemm_kernel<BM, BN, WM, WN, false>), dim3(grid), dim3(64 * WM * WN), 0, stream,
+                       a8, as, w, c, m, n, k, n_begin, n_end, need);
+  }
+}
+
+// Tiled launch of C = diag(as) . A8 . deq(W)^T; `need` non-null selects the split-activation form.
+void launch_tiles(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m, uint32_t n,
+                  uint32_t k, const uint8_t* need, hipStream_t stream) {
+  const uint32_t cus = static_cast<uint32_t>(num_cus());
+  const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u;
+  const uint32_t tiles = tiles_m * tiles_n;
+  uint32_t main_tn = tiles_n;
+  if (tiles > cus && tiles % cus != 0 && tiles % cus <= cus / 2) {
+    main_tn = (tiles / cus) * cus / tiles_m;
+  } else if (tiles < cus / 2) {
+    main_tn = 0;                        // too few large tiles to fill the chip: small tiles throughout
+  }
+  const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
+  if (n_split > 0) launch_range<256, 256, 4, 2>(a8, as, w, c, m, n, k, 0u, n_split, cus, need, stream);
+  if (n_split < n) launch_range<128, 64, 2, 2>(a8, as, w, c, m, n, k, n_split, n, 2u * cus, need, stream);
 }
 
 }  // namespace
@@ -573,18 +722,23 @@ hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_
     }
     return hipGetLastError();
   }
-  const uint32_t cus = static_cast<uint32_t>(num_cus());
-  const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u;
-  const uint32_t tiles = tiles_m * tiles_n;
-  uint32_t main_tn = tiles_n;
-  if (tiles > cus && tiles % cus != 0 && tiles % cus <= cus / 2) {
-    main_tn = (tiles / cus) * cus / tiles_m;
-  } else if (tiles < cus / 2) {
-    main_tn = 0;                        // too few large tiles to fill the chip: small tiles throughout
-  }
-  const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
-  if (n_split > 0) launch_range<256, 256, 4, 2>(a8, as, w, c, m, n, k, 0u, n_split, cus, stream);
-  if (n_split < n) launch_range<128, 64, 2, 2>(a8, as, w, c, m, n, k, n_split, n, 2u * cus, stream);
+  launch_tiles(a8, as, w, c, m, n, k, nullptr, stream);
+  return hipGetLastError();
+}
+
+bool gemm_mxfp4_f32_supported(uint64_t m, uint64_t k) { return m >= 17 && k >= 1024 && gemm_mxfp4_a8_supported(k); }
+
+size_t gemm_mxfp4_f32_workspace_bytes(uint64_t m, uint64_t k) {
+  return static_cast<size_t>(kMaxTerms) * m * k + ((m * 4 + 255) / 256) * 256 + ((m + 255) / 256) * 256;
+}
+
+hipError_t launch_mxfp4_f32_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
+                                 uint32_t n, uint32_t k, hipStream_t stream) {
+  uint8_t* planes = static_cast<uint8_t*>(workspace);
+  float* as = reinterpret_cast<float*>(planes + static_cast<size_t>(kMaxTerms) * m * k);
+  uint8_t* need = reinterpret_cast<uint8_t*>(as) + ((static_cast<size_t>(m) * 4 + 255) / 256) * 256;
+  hipLaunchKernelGGL(split_rows_kernel, dim3(m), dim3(256), 0, stream, a, planes, as, need, m, k);
+  launch_tiles(planes, as, w, c, m, n, k, need, stream);
   return hipGetLastError();
 }
 

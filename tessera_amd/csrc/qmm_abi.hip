@@ -148,6 +148,7 @@ void* decode_scratch(const LaunchCtx& c) {
 // few-row MFMA kernels (weights read once per eight rows); one row and small matrices stay on
 // the VALU GEMV, which needs no activation pre-pass.
 constexpr uint64_t kQ4KGemmMinRows = 17;
+constexpr uint64_t kMxfp4GemmMinRows = 17;   // below: the VALU GEMV passes, exact fp32 order
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 
@@ -494,6 +495,16 @@ qmm_status run_gemm_mxfp4(const LaunchCtx& c) {
   if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, mxfp4_bytes(n, k)) ||
       !c.fits(2, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_mxfp4: a buffer is smaller than m, n, k require");
+  }
+  // From 17 rows on the weights go through the matrix cores as they are (E2M1 operand, E8M0 block
+  // scale) and the fp32 rows as a short sum of E4M3 terms (gemm_mxfp4.hip).
+  if (m >= kMxfp4GemmMinRows && m <= 0xFFFFFFFFull && n <= 0xFFFFFFFFull && qmm::gemm_mxfp4_f32_supported(m, k)) {
+    void* ws = nullptr;
+    const qmm_status st = workspace(c, qmm::gemm_mxfp4_f32_workspace_bytes(m, k), &ws);
+    if (st != QMM_OK) return st;
+    return map_hip(qmm::launch_mxfp4_f32_gemm(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), ws,
+                                              static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                              static_cast<uint32_t>(k), c.stream));
   }
   return map_hip(qmm::launch_mxfp4_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2),
                                         static_cast<uint32_t>(m), static_cast<uint32_t>(n),
@@ -1055,6 +1066,9 @@ qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_
       const size_t gemm_ws = qmm::gemm_q4k_supported(m, k) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
       *out_bytes = ((gemm_ws + 255) & ~size_t{255}) + static_cast<size_t>(m) * n * 4;
     }
+  } else if (id == "gemm_mxfp4" || id == "gemm_mxfp4_batched") {
+    const uint64_t m = sc(0), k = sc(2);
+    if (m >= kMxfp4GemmMinRows && qmm::gemm_mxfp4_f32_supported(m, k)) *out_bytes = qmm::gemm_mxfp4_f32_workspace_bytes(m, k);
   } else if (starts("gemm_q5k") || starts("gemm_q6k")) {
     const uint64_t m = sc(0), n = sc(1), k = sc(2);
     if (m >= kQ4KGemmMinRows && qmm::gemm_kquant_f16_supported(m, n, k)) *out_bytes = qmm::gemm_kquant_f16_workspace_bytes(m, n, k);

@@ -65,6 +65,13 @@ bool gemm_mxfp4_a8_supported(uint64_t k);
 hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
 
+// MXFP4 weights, fp32 activation rows (17 or more): the rows are split into E4M3 terms in the
+// workspace and multiplied on the same scaled MFMA, one pass over K per term.
+bool gemm_mxfp4_f32_supported(uint64_t m, uint64_t k);
+size_t gemm_mxfp4_f32_workspace_bytes(uint64_t m, uint64_t k);
+hipError_t launch_mxfp4_f32_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
+                                 uint32_t n, uint32_t k, hipStream_t stream);
+
 // Q4_K prefill GEMM on fp16 MFMA (gemm_q4k.hip).  `workspace` holds m*k fp16 values.
 bool gemm_q4k_supported(uint64_t m, uint64_t k);
 size_t gemm_q4k_workspace_bytes(uint64_t m, uint64_t k);

@@ -4,6 +4,7 @@
 // ProjectBatch computes C (m x n fp32) = A (m x k fp32) . deq(W)^T for a quantized weight.
 #pragma once
 
+#include <cstdlib>
 #include <map>
 #include <string>
 
@@ -46,6 +47,18 @@ struct ProjectState {
   bool honour_reference_split = false;
   // Take the reference's three launches for the dense gate/up/silu even where the fused id exists.
   bool no_fused_ffn = false;
+  // MXFP4: the per-token E4M3 activation path (ProjectWmma).  As in the reference
+  // (src/models/qwen3_5/project.cpp:236-250) it is on unless TESSERA_MXFP4_WMMA=0 and serves
+  // m <= 16; more rows keep fp32 activations ("gemm_mxfp4_batched", which this backend runs on the
+  // matrix cores without quantizing the activation).
+  bool mxfp4_wmma = [] {
+    const char* env = std::getenv("TESSERA_MXFP4_WMMA");
+    return env == nullptr || std::atoi(env) != 0;
+  }();
+  // Opt-in, not a reference setting: also send m > 16 through ProjectWmma (k % 128 == 0).  Half
+  // the time of the fp32-row id, at the price of the E4M3 rounding of the activation (about 2^-4
+  // per element) that the reference's prefill does not have.
+  bool mxfp4_fp8_prefill = false;
 };
 
 inline Expected<const Kernel*> CachedKernel(Backend& backend, ProjectState& h, const std::string& id) {
@@ -142,7 +155,7 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
                                    Buffer& out, std::size_t m, std::size_t n, std::size_t k) {
   if (m == 0 || n == 0 || k == 0) return unexpected(StatusCode::InvalidArgument);
   if (dtype == DType::F4E2M1) {
-    if (m <= 16 || k % 128 == 0) {             // the reference caps the fp8 path at m = 16; here it scales on
+    if (h.mxfp4_wmma && (m <= 16 || (h.mxfp4_fp8_prefill && k % 128 == 0))) {
       auto done = ProjectWmma(backend, h, a, w, out, m, n, k);
       if (!done) return unexpected(done.error());
       if (*done) return {};

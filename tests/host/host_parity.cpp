@@ -92,7 +92,8 @@ struct Case {
   DType dtype;
   size_t m, n, k;
   bool reference_split;
-  double rel_tol, rms_tol;     // see tests/test_gpu_q4k.py, test_gpu_gemm_q4k.py, test_gpu_gemm_mxfp4.py
+  double rel_tol, rms_tol;     // see tests/test_gpu_q4k.py, test_gpu_gemm_q4k.py, test_gpu_gemm_mxfp4.py, test_gpu_gemm_mxfp4_f32.py
+  bool fp8_prefill = false;    // ProjectState::mxfp4_fp8_prefill: E4M3 activations beyond 16 rows (reference: QDQ + GemmMxFp4Ref)
 };
 const Case kCases[] = {
     {"q4k decode m=1 (gemm_q4k_vec)", DType::Q4K, 1, 640, 5120, false, 1e-3, 1e-3},
@@ -109,7 +110,10 @@ const Case kCases[] = {
     {"q5k prefill m=100 (gemm_q5k_wmma, fp16 MFMA)", DType::Q5K, 100, 257, 2304, false, 1.0, 4e-3},
     {"mxfp4 w4a8 m=1 (quantize_fp8_pack_rows + gemm_mxfp4_wmma)", DType::F4E2M1, 1, 512, 1024, false, 1e-3, 1e-3},
     {"mxfp4 w4a8 m=16 (streaming scaled MFMA)", DType::F4E2M1, 16, 512, 2048, false, 1e-2, 5e-4},
-    {"mxfp4 w4a8 m=300 (tiled scaled MFMA)", DType::F4E2M1, 300, 384, 1024, false, 1e-2, 5e-4},
+    {"mxfp4 w4a8 m=300 (tiled scaled MFMA, opt-in)", DType::F4E2M1, 300, 384, 1024, false, 1e-2, 5e-4, true},
+    {"mxfp4 prefill m=300, the reference's rule (gemm_mxfp4_batched, fp32 rows on the scaled MFMA)", DType::F4E2M1, 300, 384,
+     1024, false, 2e-3, 1e-4},
+    {"mxfp4 m=17 (gemm_mxfp4_batched)", DType::F4E2M1, 17, 200, 2048, false, 2e-3, 1e-4},
 };
 
 // Front half of the dense feed-forward block through FfnGateUpSilu, fused id or three launches.
@@ -187,6 +191,7 @@ int main(int argc, char** argv) {
   for (const Case& c : kCases) {
     ProjectState h;
     h.honour_reference_split = c.reference_split;
+    h.mxfp4_fp8_prefill = c.fp8_prefill;
     const auto a = Activations(c.m, c.k);
     const auto w = c.dtype == DType::Q4K   ? Q4KWeights(c.n, c.k)
                    : c.dtype == DType::Q5K ? Q5KWeights(c.n, c.k)
@@ -200,8 +205,8 @@ int main(int argc, char** argv) {
     } else if (c.dtype == DType::Q6K) {
       orc_gemm_q6k_ref(a.data(), w.data(), ref.data(), c.m, c.n, c.k, 1);
     } else {
-      std::vector<float> qdq = a, scale(c.m);               // QuantizeFp8Ref then GemmMxFp4Ref
-      orc_quantize_fp8_ref(qdq.data(), scale.data(), c.m, c.k);
+      std::vector<float> qdq = a, scale(c.m);               // QuantizeFp8Ref (m <= 16 or opted in) then GemmMxFp4Ref
+      if (c.m <= 16 || c.fp8_prefill) orc_quantize_fp8_ref(qdq.data(), scale.data(), c.m, c.k);
       orc_gemm_mxfp4_ref(qdq.data(), w.data(), w.data() + c.n * c.k / 2, ref.data(), c.m, c.n, c.k);
     }
     auto da = Upload(*backend, a);

@@ -46,6 +46,8 @@ def test_mxfp4_dequant_and_gemm():
     ref = a.astype(np.float64) @ d2.T
     bound = k * 2.0 ** -24 * (np.abs(a).astype(np.float64) @ np.abs(d2).T)
     assert np.all(np.abs(c - ref) <= bound)
+    # the threaded entry keeps every output's fma chain
+    assert np.array_equal(oracle.gemm_mxfp4(a, w2, 4, n, k, threads=True).view(np.uint32), c.view(np.uint32))
     with pytest.raises(oracle.OracleError) as err:     # k not a multiple of 32
         oracle.gemm_mxfp4(a[:, :48], w2[: n * 48 // 2 + n * 48 // 32], 4, n, 48)
     assert err.value.code == 1

@@ -117,8 +117,10 @@ const char* qmm_kernel_name(size_t index);
  * ignored: the library picks the launch shape from the scalars.  (The Vulkan backend
  * ignores block_* the same way, backend.hpp:50-55.)  Split-K ids
  * ("gemm_q4k_vec", "gemm_q4k_rows{2..5}", "gemm_mxfp4_wmma") honour the `split` scalar
- * of their contract: the sum over the `split` output regions equals the result, so the
- * reference's reduce pass ("gemm_vec_reduce", "gemm_mxfp4_wmma_reduce") still works.
+ * of their contract: the sum over the `split` output regions equals the result (real
+ * per-slice partial sums for one row of a large Q4_K matrix, else everything in region 0 and
+ * zeros in the others), so the reference's reduce pass ("gemm_vec_reduce",
+ * "gemm_mxfp4_wmma_reduce") still works.
  */
 qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
                       void* const* buffers, const size_t* buf_bytes, size_t nbuffers,

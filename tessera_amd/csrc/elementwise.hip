@@ -459,6 +459,40 @@ hipError_t launch_add(const float* a, const float* b, float* o, uint64_t n, hipS
   return hipGetLastError();
 }
 
+// Streaming read of `n16` 16-byte words, nothing else: the time a kernel that only has to fetch
+// that many bytes takes on this device, launch ramp and tail included (the measured ceiling the
+// GEMV kernels are compared with).  Each workgroup owns a contiguous range and every thread keeps
+// eight 16-byte loads in flight; the xor of all words goes to out[0] only if it equals a value
+// chosen so that the loads cannot be dropped.
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict__ p, size_t n16, uint32_t* out) {
+  constexpr int U = 8;
+  const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+  const size_t lo = static_cast<size_t>(blockIdx.x) * per, hi = lo + per < n16 ? lo + per : n16;
+  if (lo >= hi) return;
+  uint32_t acc = 0;
+  uint4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const size_t i = lo + threadIdx.x + static_cast<size_t>(u) * 256u;
+    v[u] = p[i < hi ? i : hi - 1];
+  }
+  for (size_t i = lo + threadIdx.x; i < hi; i += U * 256u) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+      const size_t nx = i + static_cast<size_t>(U + u) * 256u;
+      v[u] = p[nx < hi ? nx : hi - 1];
+    }
+  }
+  if (acc == 0x9E3779B9u) out[0] = acc;
+}
+
+hipError_t launch_read_probe(const void* src, uint32_t* out, uint64_t bytes, hipStream_t stream) {
+  hipLaunchKernelGGL(read_probe_kernel, dim3(2048), dim3(256), 0, stream, static_cast<const uint4*>(src),
+                     static_cast<size_t>(bytes / 16), out);
+  return hipGetLastError();
+}
+
 hipError_t launch_fill_i32(int32_t* out, int32_t value, uint64_t n, hipStream_t stream) {
   hipLaunchKernelGGL(fill_i32_kernel, grid_for(n, 256), dim3(256), 0, stream, out, value, n);
   return hipGetLastError();

@@ -421,12 +421,13 @@ struct Q4KPairCodec {
 // Gate and up projection of a dense feed-forward block in one pass, ending in
 // silu(G x) * (U x) (the dense analogue of the routed-expert gate/up pass above; the
 // reference runs two GEMVs and the "silu_mul" kernel, src/backends/rocm/rocm_kernels_basic.cpp:1882-1891).
-// The P rows a workgroup lays side by side are P/2 rows of the gate matrix interleaved with
-// the same P/2 rows of the up matrix (slot row p: matrix p & 1, row p / 2), so both dot
-// products of an output element are reduced in the same round and the thread that stores it
-// has both.  The activations are loaded once for the two matrices.
+// The two matrices share the skeleton's two pipeline stages: stage 0 holds the group's rows of
+// the gate matrix, stage 1 the same rows of the up matrix, so both dot products of an output
+// element are reduced in the same round and the thread that stores it has both, while the group
+// shape (rows side by side, wavefronts per workgroup) stays the single-matrix one.  The
+// activations are loaded once for the two matrices.
 struct Q4KGateUpCodec : Q4KPairCodec {
-  static constexpr bool kPairRows = true;
+  static constexpr bool kPairStages = true;
   struct Args {
     const float* a;
     const uint8_t* w;      // gate
@@ -438,27 +439,65 @@ struct Q4KGateUpCodec : Q4KPairCodec {
                                                 const Src& src) {
     Q4KPairCodec::load_x<R>(Q4KPairCodec::Args{p.a, p.w, p.k}, chunk, valid, x, src);
   }
-  // Bit 0 of off0 (offsets are multiples of 16) carries the matrix of this lane's slot row.
-  static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
-                                                   uint32_t prow) {
-    const uint32_t hdr = (prow >> 1) * (cpr >> 2) * 144u + (chunk >> 2) * 144u;
-    return Lane{hdr | (prow & 1u), hdr + 16u + (chunk & 3u) * 32u};
+  static __device__ __forceinline__ Lane make_lane(const Args& p, uint32_t cpr, uint32_t chunk, uint32_t prow) {
+    return Q4KPairCodec::make_lane(Q4KPairCodec::Args{p.a, p.w, p.k}, cpr, chunk, prow);
   }
   static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
-                                              uint32_t cpr, Frag& f) {
-    const uint8_t* base = ((ln.off0 & 1u) ? p.up : p.w) + static_cast<size_t>(row) * ((cpr >> 2) * 144u);
-    f.h = load_u4(base + (ln.off0 & ~1u));
+                                              uint32_t cpr, Frag& f, int stage) {
+    const uint8_t* base = (stage ? p.up : p.w) + static_cast<size_t>(row) * ((cpr >> 2) * 144u);
+    f.h = load_u4(base + ln.off0);
     f.q0 = load_u4(base + ln.off1);
     f.q1 = load_u4(base + ln.off1 + 16u);
   }
   static __device__ __forceinline__ float combine(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
 };
 
-// Whether a codec interleaves two matrices over the slot rows of a group (see Q4KGateUpCodec).
+// Whether a codec spreads two matrices over the two pipeline stages (see Q4KGateUpCodec).
 template <class Codec, class = void>
-struct pair_rows : std::false_type {};
+struct pair_stages : std::false_type {};
 template <class Codec>
-struct pair_rows<Codec, std::void_t<decltype(Codec::kPairRows)>> : std::bool_constant<Codec::kPairRows> {};
+struct pair_stages<Codec, std::void_t<decltype(Codec::kPairStages)>> : std::bool_constant<Codec::kPairStages> {};
+
+// Q4_K, single activation row, K cut into `gridDim.y` slices: workgroups of slice s take columns
+// [s*k, (s+1)*k) of every weight row (k = the slice length) and write their partial dot products
+// to output region s, so a workgroup stages only its slice of the activations and the caller's
+// reduce over the regions ("gemm_vec_reduce", src/core/decode_internal.hpp:840-923) finishes the sum.
+struct Q4KSliceCodec : Q4KPairCodec {
+  static constexpr bool kSlices = true;
+  struct Args {
+    const float* a;
+    const uint8_t* w;
+    uint32_t k;           // slice length
+    uint32_t row_bytes;   // bytes of a whole weight row
+  };
+  static __device__ __forceinline__ void select_slice(Args& p, uint32_t slice) {
+    p.a += static_cast<size_t>(slice) * p.k;
+    p.w += static_cast<size_t>(slice) * (p.k / 256u) * 144u;
+  }
+  template <int R, class Src>
+  static __device__ __forceinline__ void load_x(const Args& p, uint32_t chunk, bool valid, X<R>& x,
+                                                const Src& src) {
+    Q4KPairCodec::load_x<R>(Q4KPairCodec::Args{p.a, p.w, p.k}, chunk, valid, x, src);
+  }
+  static __device__ __forceinline__ Lane make_lane(const Args& p, uint32_t, uint32_t chunk, uint32_t prow) {
+    const uint32_t hdr = prow * p.row_bytes + (chunk >> 2) * 144u;
+    return Lane{hdr, hdr + 16u + (chunk & 3u) * 32u};
+  }
+  static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row, uint32_t, Frag& f) {
+    const uint8_t* base = p.w + static_cast<size_t>(row) * p.row_bytes;
+    f.h = load_u4(base + ln.off0);
+    f.q0 = load_u4(base + ln.off1);
+    f.q1 = load_u4(base + ln.off1 + 16u);
+  }
+  template <int R>
+  static __device__ __forceinline__ float finish(const Args&, uint32_t, int, float v) {
+    return v;
+  }
+};
+template <class Codec, class = void>
+struct k_slices : std::false_type {};
+template <class Codec>
+struct k_slices<Codec, std::void_t<decltype(Codec::kSlices)>> : std::bool_constant<Codec::kSlices> {};
 
 // ----------------------------------------------------------------------------
 // Q5_K: 176-byte super-block = fp16 d, fp16 dmin, 12 bytes of 6-bit scales/mins (packed as in
@@ -1139,6 +1178,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   __shared__ float red[2][D][P][R][LR ? 1 : kMaxWaves];
   __shared__ float part[2][D][R][LR ? MAXT : 1];
 
+  if constexpr (k_slices<Codec>::value) {     // blockIdx.y = K slice and output region
+    Codec::select_slice(args, blockIdx.y);
+    c += static_cast<size_t>(blockIdx.y) * R * ldc;
+  }
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t slots = P * cpr;
@@ -1161,22 +1204,28 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // last group for the loads (a prefetch must not pull the next workgroup's rows, which would
   // come from HBM a second time through another XCD's L2) and dropped at the store; rows past
   // n inside the last group re-read the group's first row.
-  // PR = output rows per group; a paired codec spends two slot rows (one per matrix) on each.
-  constexpr bool kPaired = pair_rows<Codec>::value;
-  constexpr uint32_t PR = kPaired ? P / 2 : P;
-  static_assert(!kPaired || P % 2 == 0, "a paired codec needs an even number of slot rows");
+  // A paired codec gives the two stages of the pipeline to its two matrices: a round then
+  // covers one group (both matrices) instead of D groups.
+  constexpr bool kPaired = pair_stages<Codec>::value;
+  static_assert(!kPaired || D == 2, "a paired codec uses exactly two stages");
+  constexpr uint32_t PR = P;
+  constexpr uint32_t kGroupsPerRound = kPaired ? 1u : static_cast<uint32_t>(D);
   const uint32_t groups = (n + PR - 1) / PR;
   const uint32_t g0 = blockIdx.x * groups_per_wg;
   const uint32_t g1 = g0 + groups_per_wg < groups ? g0 + groups_per_wg : groups;
   const Lane ln = Codec::make_lane(args, cpr, chunk, prow);
-  const uint32_t prow_out = kPaired ? prow >> 1 : prow;      // output row inside the group
-  const uint32_t prow_first = kPaired ? prow & 1u : 0u;      // slot row of the group's first row, same matrix
-  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, (groups - 1u) * PR + prow_out < n ? prow : prow_first);
+  const Lane ln_tail = Codec::make_lane(args, cpr, chunk, (groups - 1u) * PR + prow < n ? prow : 0u);
   const bool ragged = n % PR != 0;
-  auto fetch = [&](uint32_t grp, typename Codec::Frag& f) {
+  // Stage d of the round that starts at group `gbase`: group gbase + d, or matrix d of gbase.
+  auto fetch = [&](uint32_t gbase, int d, typename Codec::Frag& f) {
+    uint32_t grp = kPaired ? gbase : gbase + static_cast<uint32_t>(d);
     grp = grp < g1 ? grp : g1 - 1u;
     const bool tail = ragged && grp == groups - 1u;
-    Codec::load(args, tail ? ln_tail : ln, grp * PR, cpr, f);
+    if constexpr (kPaired) {
+      Codec::load(args, tail ? ln_tail : ln, grp * PR, cpr, f, d);
+    } else {
+      Codec::load(args, tail ? ln_tail : ln, grp * PR, cpr, f);
+    }
   };
 
   typename Codec::Frag frag[D];
@@ -1203,7 +1252,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
         const uint32_t e = (t + i * blockDim.x) * 4u;
         xr[i] = *reinterpret_cast<const float4*>(args.a + (e < k ? e : k - 4u));
       }
-      fetch(g0, frag[0]);
+      fetch(g0, 0, frag[0]);
 #pragma unroll
       for (int i = 0; i < kXPer; ++i) {
         const uint32_t e = (t + i * blockDim.x) * 4u;
@@ -1211,12 +1260,12 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       }
       lds_barrier();
 #pragma unroll
-      for (int d = 1; d < D; ++d) fetch(g0 + d, frag[d]);
+      for (int d = 1; d < D; ++d) fetch(g0, d, frag[d]);
       Codec::template load_x<R>(args, chunk, valid, x, StagedX{xs, 0u, kStride});
     } else {
       // Weight loads first, activations second: both are in flight before anything waits.
 #pragma unroll
-      for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
+      for (int d = 0; d < D; ++d) fetch(g0, d, frag[d]);
       for (uint32_t base = 0; base < k; base += kPiece) {
         const uint32_t len = k - base < kPiece ? k - base : kPiece;
         if (base != 0) lds_barrier();  // the previous piece has been read
@@ -1235,7 +1284,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
     }
   } else {
 #pragma unroll
-    for (int d = 0; d < D; ++d) fetch(g0 + d, frag[d]);
+    for (int d = 0; d < D; ++d) fetch(g0, d, frag[d]);
     Codec::template load_x<R>(args, chunk, valid, x, 0);
   }
 
@@ -1247,10 +1296,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   auto round_wave = [&](uint32_t g, auto refill) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      if (!decltype(refill)::value && g + d >= g1) break;
+      if (!kPaired && !decltype(refill)::value && g + d >= g1) break;
       float v[R];
       Codec::template dot<R>(frag[d], x, v);
-      if constexpr (decltype(refill)::value) fetch(g + D + d, frag[d]);
+      if constexpr (decltype(refill)::value) fetch(g + kGroupsPerRound, d, frag[d]);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (two) {
@@ -1267,20 +1316,20 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       }
     }
     lds_barrier();  // LDS only: the prefetched global loads stay in flight across it
-    if (t < D * PR * R) {
+    if (t < kGroupsPerRound * PR * R) {
       const uint32_t d = t / (PR * R), po = (t / R) % PR, r = t % R;
       const uint32_t row = (g + d) * PR + po;
       if (g + d < g1 && row < n) {
-        auto slot_sum = [&](uint32_t p) {
-          const uint32_t w_lo = (p * cpr) >> 6, w_hi = ((p + 1u) * cpr - 1u) >> 6;
+        auto slot_sum = [&](uint32_t stage) {
+          const uint32_t w_lo = (po * cpr) >> 6, w_hi = ((po + 1u) * cpr - 1u) >> 6;
           float sum = 0.0f;
-          for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][d][p][r][w];
+          for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][stage][po][r][w];
           return sum;
         };
         if constexpr (kPaired) {
-          c[static_cast<size_t>(r) * ldc + row] = Codec::combine(slot_sum(2u * po), slot_sum(2u * po + 1u));
+          c[static_cast<size_t>(r) * ldc + row] = Codec::combine(slot_sum(0u), slot_sum(1u));
         } else {
-          c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, slot_sum(po));
+          c[static_cast<size_t>(r) * ldc + row] = Codec::template finish<R>(args, row, r, slot_sum(d));
         }
       }
     }
@@ -1290,21 +1339,21 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   auto round_lds = [&](uint32_t g, auto refill) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      if (!decltype(refill)::value && g + d >= g1) break;
+      if (!kPaired && !decltype(refill)::value && g + d >= g1) break;
       float v[R];
       Codec::template dot<R>(frag[d], x, v);
-      if constexpr (decltype(refill)::value) fetch(g + D + d, frag[d]);
+      if constexpr (decltype(refill)::value) fetch(g + kGroupsPerRound, d, frag[d]);
       // Selected, never multiplied by a 0/1 mask (see to_a above).
 #pragma unroll
       for (int r = 0; r < R; ++r) part[buf][d][r][t] = valid ? v[r] : 0.0f;
     }
     lds_barrier();  // LDS only: the prefetched global loads stay in flight across it
-    for (uint32_t o = t >> 4; o < D * PR * R; o += blockDim.x >> 4) {
+    for (uint32_t o = t >> 4; o < kGroupsPerRound * PR * R; o += blockDim.x >> 4) {
       const uint32_t d = o / (PR * R), po = (o / R) % PR, r = o % R;
       const uint32_t row = (g + d) * PR + po;
       const bool live = g + d < g1 && row < n;
-      auto slot_sum = [&](uint32_t p) {
-        const float* src = &part[buf][d][r][p * cpr];
+      auto slot_sum = [&](uint32_t stage) {
+        const float* src = &part[buf][stage][r][po * cpr];
         float sum = 0.0f;
         if (live) {
           for (uint32_t i = t & 15u; i < cpr; i += 16u) sum += src[i];
@@ -1313,10 +1362,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       };
       float res;
       if constexpr (kPaired) {
-        const float first = slot_sum(2u * po), second = slot_sum(2u * po + 1u);
+        const float first = slot_sum(0u), second = slot_sum(1u);
         res = Codec::combine(first, second);
       } else {
-        res = Codec::template finish<R>(args, live ? row : 0u, r, slot_sum(po));
+        res = Codec::template finish<R>(args, live ? row : 0u, r, slot_sum(d));
       }
       if (live && (t & 15u) == 0u) c[static_cast<size_t>(r) * ldc + row] = res;
     }
@@ -1327,7 +1376,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   };
 
   uint32_t g = g0;
-  for (; g + D < g1; g += D) round(g, std::true_type{});
+  for (; g + kGroupsPerRound < g1; g += kGroupsPerRound) round(g, std::true_type{});
   if (g < g1) round(g, std::false_type{});
 }
 
@@ -1394,20 +1443,8 @@ int g_num_cus = 256;
 // to whole wavefronts; picks the P that idles the fewest lanes, larger P on ties
 // (fewer, fuller workgroups share one copy of the activations).
 template <uint32_t kMaxP>
-GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads, bool even_p = false) {
+GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads) {
   GemvPlan g{cpr, 0, 1, false};
-  if (even_p) {
-    // paired codecs: the largest even P that fits, preferring full wavefronts
-    if (cpr < 64) return g;   // p stays 1: the caller rejects it
-    double best = 0.0;
-    for (uint32_t p = 2; p <= kMaxP; p += 2) {
-      const uint32_t t = (p * cpr + 63u) / 64u * 64u;
-      if (t > max_threads) break;
-      const double fill = static_cast<double>(p * cpr) / t;
-      if (fill >= best) best = fill, g.p = p, g.threads = t;
-    }
-    return g;
-  }
   if (cpr == 4 || cpr == 8 || cpr == 16 || cpr == 32) {
     g.smallk = true;
     g.threads = 256;
@@ -1436,21 +1473,20 @@ GemvPlan plan_gemv(uint32_t cpr, uint32_t max_threads, bool even_p = false) {
 // to fuller wavefronts, then to larger P.  At 17408x5120 Q4_K this picks 9 rows (12 wavefronts,
 // 8 stages) over 8 rows (10 wavefronts, 9 stages).
 template <uint32_t kMaxP>
-GemvPlan plan_gemv_balanced(uint32_t cpr, uint32_t max_threads, uint32_t n, bool even_p) {
+GemvPlan plan_gemv_balanced(uint32_t cpr, uint32_t max_threads, uint32_t n) {
   GemvPlan g{cpr, (cpr + 63u) / 64u * 64u, 1, false};
   const uint32_t waves_per_simd = (max_threads / 64u + 3u) / 4u;
   const uint32_t cus = static_cast<uint32_t>(g_num_cus);
   uint64_t best_cost = ~0ull;
   uint32_t best_rank = 0;
   double best_fill = 0.0;
-  for (uint32_t p = even_p ? 2u : 1u; p <= kMaxP; p += even_p ? 2u : 1u) {
+  for (uint32_t p = 1u; p <= kMaxP; ++p) {
     const uint32_t t = (p * cpr + 63u) / 64u * 64u;
     if (t > max_threads) break;
     const uint32_t w = t / 64u;
     uint32_t per_cu = (4u * waves_per_simd) / w;
     if (per_cu == 0) per_cu = 1;
-    const uint32_t pr = even_p ? p / 2u : p;
-    const uint32_t groups = (n + pr - 1u) / pr;
+    const uint32_t groups = (n + p - 1u) / p;
     uint32_t grid = cus * per_cu;
     if (grid > groups) grid = groups;
     const uint32_t per_wg = (groups + grid - 1u) / grid;
@@ -1481,16 +1517,17 @@ struct balance_simds<Codec, std::void_t<decltype(Codec::kBalanceSimds)>> : std::
 
 template <class Codec, int R, int MAXT, int D, uint32_t P>
 hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n, uint32_t cpr,
-                         uint32_t ldc, uint32_t threads, hipStream_t stream) {
+                         uint32_t ldc, uint32_t threads, hipStream_t stream, uint32_t slices = 1) {
   // Resident workgroups per CU under __launch_bounds__(MAXT): the register budget
   // admits ceil(MAXT/256) wavefronts per SIMD whatever the block size.
   const uint32_t waves = threads / 64u;
   const uint32_t waves_per_simd = (MAXT / 64u + 3u) / 4u;
   uint32_t per_cu = (4u * waves_per_simd) / waves;
   if (per_cu == 0) per_cu = 1;
-  constexpr uint32_t PR = pair_rows<Codec>::value ? P / 2 : P;
+  constexpr uint32_t PR = P;
   const uint32_t groups = (n + PR - 1) / PR;
-  uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu;
+  uint32_t grid = static_cast<uint32_t>(g_num_cus) * per_cu / slices;     // workgroups per K slice
+  if (grid == 0) grid = 1;
   if (grid > groups) grid = groups;
   uint32_t per_wg = (groups + grid - 1) / grid;
   grid = (groups + per_wg - 1) / per_wg;
@@ -1500,36 +1537,37 @@ hipError_t launch_gemv_p(const typename Codec::Args& args, float* c, uint32_t n,
   constexpr uint32_t kSmall = R == 1 ? 8192u : (R == 2 ? 4096u : 2048u);
   if constexpr (R == 1 && Codec::kStageX) {
     if (args.k > kSmall && args.k <= 32768u && per_cu == 1) {
-      hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, 32768u>), dim3(grid), dim3(threads), 0,
+      hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, 32768u>), dim3(grid, slices), dim3(threads), 0,
                          stream, args, c, n, cpr, ldc, per_wg);
       return hipGetLastError();
     }
   }
   if (cpr < 64u) {
-    hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall, true>), dim3(grid), dim3(threads), 0,
+    hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall, true>), dim3(grid, slices), dim3(threads), 0,
                        stream, args, c, n, cpr, ldc, per_wg);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall>), dim3(grid), dim3(threads), 0, stream,
+  hipLaunchKernelGGL((gemv_kernel<Codec, R, P, D, MAXT, kSmall>), dim3(grid, slices), dim3(threads), 0, stream,
                      args, c, n, cpr, ldc, per_wg);
   return hipGetLastError();
 }
 
 template <class Codec, int R, int MAXT, int D, uint32_t kMaxP = 2>
 hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n, uint32_t k,
-                         uint32_t ldc, hipStream_t stream) {
+                         uint32_t ldc, hipStream_t stream, uint32_t slices = 1) {
   const uint32_t cpr = Codec::chunks_per_row(k);
-  GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT, pair_rows<Codec>::value);
+  GemvPlan g = plan_gemv<kMaxP>(cpr, MAXT);
   // Rows shorter than a wavefront (and not of the small-K kernel's lengths) also go side by
   // side in a workgroup: plan_gemv would give each a workgroup of one partly idle wavefront.
   // Several activation rows make every codec's loop arithmetic-bound (a multiply-add per weight
   // and row), so those are planned by SIMD load as well: MXFP4 with four fp32 rows went from 2
   // rows a workgroup (5 wavefronts: 2,1,1,1 on the SIMDs) to 3 (8 wavefronts), 42.5 -> 32.4 us.
   if (!g.smallk && ((balance_simds<Codec>::value && R == 1) || cpr < 64u || R > 1)) {
-    g = plan_gemv_balanced<kMaxP>(cpr, MAXT, n, pair_rows<Codec>::value);
+    g = plan_gemv_balanced<kMaxP>(cpr, MAXT, n * slices);
   }
-  if (pair_rows<Codec>::value && (g.p % 2u != 0 || g.smallk)) return hipErrorInvalidValue;
-  if constexpr (!pair_rows<Codec>::value) {
+  if (slices > 1 && g.smallk) return hipErrorInvalidValue;
+  if (pair_stages<Codec>::value && g.smallk) return hipErrorInvalidValue;
+  if constexpr (!pair_stages<Codec>::value) {
     if (g.smallk) {
       constexpr int U = D > 4 ? 4 : D;
       const uint32_t rows_per_wave = 64u / cpr;
@@ -1546,8 +1584,8 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
   switch (g.p) {
 #define QMM_GEMV_CASE(PP)                                                                       \
   case PP:                                                                                      \
-    if constexpr (kMaxP >= PP && (!pair_rows<Codec>::value || PP % 2 == 0))                     \
-      return launch_gemv_p<Codec, R, MAXT, D, PP>(args, c, n, cpr, ldc, g.threads, stream);     \
+    if constexpr (kMaxP >= PP)                                                                  \
+      return launch_gemv_p<Codec, R, MAXT, D, PP>(args, c, n, cpr, ldc, g.threads, stream, slices); \
     break;
     QMM_GEMV_CASE(1) QMM_GEMV_CASE(2) QMM_GEMV_CASE(3) QMM_GEMV_CASE(4) QMM_GEMV_CASE(5) QMM_GEMV_CASE(6)
     QMM_GEMV_CASE(7) QMM_GEMV_CASE(8) QMM_GEMV_CASE(9) QMM_GEMV_CASE(10) QMM_GEMV_CASE(11) QMM_GEMV_CASE(12)
@@ -1663,6 +1701,21 @@ hipError_t launch_q4k_gemv(const float* a, const uint8_t* w, float* c, uint32_t 
   return hipSuccess;
 }
 
+// One activation row with K cut into `split` slices, partial sums to `split` output regions of n
+// floats: slices of 64 to 512 chunks (4096..32768 weights) on matrices large enough to fill the chip.
+bool q4k_gemv_split_supported(uint64_t n, uint64_t k, uint64_t split) {
+  if (split < 2 || split > 8 || k % (256 * split) != 0) return false;
+  const uint64_t slice = k / split;
+  return slice >= 4096 && slice <= 32768 && n * k >= (1ull << 24) && n <= 0xFFFFFFFFull / split;
+}
+
+hipError_t launch_q4k_gemv_split(const float* a, const uint8_t* w, float* c, uint32_t n, uint32_t k, uint32_t split,
+                                 hipStream_t stream) {
+  const uint32_t slice = k / split;
+  Q4KSliceCodec::Args args{a, w, slice, (k / 256u) * 144u};
+  return launch_gemv_r<Q4KSliceCodec, 1, 768, 2, 12>(args, c, n, slice, n, stream, split);
+}
+
 // silu(G x) * (U x) for one activation row, one launch: a row of 64 to 384 chunks of 64 weights
 // (two slot rows of it must fit a 768-thread workgroup and a wavefront may span two rows at most).
 bool ffn_gate_up_q4k_supported(uint64_t k) { return k % 256 == 0 && k >= 4096 && k <= 24576; }
@@ -1670,7 +1723,7 @@ bool ffn_gate_up_q4k_supported(uint64_t k) { return k % 256 == 0 && k >= 4096 &&
 hipError_t launch_ffn_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up, float* out,
                                   uint32_t n, uint32_t k, hipStream_t stream) {
   Q4KGateUpCodec::Args args{x, gate, k, up};
-  return launch_gemv_r<Q4KGateUpCodec, 1, 768, 2, 8>(args, out, n, k, n, stream);
+  return launch_gemv_r<Q4KGateUpCodec, 1, 768, 2, 9>(args, out, n, k, n, stream);
 }
 
 // Q5_K: one row per weight pass (a lane keeps 64 activations and five 16-byte loads per stage).

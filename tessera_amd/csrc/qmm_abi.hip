@@ -197,8 +197,9 @@ qmm_status run_gemm_q4k(const LaunchCtx& c) {
 
 // "gemm_q4k_vec" and "gemm_q4k_rows{R}": buffers A, W, C; scalars m, n, k, split
 // (src/backends/rocm/rocm_kernels_gemv.cpp:17-24,103-156).  C has `split` regions of
-// m*n floats whose sum is the result: region 0 receives the whole dot product and
-// regions 1..split-1 are zeroed, so "gemm_vec_reduce" over them yields the result.
+// m*n floats whose sum is the result: either every region receives the partial sums of its K
+// slice (one row, slices of 4096 weights or more), or region 0 receives the whole dot product and
+// regions 1..split-1 are zeroed; "gemm_vec_reduce" over them yields the result either way.
 qmm_status run_gemm_q4k_split(const LaunchCtx& c, uint64_t rows_required) {
   if (!counts(c, 3, 4)) return bad("gemm_q4k_vec/rows: expects 3 buffers and 4 scalars");
   const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], split = c.sc[3];
@@ -210,6 +211,12 @@ qmm_status run_gemm_q4k_split(const LaunchCtx& c, uint64_t rows_required) {
     return bad("gemm_q4k_vec/rows: a buffer is smaller than m, n, k, split require");
   }
   float* out = c.ptr<float>(2);
+  // One row of a large matrix with long enough slices: real partial sums, one region per slice,
+  // each workgroup staging only its slice of the activations.
+  if (m == 1 && n <= 0xFFFFFFFFull && k <= 0xFFFFFFFFull && qmm::q4k_gemv_split_supported(n, k, split)) {
+    return map_hip(qmm::launch_q4k_gemv_split(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, static_cast<uint32_t>(n),
+                                              static_cast<uint32_t>(k), static_cast<uint32_t>(split), c.stream));
+  }
   qmm_status st = q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, m, n, k);
   if (st == QMM_OK && split > 1) {
     st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
@@ -252,6 +259,15 @@ qmm_status run_add(const LaunchCtx& c) {
   const u128 bytes = static_cast<u128>(n) * 4;
   if (!c.fits(0, bytes) || !c.fits(1, bytes) || !c.fits(2, bytes)) return bad("add: a buffer is smaller than n requires");
   return map_hip(qmm::launch_add(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<float>(2), n, c.stream));
+}
+
+// "read_probe" (not a reference id; a measuring aid): buffers Src, Out (at least 4 bytes, left
+// untouched); scalar bytes (a multiple of 16).  Reads Src once and does nothing else.
+qmm_status run_read_probe(const LaunchCtx& c) {
+  if (!counts(c, 2, 1)) return bad("read_probe: expects 2 buffers and 1 scalar");
+  const uint64_t bytes = c.sc[0];
+  if (bytes == 0 || bytes % 16 != 0 || !c.fits(0, bytes) || !c.fits(1, 4)) return bad("read_probe: bytes must be a non-zero multiple of 16 within the buffer");
+  return map_hip(qmm::launch_read_probe(c.ptr<const void>(0), c.ptr<uint32_t>(1), bytes, c.stream));
 }
 
 // "fill": buffer 0 is an int32 array; scalars value, count (include/tessera/backend.hpp:151-152,393-396).
@@ -833,6 +849,7 @@ const Entry kTable[] = {
     {"silu_mul", run_silu_mul},
     {"add", run_add},
     {"fill", run_fill},
+    {"read_probe", run_read_probe},
     {"rmsnorm", run_rmsnorm},
     {"embedding_f32", run_embedding_f32},
     {"embedding_bf16", run_embedding_bf16},

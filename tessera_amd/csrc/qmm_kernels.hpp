@@ -109,12 +109,19 @@ hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64
 hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream);
 hipError_t launch_add(const float* a, const float* b, float* o, uint64_t n, hipStream_t stream);
 hipError_t launch_fill_i32(int32_t* out, int32_t value, uint64_t n, hipStream_t stream);
+hipError_t launch_read_probe(const void* src, uint32_t* out, uint64_t bytes, hipStream_t stream);
 hipError_t launch_rmsnorm(const float* x, const float* w, float* y, uint64_t rows, uint64_t cols, float eps,
                           hipStream_t stream);
 hipError_t launch_embedding(int kind, const uint32_t* ids, const void* table, float* out, uint64_t rows,
                             uint64_t cols, uint64_t vocab, hipStream_t stream);
 hipError_t launch_silu_mul(const float* g, const float* u, float* o, uint64_t n, hipStream_t stream);
 hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
+
+// Q4_K, one activation row, K cut into `split` slices whose partial sums go to `split` output
+// regions of n floats (the caller's reduce adds them).
+bool q4k_gemv_split_supported(uint64_t n, uint64_t k, uint64_t split);
+hipError_t launch_q4k_gemv_split(const float* a, const uint8_t* w, float* c, uint32_t n, uint32_t k, uint32_t split,
+                                 hipStream_t stream);
 
 // Dense feed-forward gate and up projections with the activation fused, one activation row:
 // out[j] = silu(G x)[j] * (U x)[j], both matrices n rows of Q4_K.

@@ -182,6 +182,35 @@ def test_vec_split_contract_and_reduce(backend, n, k, split):
     assert np.array_equal(parts.sum(axis=0, dtype=np.float32), got)
 
 
+@pytest.mark.parametrize("n,k,split", [(5120, 17408, 4), (2001, 16384, 2), (1031, 32768, 8), (4099, 8192, 2), (5120, 17408, 2)])
+def test_vec_split_regions_hold_partial_sums(backend, n, k, split):
+    """One row of a large matrix with slices of 4096 weights or more (the down projection as the
+    reference's caller issues it: GemmVecSplit(5120, 17408) = 4, src/core/decode_internal.hpp:840-885):
+    region s holds the dot products over K slice s, each within the GEMV bound of the oracle's
+    product over that slice, and gemm_vec_reduce returns their ordered sum."""
+    g = synth.rng(3 * n + k + split)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, 1, k)
+    ref = oracle.gemm_q4k(a, w, 1, n, k, threads=True)
+    da, dw = backend.Upload(a), backend.Upload(w)
+    part = backend.AllocateBuffer(4 * n * split)
+    backend.CopyH2D(part, np.full(n * split, np.nan, np.float32))
+    out = backend.AllocateBuffer(4 * n)
+    run(backend, "gemm_q4k_vec", [da, dw, part], [1, n, k, split], grid=((n + 7) // 8, split, 1))
+    run(backend, "gemm_vec_reduce", [part, out], [n, split], grid=((n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(out, dtype=np.float32)
+    parts = backend.CopyD2H(part, dtype=np.float32).reshape(split, n)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    assert np.array_equal(parts.sum(axis=0, dtype=np.float32), got)
+    blocks = w.reshape(n, k // 256, 144)
+    per = k // 256 // split
+    for s_ in range(split):
+        ws = np.ascontiguousarray(blocks[:, s_ * per:(s_ + 1) * per]).reshape(-1)
+        ref_s = oracle.gemm_q4k(a[:, s_ * per * 256:(s_ + 1) * per * 256], ws, 1, n, per * 256, threads=True)
+        assert rel_err(parts[s_], ref_s) <= TOL, (s_, rel_err(parts[s_], ref_s))
+
+
 @pytest.mark.parametrize("rows", [2, 3, 4, 5])
 def test_rows_kernels(backend, rows):
     g = synth.rng(rows)

@@ -44,6 +44,7 @@ def _load() -> C.CDLL:
         "orc_e8m0_to_float": (C.c_float, [C.c_uint8]),
         "orc_f4e2m1_to_float": (C.c_float, [C.c_uint8]),
         "orc_fp32_to_fp8_e4m3": (C.c_uint8, [C.c_float]),
+        "orc_fp32_to_fp8_e4m3_many": (None, [f32p, u8p, sz]),
         "orc_get_scale_min": (None, [sz, u8p, u8p, u8p]),
         "orc_dequantize_q4k": (None, [u8p, f32p]),
         "orc_dequantize_q4k_rows": (None, [u8p, f32p, sz]),
@@ -272,6 +273,14 @@ def quantize_fp8(data, rows: int, cols: int) -> tuple[np.ndarray, np.ndarray]:
     scale = np.empty(rows, dtype=np.float32)
     _check(_lib.orc_quantize_fp8_ref(_p(out, C.c_float), _p(scale, C.c_float), rows, cols))
     return out, scale
+
+
+def fp32_to_fp8_e4m3_many(v) -> np.ndarray:
+    """The encoder of fp32_to_fp8_e4m3 over an array (threaded)."""
+    v = _f32(v).reshape(-1)
+    out = np.empty(v.size, dtype=np.uint8)
+    _lib.orc_fp32_to_fp8_e4m3_many(_p(v, C.c_float), _p(out, C.c_uint8), v.size)
+    return out
 
 
 def quantize_fp8_pack(data, rows: int, cols: int) -> tuple[np.ndarray, np.ndarray]:

@@ -277,6 +277,12 @@ void orc_quantize_q4k(const float* x, uint8_t* blk) {
   }
 }
 
+/* orc_fp32_to_fp8_e4m3 over an array, spread over OpenMP threads (for sweeps over all inputs). */
+void orc_fp32_to_fp8_e4m3_many(const float* v, uint8_t* out, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (long long i = 0; i < (long long)n; ++i) out[i] = orc_fp32_to_fp8_e4m3(v[i]);
+}
+
 /* ---- per-row dynamic E4M3 quantize-dequantize in place (quant.cpp:180-205) ---- */
 int orc_quantize_fp8_ref(float* data, float* scale, size_t rows, size_t cols) {
   if (rows == 0 || cols == 0) return ORC_INVALID_ARGUMENT;

@@ -166,6 +166,38 @@ def test_quantize_fp8_encoder_sweep_bit_exact(backend):
     assert np.array_equal(backend.CopyD2H(dq).reshape(1, cols), codes)
 
 
+def test_quantize_fp8_encoder_every_input(backend):
+    """Every fp32 bit pattern the encoder can be handed under a unit row scale -- all 2 x 1 138 753 537
+    values with |x| <= 448, zeros and subnormals included -- through quantize_fp8_pack on the
+    device against the oracle's Fp32ToFp8E4M3Bits restatement (src/core/numerics/quant.hpp:564-565
+    states its contract), in chunks of 2^24 patterns laid out as 4096 rows that each also hold a
+    448, so that every row's scale is exactly 1.  Larger magnitudes never reach the encoder: the
+    id clamps to +-448 first (covered by the QDQ tests below).  Stops at the first mismatch."""
+    top = int(np.float32(448.0).view(np.uint32))          # 0x43E00000
+    rows, per_row = 4096, 4096
+    chunk = rows * per_row
+    pad = np.full((rows, 4), 448.0, np.float32)
+    dx = backend.AllocateBuffer(4 * rows * (per_row + 4))
+    dq, ds = backend.AllocateBuffer(rows * (per_row + 4)), backend.AllocateBuffer(4 * rows)
+    checked = 0
+    for sign in (0, 0x80000000):
+        for base in range(0, top + 1, chunk):
+            bits = np.arange(base, base + chunk, dtype=np.uint64)
+            bits = np.minimum(bits, top).astype(np.uint32) | np.uint32(sign)     # the last chunk repeats 448
+            x = np.concatenate([bits.view(np.float32).reshape(rows, per_row), pad], axis=1)
+            backend.CopyH2D(dx, x)
+            run(backend, "quantize_fp8_pack", [dx, dq, ds], [rows, per_row + 4])
+            backend.Synchronize()
+            got = backend.CopyD2H(dq).reshape(rows, per_row + 4)
+            assert np.all(backend.CopyD2H(ds, dtype=np.float32) == 1.0)
+            want = oracle.fp32_to_fp8_e4m3_many(x).reshape(rows, per_row + 4)
+            if not np.array_equal(got, want):
+                r, c = np.argwhere(got != want)[0]
+                raise AssertionError(f"input bits {int(x[r, c].view(np.uint32)):#010x}: device {got[r, c]:#04x}, oracle {want[r, c]:#04x}")
+            checked += chunk
+    assert checked >= 2 * (top + 1)
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 5120), (16, 5120), (3, 100), (4, 17408)])
 def test_quantize_fp8_qdq_bit_exact(backend, rows, cols):
     g = synth.rng(rows * 17 + cols)

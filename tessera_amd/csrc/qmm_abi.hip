@@ -150,11 +150,23 @@ void* decode_scratch(const LaunchCtx& c) {
 constexpr uint64_t kQ4KGemmMinRows = 17;
 constexpr uint64_t kMxfp4GemmMinRows = 17;   // below: the VALU GEMV passes, exact fp32 order
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
+constexpr uint64_t kQ4KRows16MinRows = 3;      // from here the 16x16x32 kernel, below the 4x4x4 one
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 
 qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
                       uint64_t k) {
   const hipStream_t s = ctx.stream;
+  // 3..16 rows of a large matrix: one pass over the weights on the 16x16x32 MFMA.
+  if (m >= kQ4KRows16MinRows && m < kQ4KGemmMinRows && n * k >= kQ4KFewRowsMinWeights && qmm::gemv_q4k_rows16_supported(m, n, k) &&
+      qmm::gemv_q4k_rows16_workspace_bytes(m, n, k) <= kDecodeScratchBytes) {
+    void* ws = decode_scratch(ctx);
+    if (ws == nullptr) {
+      g_last_error = "Q4_K: decode scratch missing";
+      return QMM_DEVICE_ERROR;
+    }
+    return map_hip(qmm::launch_q4k_rows16(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                          static_cast<uint32_t>(k), s));
+  }
   if (m >= 2 && m < kQ4KGemmMinRows && n * k >= kQ4KFewRowsMinWeights && k <= kQ4KFewRowsMaxK &&
       qmm::gemv_q4k_mfma_supported(1, n, k)) {
     void* ws = decode_scratch(ctx);   // fixed address: a recorded decode step stays valid
@@ -353,9 +365,10 @@ qmm_status run_ffn_gate_up_silu_q4k(const LaunchCtx& c) {
   qmm_status st = QMM_OK;
   if (m < kQ4KGemmMinRows) {
     // Decode-sized call: the up product goes into the fixed decode scratch, behind the room the
-    // few-row kernels may use for their activation operand, so nothing is allocated (a recorded
+    // few-row kernels may use for their activation operand or their K parts, so nothing is allocated (a recorded
     // decode step stays valid).
-    const size_t up_off = (qmm::gemv_q4k_mfma_workspace_bytes(8, k) + 255) & ~size_t{255};
+    const size_t operand = qmm::gemv_q4k_mfma_workspace_bytes(8, k), parts = qmm::gemv_q4k_rows16_workspace_bytes(m, n, k);
+    const size_t up_off = ((operand > parts ? operand : parts) + 255) & ~size_t{255};
     if (decode_scratch(c) != nullptr && up_off + up_bytes <= kDecodeScratchBytes) {
       u = reinterpret_cast<float*>(static_cast<uint8_t*>(decode_scratch(c)) + up_off);
     }

@@ -117,6 +117,13 @@ hipError_t launch_embedding(int kind, const uint32_t* ids, const void* table, fl
 hipError_t launch_silu_mul(const float* g, const float* u, float* o, uint64_t n, hipStream_t stream);
 hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
 
+// Q4_K x 2..16 activation rows in one pass over the weights on the 16x16x32 fp16 MFMA, exact on the
+// weight side (gemv_q4k_rows16.hip).  `workspace` holds the K parts' output regions.
+bool gemv_q4k_rows16_supported(uint64_t m, uint64_t n, uint64_t k);
+size_t gemv_q4k_rows16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k);
+hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,
+                             uint32_t k, hipStream_t stream);
+
 // Q4_K, one activation row, K cut into `split` slices whose partial sums go to `split` output
 // regions of n floats (the caller's reduce adds them).
 bool q4k_gemv_split_supported(uint64_t n, uint64_t k, uint64_t split);

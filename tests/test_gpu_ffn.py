@@ -63,7 +63,8 @@ def test_one_row_matches_oracle(backend, n, k):
     assert rel_err(got, want) < TOL
 
 
-@pytest.mark.parametrize("m,n,k", [(2, 300, 5120), (5, 128, 4096), (16, 64, 2048), (17, 96, 1024), (40, 256, 512)])
+@pytest.mark.parametrize("m,n,k", [(2, 300, 5120), (5, 128, 4096), (16, 64, 2048), (17, 96, 1024), (40, 256, 512),
+                                   (6, 4100, 4096), (12, 4100, 4096), (3, 2052, 8192)])   # the last three: the one-pass few-row kernel
 def test_several_rows_match_oracle(backend, m, n, k):
     g = synth.rng(730 + m)
     gate, up = synth.q4k_weights(g, n, k), synth.q4k_weights(g, n, k)

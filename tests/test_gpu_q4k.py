@@ -260,6 +260,16 @@ def test_few_rows_scaling_and_exactness(backend):
     assert same_bits_zero_sign_free(got[0], deq[:, 5])
     assert same_bits_zero_sign_free(got[1], deq[:, 4095] * np.float32(2.0 ** -100))
     assert same_bits_zero_sign_free(got[2], deq[:, 1234] * np.float32(-(2.0 ** 90)))
+    # the same through the kernels that take 5..8 and 9..16 rows in one pass
+    for rows in (6, 13):
+        a = np.zeros((rows, k), np.float32)
+        pos = [int(p) for p in g.permutation(k)[:rows]]
+        vals = np.array([1.0, 2.0 ** -100, -(2.0 ** 90), 3.0, -0.375, 2.0 ** 20, 1.0, 1.0, 1.0, 1.0, 1.0, 1.0, 1.0], np.float32)
+        for r, t_ in enumerate(pos):
+            a[r, t_] = vals[r]
+        got = gemm(backend, "gemm_q4k_batched", a, w, rows, n, k)[0]
+        for r, t_ in enumerate(pos):
+            assert same_bits_zero_sign_free(got[r], deq[:, t_] * vals[r]), (rows, r, t_)
     # rows of very different magnitude, a zero row, and a row with a 1000x outlier
     a = synth.activations_f32(g, 5, k)
     a[0] *= np.float32(1e-30)

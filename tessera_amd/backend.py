@@ -75,6 +75,8 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
         "qmm_static_scratch_bytes": (sz, []),
         "qmm_workspace_bytes": (C.c_int32, [C.c_size_t, u64p, sz, C.POINTER(sz)]),
         "qmm_set_workspace": (C.c_int32, [vp, sz]),
+        "qmm_set_q4k_tensor_rows": (C.c_int32, [C.c_uint32]),
+        "qmm_q4k_tensor_rows": (C.c_uint32, []),
         "qmm_sync": (C.c_int32, [vp]),
         "qmm_last_error": (C.c_char_p, []),
     }
@@ -267,6 +269,14 @@ class Backend:
             self._check(self._lib.qmm_set_workspace(None, 0), "SetWorkspace")
         else:
             self._check(self._lib.qmm_set_workspace(C.c_void_p(buffer.Handle()), buffer.Size()), "SetWorkspace")
+
+    def SetQ4KTensorRows(self, rows: int) -> None:
+        """Row count from which the Q4_K ids other than gemm_q4k_wmma use the fp16 tensor-core tile
+        (``qmm_set_q4k_tensor_rows``; default 64 as the reference's table, at least 17, 0 = default)."""
+        self._check(self._lib.qmm_set_q4k_tensor_rows(int(rows)), "SetQ4KTensorRows")
+
+    def Q4KTensorRows(self) -> int:
+        return int(self._lib.qmm_q4k_tensor_rows())
 
     def StaticScratchBytes(self) -> int:
         return int(self._lib.qmm_static_scratch_bytes())

@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -141,23 +142,42 @@ void* decode_scratch(const LaunchCtx& c) {
   return c.no_alloc ? g_static_scratch[g_device] : g_decode_scratch;
 }
 
-// From this many rows on, Q4_K goes to the tiled fp16 MFMA GEMM: one more than the largest
-// speculative-verify batch (16), which stays on the exact fp32-accumulate paths as in the
-// reference (its fp16 tensor-core tile starts at 64 rows).  Below it, 2 and more rows of
-// a matrix with at least kQ4KFewRowsMinWeights weights go, eight at a time, to the exact
-// few-row MFMA kernels (weights read once per eight rows); one row and small matrices stay on
-// the VALU GEMV, which needs no activation pre-pass.
+// Q4_K regimes by activation rows.  One row and small matrices: the VALU GEMV.  2..16 rows of a
+// matrix with at least kQ4KFewRowsMinWeights weights: the exact few-row MFMA kernels (weights read
+// once).  The tiled fp16 MFMA GEMM, whose operands are rounded to fp16 as in the reference's
+// tensor-core tile: "gemm_q4k_wmma" from kQ4KGemmMinRows rows, the other ids from
+// g_q4k_tensor_rows rows -- 64 by default, where the reference's own regime table switches to its
+// fp16 tile (src/core/decode_internal.hpp:1349-1361), so that below it results keep the fp32
+// contract of the reference's tiled kernel; more rows than 16 below that run sixteen at a time
+// through the exact kernels.  qmm_set_q4k_tensor_rows lowers it (at least kQ4KGemmMinRows).
 constexpr uint64_t kQ4KGemmMinRows = 17;
+constexpr uint64_t kQ4KTensorRowsDefault = 64;
+std::atomic<uint64_t> g_q4k_tensor_rows{kQ4KTensorRowsDefault};
 constexpr uint64_t kMxfp4GemmMinRows = 17;   // below: the VALU GEMV passes, exact fp32 order
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KRows16MinRows = 3;      // from here the 16x16x32 kernel, below the 4x4x4 one
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
 
 qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
-                      uint64_t k) {
+                      uint64_t k, uint64_t f16_from) {
   const hipStream_t s = ctx.stream;
+  if (m >= f16_from && qmm::gemm_q4k_supported(m, k)) {
+    void* ws = nullptr;
+    const qmm_status st = workspace(ctx, qmm::gemm_q4k_workspace_bytes(m, k), &ws);
+    if (st != QMM_OK) return st;
+    return map_hip(qmm::launch_q4k_gemm(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                        static_cast<uint32_t>(k), s));
+  }
+  if (m > 16 && n * k >= kQ4KFewRowsMinWeights) {
+    // exact, sixteen rows at a time (each chunk takes the regime of its own row count)
+    for (uint64_t r = 0; r < m; r += 16) {
+      const qmm_status st = q4k_matmul(ctx, a + r * k, w, c + r * n, m - r < 16 ? m - r : 16, n, k, f16_from);
+      if (st != QMM_OK) return st;
+    }
+    return QMM_OK;
+  }
   // 3..16 rows of a large matrix: one pass over the weights on the 16x16x32 MFMA.
-  if (m >= kQ4KRows16MinRows && m < kQ4KGemmMinRows && n * k >= kQ4KFewRowsMinWeights && qmm::gemv_q4k_rows16_supported(m, n, k) &&
+  if (m >= kQ4KRows16MinRows && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemv_q4k_rows16_supported(m, n, k) &&
       qmm::gemv_q4k_rows16_workspace_bytes(m, n, k) <= kDecodeScratchBytes) {
     void* ws = decode_scratch(ctx);
     if (ws == nullptr) {
@@ -167,7 +187,7 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
     return map_hip(qmm::launch_q4k_rows16(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                           static_cast<uint32_t>(k), s));
   }
-  if (m >= 2 && m < kQ4KGemmMinRows && n * k >= kQ4KFewRowsMinWeights && k <= kQ4KFewRowsMaxK &&
+  if (m >= 2 && m <= 16 && n * k >= kQ4KFewRowsMinWeights && k <= kQ4KFewRowsMaxK &&
       qmm::gemv_q4k_mfma_supported(1, n, k)) {
     void* ws = decode_scratch(ctx);   // fixed address: a recorded decode step stays valid
     if (ws == nullptr || qmm::gemv_q4k_mfma_workspace_bytes(8, k) > kDecodeScratchBytes) {
@@ -182,21 +202,18 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
     }
     return QMM_OK;
   }
-  if (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) {
-    void* ws = nullptr;
-    const qmm_status st = workspace(ctx, qmm::gemm_q4k_workspace_bytes(m, k), &ws);
-    if (st != QMM_OK) return st;
-    return map_hip(qmm::launch_q4k_gemm(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
-                                        static_cast<uint32_t>(k), s));
-  }
   return map_hip(qmm::launch_q4k_gemv(a, w, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                       static_cast<uint32_t>(k), s));
+}
+qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
+                      uint64_t k) {
+  return q4k_matmul(ctx, a, w, c, m, n, k, g_q4k_tensor_rows.load(std::memory_order_relaxed));
 }
 
 // "gemm_q4k", "gemm_q4k_row", "gemm_q4k_batched", "gemm_q4k_wmma": buffers A, W, C;
 // scalars m, n, k (include/tessera/backend.hpp:153-161,207-209,397-415;
 // src/core/decode_internal.hpp:1484-1504).
-qmm_status run_gemm_q4k(const LaunchCtx& c) {
+qmm_status run_gemm_q4k_id(const LaunchCtx& c, bool wmma) {
   if (!counts(c, 3, 3)) return bad("gemm_q4k: expects 3 buffers and 3 scalars");
   const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
   if (!dims_ok(m, n, k) || k % 256 != 0) return bad("gemm_q4k: m, n, k must be non-zero and k a multiple of 256");
@@ -204,8 +221,11 @@ qmm_status run_gemm_q4k(const LaunchCtx& c) {
       !c.fits(2, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_q4k: a buffer is smaller than m, n, k require");
   }
-  return q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k);
+  return q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k,
+                    wmma ? kQ4KGemmMinRows : g_q4k_tensor_rows.load(std::memory_order_relaxed));
 }
+qmm_status run_gemm_q4k(const LaunchCtx& c) { return run_gemm_q4k_id(c, false); }
+qmm_status run_gemm_q4k_wmma(const LaunchCtx& c) { return run_gemm_q4k_id(c, true); }
 
 // "gemm_q4k_vec" and "gemm_q4k_rows{R}": buffers A, W, C; scalars m, n, k, split
 // (src/backends/rocm/rocm_kernels_gemv.cpp:17-24,103-156).  C has `split` regions of
@@ -341,6 +361,34 @@ qmm_status run_round_bf16(const LaunchCtx& c) {
 
 // "ffn_gate_up_silu_q4k" (not a reference id; the dense analogue of "moe_experts_gate_up_q4k"):
 // buffers X (fp32 m x k), Gate, Up (Q4_K, n rows of k each), Out (fp32 m x n); scalars m, n, k.
+// Where the up product of "ffn_gate_up_silu_q4k" with several rows lives.  Below the tensor-tile
+// threshold: in the fixed decode scratch, behind the room the few-row kernels may use for their
+// activation operand or their K parts, so nothing is allocated (a recorded decode step stays
+// valid) -- when it fits.  Otherwise in the workspace, behind whatever the Q4_K GEMM keeps at its
+// start (a request for that smaller size returns the same base, so the two do not overlap).
+struct FfnScratch {
+  bool in_decode_scratch;
+  size_t up_off;
+  size_t workspace_bytes;
+};
+FfnScratch ffn_scratch(uint64_t m, uint64_t n, uint64_t k) {
+  const size_t up_bytes = static_cast<size_t>(m) * n * 4;
+  const bool f16 = m >= g_q4k_tensor_rows.load(std::memory_order_relaxed) && qmm::gemm_q4k_supported(m, k);
+  if (!f16) {
+    const uint64_t chunk = m < 16 ? m : 16, tail = m % 16;
+    size_t room = qmm::gemv_q4k_mfma_workspace_bytes(8, k);
+    const size_t parts = qmm::gemv_q4k_rows16_workspace_bytes(chunk, n, k);
+    const size_t parts_tail = tail >= 2 ? qmm::gemv_q4k_rows16_workspace_bytes(tail, n, k) : 0;
+    room = room > parts ? room : parts;
+    room = room > parts_tail ? room : parts_tail;
+    const size_t up_off = (room + 255) & ~size_t{255};
+    if (up_off + up_bytes <= kDecodeScratchBytes) return FfnScratch{true, up_off, 0};
+    return FfnScratch{false, 0, up_bytes};
+  }
+  const size_t up_off = (qmm::gemm_q4k_workspace_bytes(m, k) + 255) & ~size_t{255};
+  return FfnScratch{false, up_off, up_off + up_bytes};
+}
+
 // Out = silu(X Gate^T) * (X Up^T), what the reference computes with two "gemm_q4k*" launches
 // and "silu_mul" (src/models/qwen3_5/trunk.cpp:294-304).  One row of a supported k is a single launch that
 // reads the activations once for both matrices; anything else runs the two products through the
@@ -360,28 +408,16 @@ qmm_status run_ffn_gate_up_silu_q4k(const LaunchCtx& c) {
   if (m == 1 && qmm::ffn_gate_up_q4k_supported(k)) {
     return map_hip(qmm::launch_ffn_gate_up_q4k(x, gate, up, out, static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
   }
-  const size_t up_bytes = static_cast<size_t>(m) * n * 4;
+  const FfnScratch lay = ffn_scratch(m, n, k);
   float* u = nullptr;
   qmm_status st = QMM_OK;
-  if (m < kQ4KGemmMinRows) {
-    // Decode-sized call: the up product goes into the fixed decode scratch, behind the room the
-    // few-row kernels may use for their activation operand or their K parts, so nothing is allocated (a recorded
-    // decode step stays valid).
-    const size_t operand = qmm::gemv_q4k_mfma_workspace_bytes(8, k), parts = qmm::gemv_q4k_rows16_workspace_bytes(m, n, k);
-    const size_t up_off = ((operand > parts ? operand : parts) + 255) & ~size_t{255};
-    if (decode_scratch(c) != nullptr && up_off + up_bytes <= kDecodeScratchBytes) {
-      u = reinterpret_cast<float*>(static_cast<uint8_t*>(decode_scratch(c)) + up_off);
-    }
-  }
-  if (u == nullptr) {
-    // The up product goes behind whatever the Q4_K GEMM keeps at the start of the workspace; a
-    // request for that smaller size returns the same base, so the two do not overlap.
-    const size_t gemm_ws = (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
-    const size_t up_off = (gemm_ws + 255) & ~size_t{255};
+  if (lay.in_decode_scratch && decode_scratch(c) != nullptr) {
+    u = reinterpret_cast<float*>(static_cast<uint8_t*>(decode_scratch(c)) + lay.up_off);
+  } else {
     void* ws = nullptr;
-    st = workspace(c, up_off + up_bytes, &ws);
+    st = workspace(c, lay.workspace_bytes, &ws);
     if (st != QMM_OK) return st;
-    u = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + up_off);
+    u = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + lay.up_off);
   }
   st = q4k_matmul(c, x, gate, out, m, n, k);
   if (st == QMM_OK) st = q4k_matmul(c, x, up, u, m, n, k);
@@ -852,7 +888,7 @@ const Entry kTable[] = {
     {"gemm_q4k", run_gemm_q4k},
     {"gemm_q4k_row", run_gemm_q4k},
     {"gemm_q4k_batched", run_gemm_q4k},
-    {"gemm_q4k_wmma", run_gemm_q4k},
+    {"gemm_q4k_wmma", run_gemm_q4k_wmma},
     {"gemm_q4k_vec", run_gemm_q4k_vec},
     {"gemm_q4k_rows2", run_gemm_q4k_rows2},
     {"gemm_q4k_rows3", run_gemm_q4k_rows3},
@@ -1089,13 +1125,11 @@ qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_
   auto starts = [&](const char* prefix) { return id.rfind(prefix, 0) == 0; };
   if (starts("gemm_q4k")) {
     const uint64_t m = sc(0), k = sc(2);
-    if (m >= kQ4KGemmMinRows && qmm::gemm_q4k_supported(m, k)) *out_bytes = qmm::gemm_q4k_workspace_bytes(m, k);
+    const uint64_t from = id == "gemm_q4k_wmma" ? kQ4KGemmMinRows : g_q4k_tensor_rows.load(std::memory_order_relaxed);
+    if (m >= from && qmm::gemm_q4k_supported(m, k)) *out_bytes = qmm::gemm_q4k_workspace_bytes(m, k);
   } else if (id == "ffn_gate_up_silu_q4k") {
     const uint64_t m = sc(0), n = sc(1), k = sc(2);
-    if (m >= kQ4KGemmMinRows) {
-      const size_t gemm_ws = qmm::gemm_q4k_supported(m, k) ? qmm::gemm_q4k_workspace_bytes(m, k) : 0;
-      *out_bytes = ((gemm_ws + 255) & ~size_t{255}) + static_cast<size_t>(m) * n * 4;
-    }
+    if (m >= 2 && n != 0 && k != 0) *out_bytes = ffn_scratch(m, n, k).workspace_bytes;
   } else if (id == "gemm_mxfp4" || id == "gemm_mxfp4_batched") {
     const uint64_t m = sc(0), k = sc(2);
     if (m >= kMxfp4GemmMinRows && qmm::gemm_mxfp4_f32_supported(m, k)) *out_bytes = qmm::gemm_mxfp4_f32_workspace_bytes(m, k);
@@ -1111,6 +1145,15 @@ qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_
   }
   return QMM_OK;
 }
+
+qmm_status qmm_set_q4k_tensor_rows(uint32_t rows) {
+  if (rows == 0) rows = static_cast<uint32_t>(kQ4KTensorRowsDefault);
+  if (rows < kQ4KGemmMinRows) return bad("qmm_set_q4k_tensor_rows: at least 17 rows (the verify batch of up to 16 stays exact)");
+  g_q4k_tensor_rows.store(rows, std::memory_order_relaxed);
+  return QMM_OK;
+}
+
+uint32_t qmm_q4k_tensor_rows(void) { return static_cast<uint32_t>(g_q4k_tensor_rows.load(std::memory_order_relaxed)); }
 
 qmm_status qmm_set_workspace(void* device_ptr, size_t bytes) {
   if ((device_ptr == nullptr) != (bytes == 0)) return bad("qmm_set_workspace: pointer and size must both be set or both be zero");

@@ -1,4 +1,7 @@
-"""Q4_K prefill GEMM on fp16 MFMA (the Q4_K GEMM ids from 17 rows on) against the CPU oracle.
+"""Q4_K prefill GEMM on fp16 MFMA against the CPU oracle: gemm_q4k_wmma from 17 rows on, the other
+Q4_K ids from 64 rows on (the reference's regime table, src/core/decode_internal.hpp:1349-1361;
+below that they keep fp32 activations, sixteen rows at a time through the exact kernels) or from
+the row count set with SetQ4KTensorRows.
 
 The kernel multiplies fp16 activations by fp16 weights and accumulates in fp32, like the
 reference's tensor-core tile (src/backends/rocm/rocm_kernels_wmma.cpp:334-431).  Its weights are
@@ -19,7 +22,7 @@ import pytest
 
 import oracle
 from tessera_amd import synth
-from util import norm_err, rms_err, run, same_bits_zero_sign_free
+from util import norm_err, rel_err, rms_err, run, same_bits_zero_sign_free
 
 pytestmark = pytest.mark.gpu
 ACC_TOL = 3e-5          # fp32 accumulation order, in units of the rms output
@@ -106,7 +109,37 @@ def test_gemm_matches_oracle(backend, m, n, k, kind):
     ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
     for name in ("gemm_q4k_wmma", "gemm_q4k_batched"):
         got = gemm(backend, name, a, w, m, n, k)
-        check(got, a, w, m, n, k, ref, f"{name} {m}x{n}x{k} {kind}")
+        if name == "gemm_q4k_batched" and m < 64:
+            # fp32 activations, as the reference's tiled kernel below its tensor-core regime
+            assert rel_err(got, ref) <= 1e-3 and rms_err(got, ref) <= 1e-4, (name, m, rel_err(got, ref), rms_err(got, ref))
+        else:
+            check(got, a, w, m, n, k, ref, f"{name} {m}x{n}x{k} {kind}")
+
+
+def test_tensor_rows_setting(backend):
+    """gemm_q4k_batched between 17 and 63 rows: exact by default (the one-pass few-row kernel,
+    sixteen rows at a time), the fp16 tile -- bit for bit gemm_q4k_wmma's result -- once the caller
+    lowers the threshold; fewer than 17 is refused; 0 restores the default."""
+    g = synth.rng(515)
+    m, n, k = 40, 4100, 4096                  # 16.8 M weights: the few-row kernels take it
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
+    assert backend.Q4KTensorRows() == 64
+    exact = gemm(backend, "gemm_q4k_batched", a, w, m, n, k)
+    tile = gemm(backend, "gemm_q4k_wmma", a, w, m, n, k)
+    assert rel_err(exact, ref) <= 1e-3 and rms_err(exact, ref) <= 1e-4
+    assert rms_err(tile, ref) > rms_err(exact, ref)
+    try:
+        backend.SetQ4KTensorRows(17)
+        assert backend.Q4KTensorRows() == 17
+        assert np.array_equal(gemm(backend, "gemm_q4k_batched", a, w, m, n, k), tile)
+        with pytest.raises(Exception):
+            backend.SetQ4KTensorRows(16)
+    finally:
+        backend.SetQ4KTensorRows(0)
+    assert backend.Q4KTensorRows() == 64
+    assert np.array_equal(gemm(backend, "gemm_q4k_batched", a, w, m, n, k), exact)
 
 
 def test_gemm_one_hot_is_the_fp16_dequant(backend):

@@ -270,6 +270,15 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
                                          scalars=[m, nn, k, 1, 0]))], 10, graph=False)
         prefill[f"mxfp4_{label}"].update({"ms_with_quantize": round(us / 1e3, 4),
                                           "TFLOPs_with_quantize": round(2 * m * nn * k / us / 1e6, 1)})
+        if nn == n:
+            # the same weights in the reference's load-time fragment order (PermuteMxFp4ToWmma, wperm = 1)
+            wp = torch.empty_like(w_mx)
+            backend.LaunchKernel(backend.LoadKernel("permute_mxfp4_wmma"),
+                                 KernelLaunch(grid_x=1, buffers=[wrap(w_mx), wrap(wp)], scalars=[n, k, 0]))
+            us = timed_us([(kg, KernelLaunch(grid_x=nn // 64, buffers=[wrap(a8), wrap(wp), wrap(asc), wrap(wref), wrap(y)],
+                                             scalars=[m, nn, k, 1, 1]))], 10, graph=False)
+            prefill[f"mxfp4_{label}"].update({"ms_wperm": round(us / 1e3, 4), "TFLOPs_wperm": round(2 * m * nn * k / us / 1e6, 1)})
+            del wp
         # fp32 activation rows, not quantized ("gemm_mxfp4_batched", the reference's prefill id): bf16-valued
         # rows are two E4M3 terms, so the matrix cores do twice the E4M3 x E2M1 work counted here
         us = timed_us([(kmb, KernelLaunch(grid_x=(nn + 7) // 8, buffers=[wrap(a), wrap(wm), wrap(y)], scalars=[m, nn, k]))],

@@ -63,6 +63,7 @@ def _load() -> C.CDLL:
         "orc_gemm_mxfp4_ref_omp": (C.c_int, [f32p, u8p, u8p, f32p, sz, sz, sz]),
         "orc_dequantize_mxfp4": (C.c_int, [u8p, f32p, sz, sz]),
         "orc_gemm_fp8_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
+        "orc_permute_mxfp4_to_wmma": (C.c_int, [u8p, u8p, sz, sz]),
         "orc_fold_entry": (C.c_uint8, [C.c_uint, C.c_uint]),
         "orc_fold_entry_rne": (C.c_uint8, [C.c_uint, C.c_uint]),
         "orc_fold_mxfp4_to_fp8": (C.c_int, [u8p, u8p, u8p, u8p, sz, sz]),
@@ -291,6 +292,15 @@ def quantize_fp8_pack(data, rows: int, cols: int) -> tuple[np.ndarray, np.ndarra
     _check(_lib.orc_quantize_fp8_pack_ref(_p(src, C.c_float), _p(codes, C.c_uint8),
                                           _p(scale, C.c_float), rows, cols))
     return codes, scale
+
+
+def permute_mxfp4_to_wmma(packed, n: int, k: int) -> np.ndarray:
+    """Packed MXFP4 (nibble bytes then scales) with the nibble bytes in the 16-row fragment order;
+    the scales stay where they are."""
+    blob, s = split_mxfp4(packed, n, k)
+    out = np.empty_like(blob)
+    _check(_lib.orc_permute_mxfp4_to_wmma(_p(blob, C.c_uint8), _p(out, C.c_uint8), n, k))
+    return np.concatenate([out.reshape(-1), s.reshape(-1)])
 
 
 def fold_mxfp4_to_fp8(packed, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:

@@ -632,6 +632,26 @@ int orc_fold_mxfp4_to_fp8(const uint8_t* w, const uint8_t* s, uint8_t* out, uint
   return ORC_OK;
 }
 
+/* ---- MXFP4 nibble bytes, row-major -> the 16-row fragment order of the fp8 tensor-core kernel
+ *      (PermuteMxFp4ToWmma, quant.cpp:926-954): input byte (t, r, s, h, b) =
+ *      (((t*16 + r)*ks + s)*2 + h)*4 + b goes to (((t*ks + s)*2 + h)*16 + r)*4 + b, ks = cols/16 ---- */
+int orc_permute_mxfp4_to_wmma(const uint8_t* packed, uint8_t* out, size_t rows, size_t cols) {
+  if (rows == 0 || cols == 0 || rows % 16 != 0 || cols % 16 != 0) return ORC_INVALID_ARGUMENT;
+  const size_t nt = rows / 16, ks = cols / 16;
+  for (size_t t = 0; t < nt; ++t) {
+    for (size_t s = 0; s < ks; ++s) {
+      for (size_t h = 0; h < 2; ++h) {
+        for (size_t r = 0; r < 16; ++r) {
+          const size_t in = (((t * 16 + r) * ks + s) * 2 + h) * 4;
+          const size_t o = (((t * ks + s) * 2 + h) * 16 + r) * 4;
+          for (size_t b = 0; b < 4; ++b) out[o + b] = packed[in + b];
+        }
+      }
+    }
+  }
+  return ORC_OK;
+}
+
 /* ---- folded W4A8 GEMM: (sum fma(a8, w8)) * As[m] * 2^(wref-127)
  *      (quant.cpp:900-924) ---- */
 int orc_gemm_mxfp4_fp8_ref(const uint8_t* a8, const float* as, const uint8_t* w8,

@@ -563,6 +563,38 @@ hipError_t launch_quantize_fp8_pack_bf16(const uint16_t* in, uint8_t* out, float
   return hipGetLastError();
 }
 
+// Packed MXFP4 nibble bytes between row-major and the reference's 16-row fragment order
+// (PermuteMxFp4ToWmma, src/core/numerics/quant.cpp:926-954): dword (t, r, s, h) of the row-major
+// matrix, ((t*16 + r) * k/16 + s) * 2 + h, sits at ((t * k/16 + s) * 2 + h) * 16 + r.  One thread per
+// dword; the threads past the nibble bytes copy the scale bytes unchanged.
+__global__ __launch_bounds__(256) void permute_mxfp4_wmma_kernel(const uint32_t* __restrict__ in, uint32_t* __restrict__ out,
+                                                                 uint64_t n, uint64_t k, int inverse) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  const uint64_t blob_dwords = n * k / 8, scale_dwords = n * k / 32 / 4;
+  if (i >= blob_dwords + scale_dwords) return;
+  if (i >= blob_dwords) {
+    out[i] = in[i];
+    return;
+  }
+  const uint64_t ks = k / 16;
+  // i indexes the fragment order: r fastest, then h, then s, then t
+  const uint64_t r = i % 16, h = (i / 16) % 2, s_ = (i / 32) % ks, t = i / (32 * ks);
+  const uint64_t row_major = ((t * 16 + r) * ks + s_) * 2 + h;
+  if (inverse) {
+    out[row_major] = in[i];
+  } else {
+    out[i] = in[row_major];
+  }
+}
+
+hipError_t launch_permute_mxfp4_wmma(const uint8_t* in, uint8_t* out, uint64_t n, uint64_t k, bool inverse,
+                                     hipStream_t stream) {
+  const uint64_t dwords = n * k / 8 + n * k / 128;
+  hipLaunchKernelGGL(permute_mxfp4_wmma_kernel, grid_for(dwords, 256), dim3(256), 0, stream,
+                     reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n, k, inverse ? 1 : 0);
+  return hipGetLastError();
+}
+
 hipError_t launch_mxfp4_row_ref(const uint8_t* w, uint8_t* wref, uint64_t n, uint64_t k,
                                 hipStream_t stream) {
   hipLaunchKernelGGL(mxfp4_row_ref_kernel, grid_for(n, 4), dim3(256), 0, stream, w, wref, n, k);

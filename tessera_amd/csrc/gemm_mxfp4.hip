@@ -52,7 +52,14 @@ __device__ __forceinline__ void direct_load4(const void* base, uint32_t voff, ui
 // planes of m x k codes, term t weighing 2^(-4t); `need` says how many terms each row has.  A
 // tile walks K once per term it needs, all into the same accumulators, the term's weight being
 // the E8M0 scale of the A operand.
-template <int BM, int BN, int WM, int WN, bool SPLIT>
+//
+// WPERM: the nibble bytes of W are in the reference's 16-row fragment order (PermuteMxFp4ToWmma,
+// src/core/numerics/quant.cpp:926-954: dword (tile t, 16-wide K step s, half h, row r) at
+// ((t * k/16 + s) * 2 + h) * 16 + r; the scales stay row-major).  The 16 rows x 128 K of one
+// direct-load block are still 1 KB of contiguous memory, only transposed inside, so the block is
+// fetched dword by dword (global_load_lds_dword), each lane asking for the dword that belongs at
+// its LDS position: the LDS image, and everything after it, is the row-major one.
+template <int BM, int BN, int WM, int WN, bool SPLIT, bool WPERM = false>
 __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
     const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
     float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t n_begin, uint32_t n_end,
@@ -62,7 +69,8 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   static_assert((BM / 8) % kWaves == 0 && (BN / 16) % kWaves == 0, "direct-load blocks divide among the wavefronts");
   constexpr int kTI = BM / WM / 32, kTJ = BN / WN / 32;      // MFMA tiles per wavefront
   constexpr int kABlk = BM / 8 / kWaves, kBBlk = BN / 16 / kWaves;  // 1 KB direct-load blocks per wavefront
-  constexpr int kDma = kABlk + kBBlk + 1;                    // direct loads a wavefront issues per stage
+  constexpr int kBLoads = WPERM ? 4 : 1;                     // load instructions per weight block
+  constexpr int kDma = kABlk + kBBlk * kBLoads + 1;          // direct loads a wavefront issues per stage
   constexpr uint32_t kBBase = BM * kKS, kSBase = kBBase + BN * kKS / 2;
   constexpr uint32_t kStage = kSBase + BN * 4;
   __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kStage];
@@ -84,7 +92,7 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   // stage; rows past the matrix edge are clamped to the last row (never stored).
   struct Source {
     const uint8_t *a, *b, *s;           // tile origins (wave-uniform)
-    uint32_t a_off[kABlk], b_off[kBBlk], s_off;
+    uint32_t a_off[kABlk], b_off[kBBlk][kBLoads], s_off;
     uint32_t terms;                     // passes over K (SPLIT)
   };
   const size_t plane = static_cast<size_t>(m) * k;
@@ -104,7 +112,7 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
     const uint32_t m0 = (tile / tiles_n) * BM, n0 = n_begin + (tile % tiles_n) * BN;
     src.terms = tile_terms(m0);
     src.a = a8 + static_cast<size_t>(m0) * k;
-    src.b = w + static_cast<size_t>(n0) * row_bytes;
+    src.b = w + static_cast<size_t>(n0) * row_bytes;        // also the origin of 16-row tile n0 / 16 in fragment order
     src.s = w + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(n0) * row_blocks;
 #pragma unroll
     for (int i = 0; i < kABlk; ++i) {
@@ -114,9 +122,22 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
     }
 #pragma unroll
     for (int i = 0; i < kBBlk; ++i) {
-      const uint32_t row = 16u * (wave * kBBlk + i) + lane / 4u;
-      const uint32_t chunk = (lane % 4u) ^ ((row >> 2) & 3u);
-      src.b_off[i] = (n0 + row < n ? row : n - 1u - n0) * row_bytes + chunk * 16u;
+      if constexpr (WPERM) {
+        // LDS dword d = j * 64 + lane of the block is dword d % 4 of chunk position (d % 16) / 4 of
+        // row d / 16, i.e. dword wd = 4 * (position ^ swizzle) + d % 4 of the row's 64 bytes.
+        const uint32_t blk = wave * kBBlk + i;
+        const uint32_t blk_in = n0 + 16u * blk < n ? blk : (n - 1u - n0) / 16u;    // n is a multiple of 16
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t d = j * 64u + lane, row = d / 16u, pos = (d % 16u) / 4u;
+          const uint32_t wd = 4u * (pos ^ ((row >> 2) & 3u)) + d % 4u;
+          src.b_off[i][j] = blk_in * 16u * row_bytes + (wd * 16u + row) * 4u;
+        }
+      } else {
+        const uint32_t row = 16u * (wave * kBBlk + i) + lane / 4u;
+        const uint32_t chunk = (lane % 4u) ^ ((row >> 2) & 3u);
+        src.b_off[i][0] = (n0 + row < n ? row : n - 1u - n0) * row_bytes + chunk * 16u;
+      }
     }
     const uint32_t row = 64u * (wave % (BN / 64)) + lane;
     src.s_off = (n0 + row < n ? row : n - 1u - n0) * row_blocks;
@@ -124,12 +145,19 @@ __global__ __launch_bounds__(64 * WM * WN) void mxfp4_a8_gemm_kernel(
   auto issue_stage = [&](uint32_t stage_off, const Source& src, uint32_t k0, uint32_t term) {
     const uint32_t stage = lds_base + stage_off;
     const uint8_t* ga = src.a + (SPLIT ? term * plane : 0) + k0;
-    const uint8_t* gb = src.b + k0 / 2;
+    const uint8_t* gb = src.b + (WPERM ? k0 * 8u : k0 / 2);     // fragment order: 128 bytes per 16-wide K step of a tile
     const uint8_t* gs = src.s + k0 / 32;
 #pragma unroll
     for (int i = 0; i < kABlk; ++i) direct_load16(ga, src.a_off[i], stage + (wave * kABlk + i) * 1024u);
 #pragma unroll
-    for (int i = 0; i < kBBlk; ++i) direct_load16(gb, src.b_off[i], stage + kBBase + (wave * kBBlk + i) * 1024u);
+    for (int i = 0; i < kBBlk; ++i) {
+      if constexpr (WPERM) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) direct_load4(gb, src.b_off[i][j], stage + kBBase + (wave * kBBlk + i) * 1024u + j * 256u);
+      } else {
+        direct_load16(gb, src.b_off[i][0], stage + kBBase + (wave * kBBlk + i) * 1024u);
+      }
+    }
     direct_load4(gs, src.s_off, stage + kSBase + (wave % (BN / 64)) * 256u);
   };
 
@@ -667,10 +695,13 @@ namespace {
 template <int BM, int BN, int WM, int WN>
 void launch_range(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m, uint32_t n,
                   uint32_t k, uint32_t n_begin, uint32_t n_end, uint32_t max_groups, const uint8_t* need,
-                  hipStream_t stream) {
+                  bool wperm, hipStream_t stream) {
   const uint32_t tiles = ((m + BM - 1) / BM) * ((n_end - n_begin + BN - 1) / BN);
   const uint32_t grid = tiles < max_groups ? tiles : max_groups;
-  if (need != nullptr) {
+  if (wperm) {
+    hipLaunchKernelGGL((mxfp4_a8_gemm_kernel<BM, BN, WM, WN, false, true>), dim3(grid), dim3(64 * WM * WN), 0, stream,
+                       a8, as, w, c, m, n, k, n_begin, n_end, need);
+  } else if (need != nullptr) {
     hipLaunchKernelGGL((mxfp4_a8_gemm_kernel<BM, BN, WM, WN, true>), dim3(grid), dim3(64 * WM * WN), 0, stream,
                        a8, as, w, c, m, n, k, n_begin, n_end, need);
   } else {
@@ -681,7 +712,7 @@ void launch_range(const uint8_t* a8, const float* as, const uint8_t* w, float* c
 
 // Tiled launch of C = diag(as) . A8 . deq(W)^T; `need` non-null selects the split-activation form.
 void launch_tiles(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m, uint32_t n,
-                  uint32_t k, const uint8_t* need, hipStream_t stream) {
+                  uint32_t k, const uint8_t* need, bool wperm, hipStream_t stream) {
   const uint32_t cus = static_cast<uint32_t>(num_cus());
   const uint32_t tiles_m = (m + 255u) / 256u, tiles_n = (n + 255u) / 256u;
   const uint32_t tiles = tiles_m * tiles_n;
@@ -692,8 +723,8 @@ void launch_tiles(const uint8_t* a8, const float* as, const uint8_t* w, float* c
     main_tn = 0;                        // too few large tiles to fill the chip: small tiles throughout
   }
   const uint32_t n_split = main_tn * 256u < n ? main_tn * 256u : n;
-  if (n_split > 0) launch_range<256, 256, 4, 2>(a8, as, w, c, m, n, k, 0u, n_split, cus, need, stream);
-  if (n_split < n) launch_range<128, 64, 2, 2>(a8, as, w, c, m, n, k, n_split, n, 2u * cus, need, stream);
+  if (n_split > 0) launch_range<256, 256, 4, 2>(a8, as, w, c, m, n, k, 0u, n_split, cus, need, wperm, stream);
+  if (n_split < n) launch_range<128, 64, 2, 2>(a8, as, w, c, m, n, k, n_split, n, 2u * cus, need, wperm, stream);
 }
 
 }  // namespace
@@ -722,7 +753,17 @@ hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_
     }
     return hipGetLastError();
   }
-  launch_tiles(a8, as, w, c, m, n, k, nullptr, stream);
+  launch_tiles(a8, as, w, c, m, n, k, nullptr, false, stream);
+  return hipGetLastError();
+}
+
+// The tiled kernel on weights in the reference's fragment order (n a multiple of 16, more than 32 rows).
+bool gemm_mxfp4_a8_wperm_supported(uint64_t m, uint64_t n, uint64_t k) {
+  return m > 32 && n % 16 == 0 && k >= 1024 && gemm_mxfp4_a8_supported(k);
+}
+hipError_t launch_mxfp4_a8_gemm_wperm(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m,
+                                      uint32_t n, uint32_t k, hipStream_t stream) {
+  launch_tiles(a8, as, w, c, m, n, k, nullptr, true, stream);
   return hipGetLastError();
 }
 
@@ -738,7 +779,7 @@ hipError_t launch_mxfp4_f32_gemm(const float* a, const uint8_t* w, float* c, voi
   float* as = reinterpret_cast<float*>(planes + static_cast<size_t>(kMaxTerms) * m * k);
   uint8_t* need = reinterpret_cast<uint8_t*>(as) + ((static_cast<size_t>(m) * 4 + 255) / 256) * 256;
   hipLaunchKernelGGL(split_rows_kernel, dim3(m), dim3(256), 0, stream, a, planes, as, need, m, k);
-  launch_tiles(planes, as, w, c, m, n, k, need, stream);
+  launch_tiles(planes, as, w, c, m, n, k, need, false, stream);
   return hipGetLastError();
 }
 

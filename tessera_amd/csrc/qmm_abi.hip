@@ -603,9 +603,8 @@ qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
   const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], split = c.sc[3], wperm = c.sc[4];
   if (!dims_ok(m, n, k) || k % 32 != 0) return bad("gemm_mxfp4_wmma: bad m, n, k");
   if (split == 0 || split > 64) return bad("gemm_mxfp4_wmma: bad split");
-  if (wperm != 0) {
-    g_last_error = "gemm_mxfp4_wmma: pre-permuted weights are not supported";
-    return QMM_UNSUPPORTED_FEATURE;
+  if (wperm > 1 || (wperm == 1 && (n % 16 != 0 || k % 16 != 0))) {
+    return bad("gemm_mxfp4_wmma: wperm is 0 or 1, and fragment-ordered weights have n and k multiples of 16");
   }
   const u128 region = static_cast<u128>(m) * n * 4;
   if (!c.fits(0, static_cast<u128>(m) * k) || !c.fits(1, mxfp4_bytes(n, k)) || !c.fits(2, m * 4) ||
@@ -613,11 +612,30 @@ qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
     return bad("gemm_mxfp4_wmma: a buffer is smaller than m, n, k, split require");
   }
   float* out = c.ptr<float>(4);
+  const uint8_t* w = c.ptr<const uint8_t>(1);
+  if (wperm == 1) {
+    // Weights in the reference's fragment order (PermuteMxFp4ToWmma, quant.cpp:926-954): the tiled
+    // kernel reads them as they are; the few-row and single-row kernels want row-major runs, so
+    // for them the matrix is put back into row-major order in the workspace first.
+    if (m <= 0xFFFFFFFFull && n <= 0xFFFFFFFFull && qmm::gemm_mxfp4_a8_wperm_supported(m, n, k)) {
+      qmm_status st = map_hip(qmm::launch_mxfp4_a8_gemm_wperm(
+          c.ptr<const uint8_t>(0), c.ptr<const float>(2), w, out, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+          static_cast<uint32_t>(k), c.stream));
+      if (st == QMM_OK && split > 1) st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
+      return st;
+    }
+    void* ws = nullptr;
+    qmm_status st = workspace(c, static_cast<size_t>(mxfp4_bytes(n, k)), &ws);
+    if (st != QMM_OK) return st;
+    st = map_hip(qmm::launch_permute_mxfp4_wmma(w, static_cast<uint8_t*>(ws), n, k, true, c.stream));
+    if (st != QMM_OK) return st;
+    w = static_cast<const uint8_t*>(ws);
+  }
   // Regime: a single row stays on the VALU GEMV; from two rows on the scaled MFMA takes over
   // (a streaming kernel up to 32 rows, the tiled GEMM above that).
   if (m > 1 && k >= 1024 && qmm::gemm_mxfp4_a8_supported(k)) {
     qmm_status st = map_hip(qmm::launch_mxfp4_a8_gemm(
-        c.ptr<const uint8_t>(0), c.ptr<const float>(2), c.ptr<const uint8_t>(1), out,
+        c.ptr<const uint8_t>(0), c.ptr<const float>(2), w, out,
         static_cast<uint32_t>(m), static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
     if (st == QMM_OK && split > 1) {
       st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
@@ -625,12 +643,25 @@ qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
     return st;
   }
   qmm_status st = map_hip(qmm::launch_mxfp4_a8_gemv(
-      c.ptr<const uint8_t>(0), c.ptr<const float>(2), c.ptr<const uint8_t>(1), out,
+      c.ptr<const uint8_t>(0), c.ptr<const float>(2), w, out,
       static_cast<uint32_t>(m), static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
   if (st == QMM_OK && split > 1) {
     st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
   }
   return st;
+}
+
+// "permute_mxfp4_wmma" (not a reference id; the device form of the reference's load-time
+// PermuteMxFp4ToWmma, src/core/numerics/quant.cpp:926-954): buffers In, Out (packed MXFP4, n*k/2
+// nibble bytes then n*k/32 scale bytes); scalars n, k (multiples of 16 and 32), inverse (0: row-major
+// -> fragment order, 1: back).  The scale bytes are copied unchanged.
+qmm_status run_permute_mxfp4_wmma(const LaunchCtx& c) {
+  if (!counts(c, 2, 3)) return bad("permute_mxfp4_wmma: expects 2 buffers and 3 scalars");
+  const uint64_t n = c.sc[0], k = c.sc[1], inverse = c.sc[2];
+  if (!dims_ok(1, n, k) || n % 16 != 0 || k % 32 != 0 || inverse > 1) return bad("permute_mxfp4_wmma: n a multiple of 16, k of 32, inverse 0 or 1");
+  if (!c.fits(0, mxfp4_bytes(n, k)) || !c.fits(1, mxfp4_bytes(n, k))) return bad("permute_mxfp4_wmma: buffer too small");
+  if (c.buf[0] == c.buf[1]) return bad("permute_mxfp4_wmma: not in place");
+  return map_hip(qmm::launch_permute_mxfp4_wmma(c.ptr<const uint8_t>(0), c.ptr<uint8_t>(1), n, k, inverse == 1, c.stream));
 }
 
 // "dequant_mxfp4" (not a reference id): buffers W (packed), Out (n x k fp32); scalars n, k.
@@ -945,6 +976,7 @@ const Entry kTable[] = {
     {"gemm_q6k_rows5", run_gemm_q6k_rows5},
     {"dequant_q6k", run_dequant_q6k},
     {"dequant_mxfp4", run_dequant_mxfp4},
+    {"permute_mxfp4_wmma", run_permute_mxfp4_wmma},
     {"quantize_fp8_pack_a16", run_quantize_fp8_pack_a16},
 };
 constexpr size_t kTableSize = sizeof(kTable) / sizeof(kTable[0]);
@@ -1130,6 +1162,9 @@ qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_
   } else if (id == "ffn_gate_up_silu_q4k") {
     const uint64_t m = sc(0), n = sc(1), k = sc(2);
     if (m >= 2 && n != 0 && k != 0) *out_bytes = ffn_scratch(m, n, k).workspace_bytes;
+  } else if (id == "gemm_mxfp4_wmma") {
+    const uint64_t m = sc(0), n = sc(1), k = sc(2), wperm = sc(4);
+    if (wperm == 1 && !qmm::gemm_mxfp4_a8_wperm_supported(m, n, k)) *out_bytes = static_cast<size_t>(mxfp4_bytes(n, k));
   } else if (id == "gemm_mxfp4" || id == "gemm_mxfp4_batched") {
     const uint64_t m = sc(0), k = sc(2);
     if (m >= kMxfp4GemmMinRows && qmm::gemm_mxfp4_f32_supported(m, k)) *out_bytes = qmm::gemm_mxfp4_f32_workspace_bytes(m, k);

@@ -65,6 +65,15 @@ bool gemm_mxfp4_a8_supported(uint64_t k);
 hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
 
+// The same with W's nibble bytes in the reference's 16-row fragment order (PermuteMxFp4ToWmma,
+// src/core/numerics/quant.cpp:926-954), tiled kernel only.
+bool gemm_mxfp4_a8_wperm_supported(uint64_t m, uint64_t n, uint64_t k);
+hipError_t launch_mxfp4_a8_gemm_wperm(const uint8_t* a8, const float* as, const uint8_t* w, float* c, uint32_t m,
+                                      uint32_t n, uint32_t k, hipStream_t stream);
+// Packed MXFP4 (nibble bytes then scales) between row-major and that fragment order; the scales are copied.
+hipError_t launch_permute_mxfp4_wmma(const uint8_t* in, uint8_t* out, uint64_t n, uint64_t k, bool inverse,
+                                     hipStream_t stream);
+
 // MXFP4 weights, fp32 activation rows (17 or more): the rows are split into E4M3 terms in the
 // workspace and multiplied on the same scaled MFMA, one pass over K per term.
 bool gemm_mxfp4_f32_supported(uint64_t m, uint64_t k);

@@ -87,3 +87,56 @@ def test_down_projection_shape_prefill_rows(backend):
     codes, scale = oracle.quantize_fp8_pack(x[rows], len(rows), k)
     ref = oracle.gemm_mxfp4_w4a8(codes, scale, w, len(rows), n, k)
     assert rms_err(got[rows], ref) <= 5e-4, rms_err(got[rows], ref)
+
+
+# ---- weights pre-permuted at load (the reference's PermuteMxFp4ToWmma, quant.cpp:926-954, wperm = 1) ----
+@pytest.mark.parametrize("n,k", [(16, 32), (48, 256), (272, 1024), (1040, 5120)])
+def test_permute_id_is_the_reference_permutation(backend, n, k):
+    """permute_mxfp4_wmma on the device against the oracle's restatement, and back again."""
+    g = synth.rng(n + k)
+    w = synth.mxfp4_weights(g, n, k, -20, 20)
+    want = oracle.permute_mxfp4_to_wmma(w, n, k)
+    dw, dp, db = backend.Upload(w), backend.AllocateBuffer(w.size), backend.AllocateBuffer(w.size)
+    run(backend, "permute_mxfp4_wmma", [dw, dp], [n, k, 0], grid=((w.size + 255) // 256, 1, 1))
+    run(backend, "permute_mxfp4_wmma", [dp, db], [n, k, 1], grid=((w.size + 255) // 256, 1, 1))
+    backend.Synchronize()
+    assert np.array_equal(backend.CopyD2H(dp), want)
+    assert np.array_equal(backend.CopyD2H(db), w)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 1024), (4, 272, 2048), (16, 128, 512), (32, 96, 1024), (33, 272, 1024),
+                                   (130, 1040, 1024), (300, 64, 2048), (64, 336, 5120), (40, 48, 1056)])
+def test_wperm_gives_the_same_result(backend, m, n, k):
+    """gemm_mxfp4_wmma with wperm = 1 on the permuted copy equals wperm = 0 on the GGUF layout bit
+    for bit, in every regime (single row, few rows, tiled; ragged last tiles; a K the tiled kernel
+    does not take); the permuted copy's dequant dump after permuting back is the oracle's."""
+    g = synth.rng(31 * m + n + k)
+    w = synth.mxfp4_weights(g, n, k, -8, -4)
+    x = synth.activations_bf16_outliers(g, m, k)
+    wp = oracle.permute_mxfp4_to_wmma(w, n, k)
+    dx = backend.Upload(x)
+    da8, das = backend.AllocateBuffer(m * k), backend.AllocateBuffer(4 * m)
+    dref = backend.AllocateBuffer(n)
+    run(backend, "quantize_fp8_pack_rows", [dx, da8, das], [m, k], grid=(m, 1, 1))
+    outs = []
+    for weights, wperm in ((w, 0), (wp, 1)):
+        dw, out = backend.Upload(weights), backend.AllocateBuffer(4 * m * n)
+        run(backend, "gemm_mxfp4_wmma", [da8, dw, das, dref, out], [m, n, k, 1, wperm], grid=((n + 63) // 64, 1, 1))
+        backend.Synchronize()
+        outs.append(backend.CopyD2H(out, dtype=np.float32))
+    assert np.array_equal(outs[0], outs[1])
+    codes, scale = oracle.quantize_fp8_pack(x, m, k)
+    ref = oracle.gemm_mxfp4_w4a8(codes, scale, w, m, n, k)
+    assert rms_err(outs[1].reshape(m, n), ref) <= 5e-4
+
+
+def test_wperm_needs_whole_fragments(backend):
+    from tessera_amd import StatusCode, StatusError
+    g = synth.rng(8)
+    m, n, k = 4, 40, 256                       # n is not a multiple of 16
+    w = synth.mxfp4_weights(g, n, k)
+    bufs = [backend.AllocateBuffer(m * k), backend.Upload(w), backend.AllocateBuffer(4 * m), backend.AllocateBuffer(n),
+            backend.AllocateBuffer(4 * m * n)]
+    with pytest.raises(StatusError) as e:
+        run(backend, "gemm_mxfp4_wmma", bufs, [m, n, k, 1, 1])
+    assert e.value.code == StatusCode.InvalidArgument

@@ -247,9 +247,9 @@ def test_w4a8_wmma_contract(backend, n, k, m, split):
     w8, wref = oracle.fold_mxfp4_to_fp8(w, n, k)
     folded = oracle.gemm_mxfp4_fp8(codes, scale, w8, wref, m, n, k)
     assert rel_err(got, folded) <= tol
-    with pytest.raises(StatusError) as e:   # pre-permuted weights are not part of this build
-        run(backend, "gemm_mxfp4_wmma", [da8, dw, das, dref, part], [m, n, k, split, 1])
-    assert e.value.code == StatusCode.UnsupportedFeature
+    with pytest.raises(StatusError) as e:   # wperm is 0 or 1
+        run(backend, "gemm_mxfp4_wmma", [da8, dw, das, dref, part], [m, n, k, split, 2])
+    assert e.value.code == StatusCode.InvalidArgument
 
 
 # rows longer than 16384 take the 32-weights-a-lane codec (17408: the dense down projection)

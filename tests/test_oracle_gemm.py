@@ -53,6 +53,21 @@ def test_mxfp4_dequant_and_gemm():
     assert err.value.code == 1
 
 
+def test_permute_mxfp4_to_wmma():
+    """The fragment-order permutation against an independent statement of it (an axis transpose of
+    the nibble bytes seen as [tile][row][k step][half][4 bytes]); the scales do not move."""
+    g = synth.rng(12)
+    n, k = 48, 96
+    w = synth.mxfp4_weights(g, n, k)
+    got = oracle.permute_mxfp4_to_wmma(w, n, k)
+    blob = w[: n * k // 2].reshape(n // 16, 16, k // 16, 2, 4)
+    assert np.array_equal(got[: n * k // 2], blob.transpose(0, 2, 3, 1, 4).reshape(-1))
+    assert np.array_equal(got[n * k // 2:], w[n * k // 2:])
+    assert sorted(got[: n * k // 2].tolist()) == sorted(w[: n * k // 2].tolist())
+    with pytest.raises(oracle.OracleError):
+        oracle.permute_mxfp4_to_wmma(synth.mxfp4_weights(g, 40, 96), 40, 96)     # rows not a multiple of 16
+
+
 def test_gemm_fp8():
     g = synth.rng(3)
     n, k = 12, 96

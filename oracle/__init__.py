@@ -64,6 +64,10 @@ def _load() -> C.CDLL:
         "orc_dequantize_mxfp4": (C.c_int, [u8p, f32p, sz, sz]),
         "orc_gemm_fp8_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
         "orc_permute_mxfp4_to_wmma": (C.c_int, [u8p, u8p, sz, sz]),
+        "orc_rope": (C.c_int, [f32p, sz, sz, sz, sz, C.c_uint64, C.c_double]),
+        "orc_mrope": (C.c_int, [f32p, C.POINTER(C.c_uint64), sz, sz, sz, sz, sz, sz, sz, C.c_double]),
+        "orc_attention": (C.c_int, [f32p, C.c_void_p, C.c_void_p, f32p, sz, sz, sz, sz, sz, C.c_uint64, sz, C.c_int, C.c_int]),
+        "orc_qgate_split": (C.c_int, [f32p, f32p, f32p, sz, sz, sz]),
         "orc_fold_entry": (C.c_uint8, [C.c_uint, C.c_uint]),
         "orc_fold_entry_rne": (C.c_uint8, [C.c_uint, C.c_uint]),
         "orc_fold_mxfp4_to_fp8": (C.c_int, [u8p, u8p, u8p, u8p, sz, sz]),
@@ -355,6 +359,40 @@ def embedding(kind: str, ids, table, rows: int, cols: int, vocab: int) -> np.nda
     _check(_lib.orc_embedding(code, _p(ids, C.c_uint32), table.ctypes.data_as(C.c_void_p), _p(out, C.c_float),
                               rows, cols, vocab))
     return out
+
+
+def rope(x, rows: int, heads: int, head_dim: int, rope_dim: int, pos_base: int, theta: float) -> np.ndarray:
+    io = _f32(x).reshape(-1).copy()
+    _check(_lib.orc_rope(_p(io, C.c_float), rows, heads, head_dim, rope_dim, pos_base, theta))
+    return io.reshape(rows, heads, head_dim)
+
+
+def mrope(x, pos, rows: int, heads: int, head_dim: int, rope_dim: int, sec_t: int, sec_h: int, sec_w: int,
+          theta: float) -> np.ndarray:
+    io = _f32(x).reshape(-1).copy()
+    pos = np.ascontiguousarray(pos, dtype=np.uint64).reshape(-1)
+    _check(_lib.orc_mrope(_p(io, C.c_float), _p(pos, C.c_uint64), rows, heads, head_dim, rope_dim, sec_t, sec_h, sec_w, theta))
+    return io.reshape(rows, heads, head_dim)
+
+
+def attention(q, k, v, m: int, n: int, heads: int, kv_heads: int, head_dim: int, q_base: int = 0, window: int = 0,
+              kv_f16: bool = False, causal: bool = True) -> np.ndarray:
+    """k, v: fp32 arrays, or float16 arrays when kv_f16."""
+    q = _f32(q).reshape(-1)
+    dt = np.float16 if kv_f16 else np.float32
+    k, v = np.ascontiguousarray(k, dtype=dt).reshape(-1), np.ascontiguousarray(v, dtype=dt).reshape(-1)
+    out = np.empty(m * heads * head_dim, dtype=np.float32)
+    _check(_lib.orc_attention(_p(q, C.c_float), k.ctypes.data_as(C.c_void_p), v.ctypes.data_as(C.c_void_p),
+                              _p(out, C.c_float), m, n, heads, kv_heads, head_dim, q_base, window, int(kv_f16), int(causal)))
+    return out.reshape(m, heads * head_dim)
+
+
+def qgate_split(fused, heads: int, head_dim: int, rows: int) -> tuple[np.ndarray, np.ndarray]:
+    fused = _f32(fused).reshape(-1)
+    q = np.empty(rows * heads * head_dim, dtype=np.float32)
+    g = np.empty_like(q)
+    _check(_lib.orc_qgate_split(_p(fused, C.c_float), _p(q, C.c_float), _p(g, C.c_float), heads, head_dim, rows))
+    return q, g
 
 
 def ffn_gate_up_silu_q4k(x, gate, up, m: int, n: int, k: int, threads: bool = False) -> np.ndarray:

@@ -35,6 +35,14 @@
  *                                             index; out-of-range ids give zero rows)
  *   silu_mul ................................ pinned (float64 evaluation within 2 ulp, silu(0) = 0,
  *                                             silu(x) - silu(-x) = x, large |x| limits)
+ *   MXFP4 fragment-order permutation ........ pinned (an axis transpose of the bytes, numpy)
+ *   rope / mrope ............................ pinned (complex multiplication by exp(i angle) in
+ *                                             float64, position 0 = identity, pair norms kept,
+ *                                             mrope with equal positions = rope)
+ *   attention (fp32 and fp16 keys/values) ... pinned (torch softmax(q k^T / sqrt(d)) v with the
+ *                                             causal / window mask built independently; one key =
+ *                                             its value row)
+ *   qgate_split ............................. pinned (numpy reshape)
  *
  * Status codes mirror tessera::StatusCode (include/tessera/types.hpp:36-48).
  */
@@ -748,6 +756,132 @@ int orc_embedding(int kind, const uint32_t* ids, const void* table, float* out, 
       for (size_t c = 0; c < cols; ++c) o[c] = bits_f32((uint32_t)t[c] << 16);
     } else {
       orc_dequantize_q4k_rows((const uint8_t*)table + id * (cols / 256) * 144, o, cols / 256);
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- rotary embedding in place, NeoX pairing (j, j + rope_dim/2) per head, angle
+ *      (pos_base + row) * theta^(-2j/rope_dim) in double, cos and sin rounded to fp32
+ *      (src/core/numerics/attention.cpp:11-44) ---- */
+int orc_rope(float* io, size_t rows, size_t heads, size_t head_dim, size_t rope_dim, uint64_t pos_base, double theta) {
+  if (rows == 0 || heads == 0 || head_dim == 0 || rope_dim == 0 || rope_dim > head_dim || rope_dim % 2 != 0 || !(theta > 0.0)) {
+    return ORC_INVALID_ARGUMENT;
+  }
+  const size_t half = rope_dim / 2;
+  for (size_t r = 0; r < rows; ++r) {
+    const double pos = (double)(pos_base + r);
+    for (size_t h = 0; h < heads; ++h) {
+      float* base = io + (r * heads + h) * head_dim;
+      for (size_t j = 0; j < half; ++j) {
+        const double angle = pos * pow(theta, -2.0 * (double)j / (double)rope_dim);
+        const float c = (float)cos(angle), s = (float)sin(angle);
+        const float x1 = base[j], x2 = base[j + half];
+        base[j] = x1 * c - x2 * s;
+        base[j + half] = x1 * s + x2 * c;
+      }
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- multimodal rotary embedding: pair j uses the temporal, height or width position of its
+ *      row by section (pairs past the sections reuse the width id)
+ *      (src/core/numerics/attention.cpp:227-264) ---- */
+int orc_mrope(float* io, const uint64_t* pos, size_t rows, size_t heads, size_t head_dim, size_t rope_dim,
+              size_t sec_t, size_t sec_h, size_t sec_w, double theta) {
+  if (rows == 0 || heads == 0 || head_dim == 0 || rope_dim == 0 || rope_dim > head_dim || rope_dim % 2 != 0 || !(theta > 0.0)) {
+    return ORC_INVALID_ARGUMENT;
+  }
+  const size_t pairs = rope_dim / 2;
+  if (sec_t + sec_h + sec_w > pairs) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    for (size_t h = 0; h < heads; ++h) {
+      float* base = io + (r * heads + h) * head_dim;
+      for (size_t j = 0; j < pairs; ++j) {
+        const uint64_t section_pos = j < sec_t ? pos[r * 3] : (j < sec_t + sec_h ? pos[r * 3 + 1] : pos[r * 3 + 2]);
+        const double angle = (double)section_pos * pow(theta, -2.0 * (double)j / (double)rope_dim);
+        const float c = (float)cos(angle), s = (float)sin(angle);
+        const float x1 = base[j], x2 = base[j + pairs];
+        base[j] = x1 * c - x2 * s;
+        base[j + pairs] = x1 * s + x2 * c;
+      }
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- softmax(q k^T / sqrt(head_dim)) v per query row and head, grouped kv heads; query row i
+ *      sits at position q_base + i and, when causal, attends keys max(0, pos + 1 - window) .. min(pos,
+ *      n - 1) (window 0 = all of the prefix); sequential fp32 fma dots, weights divided by the sum
+ *      before they multiply v (src/core/numerics/attention.cpp:158-225).  kv_f16: keys and values are
+ *      binary16 (AttentionRefF16, attention.cpp:128-156). ---- */
+int orc_attention(const float* q, const void* k, const void* v, float* out, size_t m, size_t n, size_t heads,
+                  size_t kv_heads, size_t head_dim, uint64_t q_base, size_t window, int kv_f16, int causal) {
+  if (m == 0 || n == 0 || heads == 0 || kv_heads == 0 || head_dim == 0 || heads % kv_heads != 0) return ORC_INVALID_ARGUMENT;
+  const size_t count = n * kv_heads * head_dim;
+  float* kf = (float*)malloc(count * sizeof(float));
+  float* vf = (float*)malloc(count * sizeof(float));
+  float* scores = (float*)malloc(n * sizeof(float));
+  if (!kf || !vf || !scores) {
+    free(kf), free(vf), free(scores);
+    return ORC_OOM;
+  }
+  for (size_t i = 0; i < count; ++i) {
+    kf[i] = kv_f16 ? orc_fp16_to_float(((const uint16_t*)k)[i]) : ((const float*)k)[i];
+    vf[i] = kv_f16 ? orc_fp16_to_float(((const uint16_t*)v)[i]) : ((const float*)v)[i];
+  }
+  const size_t group = heads / kv_heads;
+  const float scale = 1.0f / sqrtf((float)head_dim);
+  for (size_t i = 0; i < m; ++i) {
+    const size_t pos = (size_t)(q_base + i);
+    const size_t last = causal ? (pos >= n ? n - 1 : pos) : n - 1;
+    size_t start = 0;
+    if (causal) {
+      start = window != 0 && pos + 1 > window ? pos + 1 - window : 0;
+      if (start > last) start = last;
+    }
+    for (size_t h = 0; h < heads; ++h) {
+      const size_t kv = h / group;
+      const float* q_row = q + (i * heads + h) * head_dim;
+      float row_max = 0.0f;
+      int first = 1;
+      for (size_t j = start; j <= last; ++j) {
+        const float* k_row = kf + (j * kv_heads + kv) * head_dim;
+        float dot = 0.0f;
+        for (size_t e = 0; e < head_dim; ++e) dot = fmaf(q_row[e], k_row[e], dot);
+        dot *= scale;
+        scores[j] = dot;
+        if (first || dot > row_max) row_max = dot, first = 0;
+      }
+      float denom = 0.0f;
+      for (size_t j = start; j <= last; ++j) {
+        scores[j] = expf(scores[j] - row_max);
+        denom += scores[j];
+      }
+      float* o_row = out + (i * heads + h) * head_dim;
+      for (size_t e = 0; e < head_dim; ++e) {
+        float acc = 0.0f;
+        for (size_t j = start; j <= last; ++j) acc = fmaf(scores[j] / denom, vf[(j * kv_heads + kv) * head_dim + e], acc);
+        o_row[e] = acc;
+      }
+    }
+  }
+  free(kf), free(vf), free(scores);
+  return ORC_OK;
+}
+
+/* ---- fused gated-attention projection (rows x heads x [query | gate]) -> queries, gates
+ *      (src/core/numerics/attention.cpp:287-309) ---- */
+int orc_qgate_split(const float* fused, float* q, float* gate, size_t heads, size_t head_dim, size_t rows) {
+  if (heads == 0 || head_dim == 0 || rows == 0) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    for (size_t h = 0; h < heads; ++h) {
+      const float* src = fused + (r * heads + h) * 2 * head_dim;
+      for (size_t e = 0; e < head_dim; ++e) {
+        q[(r * heads + h) * head_dim + e] = src[e];
+        gate[(r * heads + h) * head_dim + e] = src[head_dim + e];
+      }
     }
   }
   return ORC_OK;

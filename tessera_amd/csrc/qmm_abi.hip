@@ -327,6 +327,71 @@ qmm_status run_rmsnorm(const LaunchCtx& c) {
   return map_hip(qmm::launch_rmsnorm(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<float>(2), rows, cols, eps, c.stream));
 }
 
+// "rope": buffer X (rows x heads x head_dim fp32, rotated in place); scalars rows, heads, head_dim,
+// rope_dim, pos_base, fp32 bits of theta (include/tessera/backend.hpp:162-166,417-428).
+// "mrope": buffers X, Pos (rows x 3 u64: temporal, height, width); scalars rows, heads, head_dim,
+// rope_dim, fp32 bits of theta, sec_t, sec_h, sec_w (backend.hpp:378-385,805-818).
+qmm_status run_rope_common(const LaunchCtx& c, bool multimodal) {
+  if (!counts(c, multimodal ? 2 : 1, multimodal ? 8 : 6)) return bad("rope/mrope: wrong number of buffers or scalars");
+  const uint64_t rows = c.sc[0], heads = c.sc[1], head_dim = c.sc[2], rope_dim = c.sc[3];
+  if (rows == 0 || heads == 0 || head_dim == 0 || rope_dim == 0 || rope_dim > head_dim || head_dim % 2 != 0 || rope_dim % 2 != 0 ||
+      rows > (1u << 30) || heads > (1u << 20) || head_dim > (1u << 20)) {
+    return bad("rope/mrope: rows, heads, head_dim, rope_dim must be non-zero, the dims even, rope_dim <= head_dim");
+  }
+  const uint64_t sec_t = multimodal ? c.sc[5] : 0, sec_h = multimodal ? c.sc[6] : 0, sec_w = multimodal ? c.sc[7] : 0;
+  if (multimodal && (sec_t > rope_dim || sec_h > rope_dim || sec_w > rope_dim || sec_t + sec_h + sec_w > rope_dim / 2)) {
+    return bad("mrope: the sections hold more pairs than rope_dim / 2");
+  }
+  if (!c.fits(0, static_cast<u128>(rows) * heads * head_dim * 4) || (multimodal && !c.fits(1, static_cast<u128>(rows) * 24))) {
+    return bad("rope/mrope: a buffer is smaller than rows, heads, head_dim require");
+  }
+  const uint32_t theta_bits = static_cast<uint32_t>(c.sc[multimodal ? 4 : 5]);
+  float theta;
+  std::memcpy(&theta, &theta_bits, 4);
+  if (!(theta > 0.0f)) return bad("rope/mrope: theta must be positive");
+  return map_hip(qmm::launch_rope(c.ptr<float>(0), multimodal ? c.ptr<const uint64_t>(1) : nullptr, rows, heads, head_dim, rope_dim,
+                                  multimodal ? 0 : c.sc[4], theta, sec_t, sec_h, c.stream));
+}
+qmm_status run_rope(const LaunchCtx& c) { return run_rope_common(c, false); }
+qmm_status run_mrope(const LaunchCtx& c) { return run_rope_common(c, true); }
+
+// "attention": buffers Q (rows x heads*head_dim fp32), K, V (n x kv_heads*head_dim, fp32 or fp16), Out
+// (as Q); scalars m, n, heads, kv_heads, head_dim, q_base, row_base, window, kv_f16, causal
+// (include/tessera/backend.hpp:167-179,429-440).  Q and Out hold at least row_base + m rows.
+qmm_status run_attention(const LaunchCtx& c) {
+  if (!counts(c, 4, 10)) return bad("attention: expects 4 buffers and 10 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], heads = c.sc[2], kv_heads = c.sc[3], head_dim = c.sc[4], q_base = c.sc[5],
+                 row_base = c.sc[6], window = c.sc[7], kv_f16 = c.sc[8], causal = c.sc[9];
+  if (m == 0 || n == 0 || heads == 0 || kv_heads == 0 || head_dim == 0 || heads % kv_heads != 0) {
+    return bad("attention: m, n, heads, kv_heads, head_dim must be non-zero and heads a multiple of kv_heads");
+  }
+  if (head_dim > 256) return bad("attention: head_dim must be at most 256");
+  if (m > (1u << 24) || n > (1ull << 32) || heads > (1u << 16) || row_base > (1ull << 32) || q_base > (1ull << 40) ||
+      m * heads > 0x7FFFFFFFull || kv_f16 > 1 || causal > 1) {
+    return bad("attention: a scalar is out of range");
+  }
+  const u128 q_bytes = static_cast<u128>(row_base + m) * heads * head_dim * 4;
+  const u128 kv_bytes = static_cast<u128>(n) * kv_heads * head_dim * (kv_f16 ? 2 : 4);
+  if (!c.fits(0, q_bytes) || !c.fits(1, kv_bytes) || !c.fits(2, kv_bytes) || !c.fits(3, q_bytes)) {
+    return bad("attention: a buffer is smaller than the scalars require");
+  }
+  return map_hip(qmm::launch_attention(c.ptr<const float>(0), c.ptr<const void>(1), c.ptr<const void>(2), c.ptr<float>(3), m, n,
+                                       heads, kv_heads, head_dim, q_base, row_base, window, kv_f16 == 1, causal == 1, c.stream));
+}
+
+// "qgate_split": buffers Fused (rows x heads x 2*head_dim: per head the query then the gate), Q, G
+// (rows x heads*head_dim each); scalars heads, head_dim, rows (include/tessera/backend.hpp:386-390,819-826).
+qmm_status run_qgate_split(const LaunchCtx& c) {
+  if (!counts(c, 3, 3)) return bad("qgate_split: expects 3 buffers and 3 scalars");
+  const uint64_t heads = c.sc[0], head_dim = c.sc[1], rows = c.sc[2];
+  if (heads == 0 || head_dim == 0 || rows == 0 || heads > (1u << 20) || head_dim > (1u << 20) || rows > (1u << 30)) {
+    return bad("qgate_split: heads, head_dim and rows must be non-zero");
+  }
+  const u128 part = static_cast<u128>(rows) * heads * head_dim * 4;
+  if (!c.fits(0, part * 2) || !c.fits(1, part) || !c.fits(2, part)) return bad("qgate_split: a buffer is smaller than the scalars require");
+  return map_hip(qmm::launch_qgate_split(c.ptr<const float>(0), c.ptr<float>(1), c.ptr<float>(2), heads, head_dim, rows, c.stream));
+}
+
 // "embedding_f32", "embedding_bf16", "embedding_q4k": buffers ids (u32, rows), table (vocab x cols),
 // Out (fp32 rows x cols); scalars rows, cols, vocab (include/tessera/backend.hpp:260-265,827-839).
 qmm_status run_embedding(const LaunchCtx& c, int kind) {
@@ -931,6 +996,10 @@ const Entry kTable[] = {
     {"fill", run_fill},
     {"read_probe", run_read_probe},
     {"rmsnorm", run_rmsnorm},
+    {"rope", run_rope},
+    {"mrope", run_mrope},
+    {"attention", run_attention},
+    {"qgate_split", run_qgate_split},
     {"embedding_f32", run_embedding_f32},
     {"embedding_bf16", run_embedding_bf16},
     {"embedding_q4k", run_embedding_q4k},

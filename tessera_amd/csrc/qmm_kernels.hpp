@@ -164,4 +164,14 @@ hipError_t launch_top_k_rows(const float* logits, uint32_t* ids, float* vals, ui
 hipError_t launch_moe_scale_add(const float* a, const float* b, const float* f, float* o,
                                 uint64_t n, uint64_t idx, hipStream_t stream);
 
+// ---- non-matmul trunk pieces (trunk.hip) ---------------------------------------
+// pos3 null: "rope" (positions pos_base + row); else "mrope" (per-row (t, h, w) triples, section sizes).
+hipError_t launch_rope(float* data, const uint64_t* pos3, uint64_t rows, uint64_t heads, uint64_t head_dim, uint64_t rope_dim,
+                       uint64_t pos_base, float theta, uint64_t sec_t, uint64_t sec_h, hipStream_t stream);
+hipError_t launch_attention(const float* q, const void* k, const void* v, float* out, uint64_t m, uint64_t n, uint64_t heads,
+                            uint64_t kv_heads, uint64_t head_dim, uint64_t q_base, uint64_t row_base, uint64_t window,
+                            bool kv_f16, bool causal, hipStream_t stream);
+hipError_t launch_qgate_split(const float* fused, float* q, float* gate, uint64_t heads, uint64_t head_dim, uint64_t rows,
+                              hipStream_t stream);
+
 }  // namespace qmm

@@ -1,0 +1,149 @@
+// The non-matmul pieces of a transformer block that sit between the projections, as plain correct
+// kernels so that a trunk can run on this backend end to end: rotary embeddings, softmax attention
+// over a key/value cache, the query/gate split of gated attention.  Contracts:
+// include/tessera/backend.hpp:162-179,378-390; CPU statements src/core/numerics/attention.cpp.
+// None of them is tuned: they move kilobytes where the projections move megabytes.
+
+#include "qmm_device.hpp"
+#include "qmm_kernels.hpp"
+
+namespace qmm {
+namespace {
+
+// One thread per (row, head, pair): (x[j], x[j + pairs]) rotated by pos * theta^(-2j / rope_dim).
+// The angle, its cosine and sine are formed in double and rounded to fp32 once, as RopeRef does
+// (src/core/numerics/attention.cpp:11-44); `pos3` non-null selects the multimodal form, where pair
+// j takes the temporal, height or width position of its row (MropeRef, attention.cpp:227-264).
+__global__ __launch_bounds__(256) void rope_kernel(float* __restrict__ data, const uint64_t* __restrict__ pos3, uint64_t rows,
+                                                   uint64_t heads, uint64_t head_dim, uint64_t rope_dim, uint64_t pos_base,
+                                                   float theta, uint64_t sec_t, uint64_t sec_h) {
+  const uint64_t pairs = rope_dim / 2;
+  const uint64_t t = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (t >= rows * heads * pairs) return;
+  const uint64_t row = t / (heads * pairs), rem = t % (heads * pairs), head = rem / pairs, j = rem % pairs;
+  uint64_t p = pos_base + row;
+  if (pos3 != nullptr) p = pos3[row * 3 + (j < sec_t ? 0 : (j < sec_t + sec_h ? 1 : 2))];
+  const double angle = static_cast<double>(p) * pow(static_cast<double>(theta), -2.0 * static_cast<double>(j) / static_cast<double>(rope_dim));
+  const float c = static_cast<float>(cos(angle)), s = static_cast<float>(sin(angle));
+  float* base = data + (row * heads + head) * head_dim;
+  const float x1 = base[j], x2 = base[j + pairs];
+  base[j] = x1 * c - x2 * s;
+  base[j + pairs] = x1 * s + x2 * c;
+}
+
+// One workgroup of four wavefronts per (query row, head).  Keys are taken 64 at a time: a
+// wavefront forms the score of a key with its lanes across head_dim (coalesced key reads, a DPP
+// sum), the first wavefront turns the 64 scores into weights against the running maximum, and
+// thread e accumulates weight * v[key][e] (coalesced value reads): the usual running softmax, so
+// the result differs from AttentionRef (src/core/numerics/attention.cpp:158-225) in summation
+// order only.
+template <bool F16>
+__global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ q, const void* __restrict__ k,
+                                                        const void* __restrict__ v, float* __restrict__ out, uint64_t n,
+                                                        uint64_t heads, uint64_t kv_heads, uint64_t head_dim, uint64_t q_base,
+                                                        uint64_t row_base, uint64_t window, uint64_t causal) {
+  constexpr uint32_t kKeys = 64;
+  __shared__ float sc[kKeys], wt[kKeys], bc[2];
+  const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+  const uint64_t i = blockIdx.x / heads, h = blockIdx.x % heads, kv = h / (heads / kv_heads);
+  const uint64_t pos = q_base + i;
+  const uint64_t last = causal != 0 ? (pos >= n ? n - 1 : pos) : n - 1;
+  uint64_t start = 0;
+  if (causal != 0) {
+    start = (window != 0 && pos + 1 > window) ? pos + 1 - window : 0;
+    if (start > last) start = last;
+  }
+  const float scale = 1.0f / sqrtf(static_cast<float>(head_dim));
+  const uint64_t qb = ((row_base + i) * heads + h) * head_dim;
+  auto kv_at = [&](const void* base, uint64_t idx) {
+    if constexpr (F16) return half_bits_to_float(static_cast<const uint16_t*>(base)[idx]);
+    else return static_cast<const float*>(base)[idx];
+  };
+  float qr[4];                       // head_dim <= 256: up to four elements a lane
+#pragma unroll
+  for (int cc = 0; cc < 4; ++cc) qr[cc] = lane + 64u * cc < head_dim ? q[qb + lane + 64u * cc] : 0.0f;
+
+  float run_max = -INFINITY, run_sum = 0.0f, acc = 0.0f;
+  for (uint64_t j0 = start; j0 <= last; j0 += kKeys) {
+    const uint32_t count = last - j0 + 1 < kKeys ? static_cast<uint32_t>(last - j0 + 1) : kKeys;
+    for (uint32_t kk = wave; kk < kKeys; kk += 4u) {
+      float dot = 0.0f;
+      if (kk < count) {
+        const uint64_t kb = ((j0 + kk) * kv_heads + kv) * head_dim;
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+          if (lane + 64u * cc < head_dim) dot = fmaf(qr[cc], kv_at(k, kb + lane + 64u * cc), dot);
+        }
+      }
+      dot = wave_sum(dot);
+      if (lane == 0) sc[kk] = kk < count ? dot * scale : -INFINITY;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const float s = sc[lane];
+      const float m_new = fmaxf(run_max, wave_max(s));
+      const float w = lane < count ? expf(s - m_new) : 0.0f;
+      wt[lane] = w;
+      const float l = wave_sum(w);
+      if (lane == 0) {
+        bc[0] = m_new;
+        bc[1] = l;
+      }
+    }
+    __syncthreads();
+    const float m_new = bc[0];
+    const float corr = expf(run_max - m_new);      // 0 on the first tile (run_max = -inf)
+    run_sum = fmaf(corr, run_sum, bc[1]);
+    run_max = m_new;
+    if (t < head_dim) {
+      float a = 0.0f;
+      for (uint32_t kk = 0; kk < count; ++kk) a = fmaf(wt[kk], kv_at(v, ((j0 + kk) * kv_heads + kv) * head_dim + t), a);
+      acc = fmaf(corr, acc, a);
+    }
+    __syncthreads();
+  }
+  if (t < head_dim) out[qb + t] = acc / run_sum;
+}
+
+__global__ __launch_bounds__(256) void qgate_split_kernel(const float* __restrict__ fused, float* __restrict__ q,
+                                                          float* __restrict__ gate, uint64_t head_dim, uint64_t total) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (i >= total) return;
+  const uint64_t rh = i / head_dim, e = i % head_dim;
+  q[i] = fused[rh * 2 * head_dim + e];
+  gate[i] = fused[rh * 2 * head_dim + head_dim + e];
+}
+
+dim3 blocks_for(uint64_t count) { return dim3(static_cast<uint32_t>((count + 255) / 256)); }
+
+}  // namespace
+
+hipError_t launch_rope(float* data, const uint64_t* pos3, uint64_t rows, uint64_t heads, uint64_t head_dim, uint64_t rope_dim,
+                       uint64_t pos_base, float theta, uint64_t sec_t, uint64_t sec_h, hipStream_t stream) {
+  hipLaunchKernelGGL(rope_kernel, blocks_for(rows * heads * (rope_dim / 2)), dim3(256), 0, stream, data, pos3, rows, heads,
+                     head_dim, rope_dim, pos_base, theta, sec_t, sec_h);
+  return hipGetLastError();
+}
+
+hipError_t launch_attention(const float* q, const void* k, const void* v, float* out, uint64_t m, uint64_t n, uint64_t heads,
+                            uint64_t kv_heads, uint64_t head_dim, uint64_t q_base, uint64_t row_base, uint64_t window,
+                            bool kv_f16, bool causal, hipStream_t stream) {
+  const dim3 grid(static_cast<uint32_t>(m * heads));
+  if (kv_f16) {
+    hipLaunchKernelGGL(attention_kernel<true>, grid, dim3(256), 0, stream, q, k, v, out, n, heads, kv_heads, head_dim, q_base,
+                       row_base, window, causal ? 1ull : 0ull);
+  } else {
+    hipLaunchKernelGGL(attention_kernel<false>, grid, dim3(256), 0, stream, q, k, v, out, n, heads, kv_heads, head_dim, q_base,
+                       row_base, window, causal ? 1ull : 0ull);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_qgate_split(const float* fused, float* q, float* gate, uint64_t heads, uint64_t head_dim, uint64_t rows,
+                              hipStream_t stream) {
+  const uint64_t total = rows * heads * head_dim;
+  hipLaunchKernelGGL(qgate_split_kernel, blocks_for(total), dim3(256), 0, stream, fused, q, gate, head_dim, total);
+  return hipGetLastError();
+}
+
+}  // namespace qmm

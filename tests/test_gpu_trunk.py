@@ -1,0 +1,102 @@
+"""The non-matmul trunk ids that sit between the projections (rope, mrope, attention, qgate_split;
+contracts include/tessera/backend.hpp:162-179,378-390) against the oracle's restatements of
+RopeRef / MropeRef / AttentionRef / QGateSplitRef (src/core/numerics/attention.cpp).  Plain
+correct kernels: rope forms its angles in double as the CPU reference does (the reference's own
+device kernel uses fp32 powf/cosf/sinf), attention is a running softmax, so it differs from the
+reference in summation order only (bound 2e-6 of the largest output)."""
+import numpy as np
+import pytest
+
+import oracle
+from tessera_amd import StatusCode, StatusError, synth
+from util import run
+
+pytestmark = pytest.mark.gpu
+
+
+def f32_bits(x):
+    return int(np.float32(x).view(np.uint32))
+
+
+@pytest.mark.parametrize("rows,heads,head_dim,rope_dim,pos_base,theta", [(5, 3, 64, 64, 0, 1e4), (33, 8, 128, 64, 100000, 1e6),
+                                                                          (1, 1, 8, 2, 7, 10.0), (300, 2, 256, 256, 5, 1e4)])
+def test_rope(backend, rows, heads, head_dim, rope_dim, pos_base, theta):
+    g = synth.rng(rows + head_dim)
+    x = g.standard_normal((rows, heads, head_dim)).astype(np.float32)
+    want = oracle.rope(x, rows, heads, head_dim, rope_dim, pos_base, float(np.float32(theta)))
+    dx = backend.Upload(x)
+    run(backend, "rope", [dx], [rows, heads, head_dim, rope_dim, pos_base, f32_bits(theta)],
+        grid=((rows * heads * (rope_dim // 2) + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dx, dtype=np.float32).reshape(rows, heads, head_dim)
+    # cos and sin may differ by one fp32 unit in the last place between the host's and the device's libm
+    assert np.max(np.abs(got - want)) <= 3e-7 * np.max(np.abs(x))
+    assert np.array_equal(got[..., rope_dim:], x[..., rope_dim:])
+
+
+def test_mrope(backend):
+    g = synth.rng(3)
+    rows, heads, head_dim, rope_dim, theta = 40, 4, 128, 96, 1e4
+    x = g.standard_normal((rows, heads, head_dim)).astype(np.float32)
+    pos = g.integers(0, 5000, size=(rows, 3)).astype(np.uint64)
+    sec = (20, 16, 8)
+    want = oracle.mrope(x, pos, rows, heads, head_dim, rope_dim, *sec, theta)
+    dx, dp = backend.Upload(x), backend.Upload(pos)
+    run(backend, "mrope", [dx, dp], [rows, heads, head_dim, rope_dim, f32_bits(theta), *sec],
+        grid=((rows * heads * (rope_dim // 2) + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dx, dtype=np.float32).reshape(rows, heads, head_dim)
+    assert np.max(np.abs(got - want)) <= 3e-7 * np.max(np.abs(x))
+    with pytest.raises(StatusError) as e:
+        run(backend, "mrope", [dx, dp], [rows, heads, head_dim, rope_dim, f32_bits(theta), 40, 8, 1])
+    assert e.value.code == StatusCode.InvalidArgument
+
+
+@pytest.mark.parametrize("m,n,heads,kv_heads,head_dim,q_base,window,kv_f16,causal", [
+    (5, 12, 4, 2, 32, 7, 0, 0, 1), (3, 400, 8, 8, 64, 397, 16, 0, 1), (6, 9, 2, 1, 128, 0, 0, 1, 1),
+    (4, 300, 4, 4, 16, 0, 0, 0, 0), (2, 5, 2, 2, 8, 20, 3, 1, 1), (1, 1000, 24, 4, 256, 999, 0, 1, 1),
+    (7, 130, 6, 2, 100, 60, 0, 0, 1)])
+def test_attention(backend, m, n, heads, kv_heads, head_dim, q_base, window, kv_f16, causal):
+    g = synth.rng(m * 100 + n)
+    q = g.standard_normal((m, heads * head_dim)).astype(np.float32)
+    k = g.standard_normal((n, kv_heads * head_dim)).astype(np.float32)
+    v = g.standard_normal((n, kv_heads * head_dim)).astype(np.float32)
+    if kv_f16:
+        k, v = k.astype(np.float16), v.astype(np.float16)
+    want = oracle.attention(q, k, v, m, n, heads, kv_heads, head_dim, q_base, window, bool(kv_f16), bool(causal))
+    # the rows of this sequence sit at row_base inside a larger batch buffer; its other rows stay as they are
+    row_base, total = 2, m + 5
+    qbuf = np.zeros((total, heads * head_dim), np.float32)
+    qbuf[row_base:row_base + m] = q
+    dq, dk, dv = backend.Upload(qbuf), backend.Upload(k), backend.Upload(v)
+    dout = backend.Upload(np.full((total, heads * head_dim), 7.0, np.float32))
+    run(backend, "attention", [dq, dk, dv, dout], [m, n, heads, kv_heads, head_dim, q_base, row_base, window, kv_f16, causal],
+        grid=(m * heads, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dout, dtype=np.float32).reshape(total, heads * head_dim)
+    assert np.max(np.abs(got[row_base:row_base + m] - want)) <= 2e-6 * max(1.0, np.max(np.abs(want)))
+    assert np.all(got[:row_base] == 7.0) and np.all(got[row_base + m:] == 7.0)
+
+
+def test_attention_argument_errors(backend):
+    b = [backend.AllocateBuffer(1 << 16) for _ in range(4)]
+    for scalars in ([1, 4, 3, 2, 16, 0, 0, 0, 0, 1],       # heads not a multiple of kv_heads
+                    [1, 4, 2, 2, 512, 0, 0, 0, 0, 1],      # head_dim above 256
+                    [0, 4, 2, 2, 16, 0, 0, 0, 0, 1],       # no rows
+                    [1, 1 << 20, 2, 2, 64, 0, 0, 0, 0, 1]):  # keys beyond the buffer
+        with pytest.raises(StatusError) as e:
+            run(backend, "attention", b, scalars)
+        assert e.value.code == StatusCode.InvalidArgument
+
+
+def test_qgate_split(backend):
+    g = synth.rng(10)
+    rows, heads, head_dim = 37, 6, 72
+    fused = g.standard_normal((rows, heads, 2, head_dim)).astype(np.float32)
+    df = backend.Upload(fused)
+    dq, dg = backend.AllocateBuffer(4 * rows * heads * head_dim), backend.AllocateBuffer(4 * rows * heads * head_dim)
+    run(backend, "qgate_split", [df, dq, dg], [heads, head_dim, rows], grid=((rows * heads * head_dim + 255) // 256, 1, 1))
+    backend.Synchronize()
+    want_q, want_g = oracle.qgate_split(fused, heads, head_dim, rows)
+    assert np.array_equal(backend.CopyD2H(dq, dtype=np.float32), want_q)
+    assert np.array_equal(backend.CopyD2H(dg, dtype=np.float32), want_g)

@@ -31,7 +31,6 @@
 // inside this kernel was measured four times slower: the device-scope release and acquire it needs
 // write back and invalidate the L2 of its XCD under the workgroups still streaming weights.)
 
-#include <atomic>
 #include <type_traits>
 
 #include "qmm_device.hpp"
@@ -373,6 +372,18 @@ size_t gemv_q4k_rows16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k) {
   return static_cast<size_t>(pl.parts) * m * n * 4;
 }
 
+// The kernels ask for more dynamic LDS than the default limit allows; the limit is raised once, at
+// library initialisation (not inside a launch, which may be under stream capture).
+hipError_t gemv_q4k_rows16_prepare() {
+  const void* kernels[3] = {reinterpret_cast<const void*>(q4k_rows16_kernel<1, 1>), reinterpret_cast<const void*>(q4k_rows16_kernel<1, 2>),
+                            reinterpret_cast<const void*>(q4k_rows16_kernel<2, 1>)};
+  for (const void* kern : kernels) {
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,
                              uint32_t k, hipStream_t stream) {
   R16Plan pl;
@@ -380,22 +391,12 @@ hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* w
   R16Args args{a, w, c, static_cast<float*>(workspace), m, n, k, pl.tiles_per_wg, static_cast<uint32_t>(k / 256) / pl.parts};
   const dim3 grid(pl.row_groups, pl.parts), block(64 * pl.waves);
   const uint32_t lds = r16_lds_bytes(pl.waves, pl.mt, pl.bw);
-  hipError_t e = hipSuccess;
-  // The dynamic LDS limit of a kernel is raised once per process (not a stream operation).
-  static std::atomic<bool> raised[3] = {};
-  auto go = [&](auto kernel, int which) {
-    if (!raised[which].load(std::memory_order_acquire)) {
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
-      if (e != hipSuccess) return;
-      raised[which].store(true, std::memory_order_release);
-    }
-    hipLaunchKernelGGL(kernel, grid, block, lds, stream, args);
-  };
-  if (pl.mt == 2) go(q4k_rows16_kernel<2, 1>, 0);
-  else if (pl.bw == 1) go(q4k_rows16_kernel<1, 1>, 1);
-  else go(q4k_rows16_kernel<1, 2>, 2);
+  auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, lds, stream, args); };
+  if (pl.mt == 2) go(q4k_rows16_kernel<2, 1>);
+  else if (pl.bw == 1) go(q4k_rows16_kernel<1, 1>);
+  else go(q4k_rows16_kernel<1, 2>);
+  const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  if ((e = hipGetLastError()) != hipSuccess) return e;
   if (pl.parts > 1) return launch_vec_reduce(args.ws, c, static_cast<uint64_t>(m) * n, pl.parts, stream);
   return hipSuccess;
 }

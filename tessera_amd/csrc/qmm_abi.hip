@@ -1080,6 +1080,10 @@ qmm_status qmm_init(int device) {
     }
     g_static_scratch[device] = p;
   }
+  if ((e = qmm::gemv_q4k_rows16_prepare()) != hipSuccess) {
+    g_device = -1;
+    return map_hip(e);
+  }
   if (g_decode_scratch == nullptr) {
     if ((e = hipMalloc(&g_decode_scratch, kDecodeScratchBytes)) != hipSuccess) {
       g_decode_scratch = nullptr;

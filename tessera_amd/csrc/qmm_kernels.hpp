@@ -128,6 +128,7 @@ hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
 
 // Q4_K x 2..16 activation rows in one pass over the weights on the 16x16x32 fp16 MFMA, exact on the
 // weight side (gemv_q4k_rows16.hip).  `workspace` holds the K parts' output regions.
+hipError_t gemv_q4k_rows16_prepare();   // once per device, from qmm_init
 bool gemv_q4k_rows16_supported(uint64_t m, uint64_t n, uint64_t k);
 size_t gemv_q4k_rows16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k);
 hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,

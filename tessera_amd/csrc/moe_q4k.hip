@@ -1,0 +1,701 @@
+// Routed experts (Q4_K) for a chunk of tokens, grouped by expert: every expert's weights are
+// streamed once for all the tokens routed to it (reference per-row kernels:
+// src/backends/rocm/rocm_kernels_moe.cpp:15-79; caller src/models/qwen3_5/moe.cpp:396-423).
+
+#include "q4k_tile.hpp"
+#include "qmm_kernels.hpp"
+
+namespace qmm {
+namespace {
+
+// Grouped form for routed experts: segment e multiplies rows seg[e]..seg[e+1] of a16
+// by expert e's weights (w + e * w_stride) into the same rows of c.  Segment bounds live in
+// device memory (the routing is computed on the device); an empty segment leaves at once.
+template <int BM, int BN>
+__global__ __launch_bounds__(BN * 2) void q4k_gemm_grouped_kernel(
+    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ w,
+    float* __restrict__ c, const uint32_t* __restrict__ seg, uint64_t w_stride, uint32_t n, uint32_t k,
+    uint32_t experts, uint32_t tensors, const uint8_t* __restrict__ w2, float* __restrict__ c2, uint64_t w2_stride) {
+  // One-dimensional grid, decoded so that an expert's activation rows are fetched from HBM once:
+  // workgroups are dealt to the eight XCDs (one L2 each) by linear index, so the expert's low three
+  // bits are the index's low three bits (all its tiles on one XCD), and its column tiles of both
+  // tensors follow each other in dispatch order (its rows are still in that L2 when the next tile
+  // asks for them).  `tensors` = 2 runs a second expert tensor of the same shape against the same
+  // rows (gate and up in one launch).
+  const uint32_t tiles = (n + BN - 1) / BN;
+  const uint32_t slot = blockIdx.x / 8u, per_expert = tiles * tensors;
+  const uint32_t e = (slot / per_expert) * 8u + blockIdx.x % 8u;
+  const uint32_t tz = slot % per_expert, tile = tz % tiles;
+  if (e >= experts) return;
+  if (tz >= tiles) w = w2, c = c2, w_stride = w2_stride;
+  const uint32_t r0 = seg[e], r1 = seg[e + 1];
+  if (r1 <= r0) return;
+  const _Float16* a_e = a16 + static_cast<size_t>(r0) * k;
+  const uint8_t* w_e = w + e * w_stride;
+  float* c_e = c + static_cast<size_t>(r0) * n;
+  for (uint32_t m0 = 0; m0 < r1 - r0; m0 += BM) {
+    q4k_gemm_tile<BM, BN, BM, 32>(a_e, a_scale + r0, w_e, c_e, r1 - r0, n, k, m0, tile * BN, n);
+  }
+}
+
+}  // namespace
+
+// ---- routed experts, a whole chunk of tokens grouped by expert -----------------------------
+// (token, slot) pairs are sorted by expert so that each expert's weights are streamed once for
+// all the tokens routed to it, and the three projections run as grouped MFMA GEMMs.
+namespace {
+
+// seg[e] = first sorted position of expert e (seg[experts] = pairs); pos[p] = sorted position
+// of pair p; inv[pos[p]] = p.  Counting sort with LDS atomics: which position inside its expert's
+// segment a pair gets depends on the order the atomics land in, but a row's result does not
+// depend on where the row sits, so the outputs are the same on every run.  One workgroup of 1024.
+__device__ __forceinline__ void moe_sort_pairs(const uint32_t* __restrict__ ids, uint32_t pairs, uint32_t experts,
+                                               uint32_t* __restrict__ seg, uint32_t* __restrict__ pos,
+                                               uint32_t* __restrict__ inv) {
+  __shared__ uint32_t cursor[1024], wave_total[16];
+  const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+  cursor[t] = 0;
+  __syncthreads();
+  for (uint32_t p = t; p < pairs; p += 1024u) {
+    const uint32_t id = ids[p] < experts ? ids[p] : experts - 1u;   // a bad id cannot leave the tensor
+    atomicAdd(&cursor[id], 1u);
+  }
+  __syncthreads();
+  // exclusive prefix sum of the 1024 counts: inside each wavefront, then over the 16 totals
+  const uint32_t count = cursor[t];
+  uint32_t run = count;
+#pragma unroll
+  for (uint32_t d = 1; d < 64u; d *= 2u) {
+    const uint32_t below = __shfl_up(run, d);
+    if (lane >= d) run += below;
+  }
+  if (lane == 63u) wave_total[wave] = run;
+  __syncthreads();
+  uint32_t base = 0;
+  for (uint32_t w = 0; w < wave; ++w) base += wave_total[w];
+  const uint32_t first = base + run - count;
+  __syncthreads();
+  cursor[t] = first;
+  if (t < experts) seg[t] = first;
+  if (t == experts - 1u) seg[experts] = first + count;
+  __syncthreads();
+  for (uint32_t p = t; p < pairs; p += 1024u) {
+    const uint32_t id = ids[p] < experts ? ids[p] : experts - 1u;
+    const uint32_t at = atomicAdd(&cursor[id], 1u);
+    pos[p] = at;
+    inv[at] = p;
+  }
+}
+
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restrict__ ids, uint32_t pairs,
+                                                        uint32_t experts, uint32_t* __restrict__ seg,
+                                                        uint32_t* __restrict__ pos, uint32_t* __restrict__ inv) {
+  moe_sort_pairs(ids, pairs, experts, seg, pos, inv);
+}
+
+// The sort and the fp16 copy of the token rows do not depend on each other: workgroup 0 sorts,
+// workgroup 1 + r converts row r of x (as rows_to_f16_kernel does: divided by the row's
+// power-of-two scale, groups of 8 in the order the weight decode yields).
+__global__ __launch_bounds__(1024) void moe_prepare_kernel(const uint32_t* __restrict__ ids, uint32_t pairs,
+                                                           uint32_t experts, uint32_t* __restrict__ seg,
+                                                           uint32_t* __restrict__ pos, uint32_t* __restrict__ inv,
+                                                           const float* __restrict__ x, _Float16* __restrict__ a16,
+                                                           float* __restrict__ a_scale, uint32_t cols) {
+  if (blockIdx.x == 0) {
+    moe_sort_pairs(ids, pairs, experts, seg, pos, inv);
+    return;
+  }
+  __shared__ float red[16];
+  const uint32_t row = blockIdx.x - 1u, t = threadIdx.x;
+  const float4* in = reinterpret_cast<const float4*>(x + static_cast<size_t>(row) * cols);
+  float amax = 0.0f;
+  for (uint32_t g = t; g < cols / 4u; g += 1024u) {
+    const float4 v = in[g];
+    amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), amax));
+  }
+  amax = wave_max(amax);
+  if ((t & 63u) == 0) red[t >> 6] = amax;
+  __syncthreads();
+  amax = red[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) amax = fmaxf(amax, red[w]);
+  const float s = row_scale_for(amax), inv_s = 1.0f / s;
+  half8_t* out = reinterpret_cast<half8_t*>(a16 + static_cast<size_t>(row) * cols);
+  for (uint32_t g = t; g < cols / 8u; g += 1024u) out[g] = to_f16_group(in[2 * g], in[2 * g + 1], inv_s);
+  if (t == 0) a_scale[row] = s;
+}
+
+// phi = silu(g) * u for one sorted row, written as the fp16 operand of the down GEMM with its
+// own power-of-two row scale (phi can exceed the fp16 range).
+__global__ __launch_bounds__(256) void moe_silu_mul_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                           _Float16* __restrict__ phi16, float* __restrict__ scale,
+                                                           uint32_t inter) {
+  __shared__ float red[4];
+  const size_t base = static_cast<size_t>(blockIdx.x) * inter;
+  const float4* gp = reinterpret_cast<const float4*>(g + base);
+  const float4* up = reinterpret_cast<const float4*>(u + base);
+  auto f = [](float gv, float uv) { return (gv / (1.0f + expf(-gv))) * uv; };
+  auto phi4 = [&](uint32_t q) {
+    const float4 a = gp[q], b = up[q];
+    return make_float4(f(a.x, b.x), f(a.y, b.y), f(a.z, b.z), f(a.w, b.w));
+  };
+  float amax = 0.0f;
+  for (uint32_t q = threadIdx.x; q < inter / 4u; q += 256u) {
+    const float4 v = phi4(q);
+    amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), amax));
+  }
+  const float s = row_scale_for(block_amax(amax, red)), inv = 1.0f / s;
+  half8_t* out = reinterpret_cast<half8_t*>(phi16 + base);
+  for (uint32_t q = threadIdx.x; q < inter / 8u; q += 256u) out[q] = to_f16_group(phi4(2 * q), phi4(2 * q + 1), inv);
+  if (threadIdx.x == 0) scale[blockIdx.x] = s;
+}
+
+// phi[p][j] = silu(g[pos[p]][j]) * u[pos[p]][j]: the grouped gate and up products of (token,
+// slot) pair p, which sit at sorted row pos[p], back in the caller's pair order as fp32.
+__global__ __launch_bounds__(256) void moe_silu_scatter_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                               const uint32_t* __restrict__ pos,
+                                                               float* __restrict__ phi, uint32_t inter) {
+  const size_t src = static_cast<size_t>(pos[blockIdx.x]) * inter, dst = static_cast<size_t>(blockIdx.x) * inter;
+  const float4* gp = reinterpret_cast<const float4*>(g + src);
+  const float4* up = reinterpret_cast<const float4*>(u + src);
+  float4* out = reinterpret_cast<float4*>(phi + dst);
+  auto f = [](float gv, float uv) { return (gv / (1.0f + expf(-gv))) * uv; };
+  for (uint32_t q = threadIdx.x; q < inter / 4u; q += 256u) {
+    const float4 a = gp[q], b = up[q];
+    out[q] = make_float4(f(a.x, b.x), f(a.y, b.y), f(a.z, b.z), f(a.w, b.w));
+  }
+}
+
+// out[t][j] (+)= sum_slot wts[t][slot] * rows[pos[t*top_k + slot]][j], slots in order.
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, const uint32_t* __restrict__ pos,
+                                                          const float* __restrict__ wts, float* __restrict__ out,
+                                                          uint32_t tokens, uint32_t top_k, uint32_t hidden,
+                                                          bool accumulate) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (i >= static_cast<uint64_t>(tokens) * hidden) return;
+  const uint32_t t = static_cast<uint32_t>(i / hidden), j = static_cast<uint32_t>(i % hidden);
+  float acc = 0.0f;
+  for (uint32_t s = 0; s < top_k; ++s) {
+    acc += wts[t * top_k + s] * rows[static_cast<size_t>(pos[t * top_k + s]) * hidden + j];
+  }
+  out[i] = accumulate ? out[i] + acc : acc;
+}
+
+// ---- the chunk path for experts whose inner width fits LDS: two kernels ----------------------
+// Both take 32 rows of an expert a pass and 32 columns a compute wavefront (so every weight is
+// decoded once), stream raw super-blocks through a ring of S LDS stages with one barrier per
+// super-block, and address rows through `inv` (sorted position -> pair), so no operand is
+// gathered or scattered by a separate pass.  The direct loads are all issued by one extra
+// wavefront that computes nothing: a CU accepts only so many vector-memory instructions at a
+// time, a wavefront that issues into a full queue stands still until they are taken, and a
+// wavefront that stores results must otherwise wait for its stores whenever it waits for loads
+// (one counter covers both).  Measured on the 256-expert shape: the weight stream alone takes
+// 68 us (gate and up) and 43 us (down), the arithmetic alone 24 and 12 us; with every
+// wavefront loading its share the two added up.
+template <int WAVES>
+struct MoeTile {
+  static constexpr uint32_t kBN = WAVES * 32u;                   // columns of a workgroup's tile
+  static constexpr int kWBlocks = kBN * 144u / 1024u;            // 1 KB loads of a weight stage (exact)
+  static constexpr uint32_t kWStage = kWBlocks * 1024u;
+  static constexpr int kABlocks = 16;                            // 1 KB loads of an activation stage
+  static constexpr uint32_t kAStage = 32u * 512u;                // one super-block of K for 32 rows, fp16
+  static constexpr uint32_t kThreads = (WAVES + 1) * 64u;        // compute wavefronts and the loader
+  static_assert(kBN * 144u % 1024u == 0, "tile shape");
+};
+
+// The loader's source offsets of a weight stage: load b is chunks 64 b .. 64 b + 63 of the
+// tile's 144-byte row pieces laid end to end (chunk q = 9 * row + part).
+template <int WAVES>
+__device__ __forceinline__ void moe_weight_offsets(uint32_t lane, uint32_t row_bytes, uint32_t (&src)[MoeTile<WAVES>::kWBlocks]) {
+#pragma unroll
+  for (int b = 0; b < MoeTile<WAVES>::kWBlocks; ++b) {
+    const uint32_t q = b * 64u + lane;
+    src[b] = (q / 9u) * row_bytes + (q % 9u) * 16u;
+  }
+}
+
+template <int WAVES>
+__device__ __forceinline__ void moe_issue_weights(const uint8_t* g, const uint32_t (&src)[MoeTile<WAVES>::kWBlocks],
+                                                  uint32_t lds_stage) {
+#pragma unroll
+  for (int b = 0; b < MoeTile<WAVES>::kWBlocks; ++b) direct_load16(g, src[b], lds_stage + b * 1024u);
+}
+
+// The loader's barrier: at most BEHIND younger loads may still be in flight (loads complete in
+// order), so the next stage has landed.  The compute wavefronts' barrier: their LDS reads of the
+// stage they leave are done.
+template <int BEHIND>
+__device__ __forceinline__ void moe_loader_barrier(bool ring_full) {
+  static_assert(BEHIND < 64, "vmcnt field");
+  if (ring_full) {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(BEHIND) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  }
+}
+__device__ __forceinline__ void moe_compute_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// One super-block (256 K values) of the 32 x 32 product of a wavefront: `raw` is the lane's
+// weight row in the raw stage, a_chunk(c) the address of 16-byte chunk c (8 K values) of the
+// lane's activation row.
+template <typename AChunk>
+__device__ __forceinline__ void moe_block_mma(const uint8_t* raw, uint32_t kg, AChunk&& a_chunk, float16_t& acc) {
+  const BlockHead head = load_block_head(raw);
+  uint32_t qw[4], qs8[4];
+  unrolled<8>([&](auto step) {
+    constexpr int sb = decltype(step)::value;
+    half8_t b[2];
+    decode_subblock<sb, true>(raw, kg, head, qw, qs8, b);
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const half8_t af = *reinterpret_cast<const half8_t*>(a_chunk(sb * 4u + tt * 2u + kg));
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[tt], acc, 0, 0, 0);
+    }
+  });
+}
+
+__device__ __forceinline__ void zero_acc(float16_t& acc) {
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+}
+
+// phi[p][c] = silu((gate_e x_t)(c)) * (up_e x_t)(c) for the pairs p = (t, slot) of expert e and
+// the columns of the workgroup's tile, written in pair order as fp32.  x comes as one fp16 copy
+// per token (a16, scale a_scale): the direct loads of a pass fetch the tokens of its 32 pairs.
+// Gate runs over all of K, then up; the gate sums wait in registers.
+template <int WAVES, int S>
+__global__ __launch_bounds__((WAVES + 1) * 64) void moe_gate_up_kernel(
+    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ gate,
+    const uint8_t* __restrict__ up, uint64_t gate_stride, uint64_t up_stride, float* __restrict__ phi,
+    const uint32_t* __restrict__ seg, const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t experts,
+    uint32_t top_k) {
+  using T = MoeTile<WAVES>;
+  constexpr int kLoads = T::kABlocks + T::kWBlocks;   // of one stage
+  __shared__ __attribute__((aligned(16))) uint8_t lds[S * (T::kAStage + T::kWStage)];
+  __shared__ uint32_t row_tok[32], row_dst[32];
+  __shared__ float row_scale[32];
+  // Grid as in q4k_gemm_grouped_kernel: an expert's tiles on one XCD, adjacent in dispatch order.
+  const uint32_t tiles = n / T::kBN;
+  const uint32_t slot = blockIdx.x / 8u;
+  const uint32_t e = (slot / tiles) * 8u + blockIdx.x % 8u, tile = slot % tiles;
+  if (e >= experts) return;
+  const uint32_t r0 = seg[e], r1 = seg[e + 1];
+  if (r1 <= r0) return;
+
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t row_blocks = k / 256u, row_bytes = row_blocks * 144u;
+  const uint32_t total = 2u * row_blocks;
+  const uint32_t lds_a = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds));
+  const uint32_t lds_w = lds_a + S * T::kAStage;
+
+  for (uint32_t m0 = r0; m0 < r1; m0 += 32u) {
+    const uint32_t live = r1 - m0 < 32u ? r1 - m0 : 32u;
+    if (t < 32u) {   // rows past the segment repeat its last row (computed, never stored)
+      const uint32_t p = inv[m0 + (t < live ? t : live - 1u)];
+      row_tok[t] = p / top_k;
+      row_dst[t] = p;
+      row_scale[t] = a_scale[p / top_k];
+    }
+    __syncthreads();
+
+    // Stage of iteration `it` is it % S.  Before iteration `it` the loads of it .. it + S - 2 are
+    // issued and stage it has landed; during it the loader issues it + S - 1 into the stage every
+    // wavefront left at the last barrier, then waits for it + 1.
+    if (wave == WAVES) {
+      const size_t tile_off = static_cast<size_t>(tile) * T::kBN * row_bytes;
+      const uint8_t* gate_e = gate + e * gate_stride + tile_off;
+      const uint8_t* up_e = up + e * up_stride + tile_off;
+      uint32_t w_src[T::kWBlocks], a_src[T::kABlocks];
+      moe_weight_offsets<WAVES>(lane, row_bytes, w_src);
+      // Activation stage = 32 rows x 512 bytes, loaded as 16 blocks of two rows; chunk c of row r
+      // sits at position c ^ r of the row, so that the 32 lanes of an MFMA operand read (same
+      // chunk, 32 rows) touch every bank once.
+#pragma unroll
+      for (int i = 0; i < T::kABlocks; ++i) {
+        const uint32_t row = 2u * i + lane / 32u;
+        a_src[i] = row_tok[row] * (k * 2u) + (((lane % 32u) ^ row) * 16u);
+      }
+      auto issue = [&](uint32_t it, uint32_t stage) {
+        const uint32_t blk = it < row_blocks ? it : it - row_blocks;
+        const uint8_t* ga = reinterpret_cast<const uint8_t*>(a16) + blk * 512u;
+#pragma unroll
+        for (int i = 0; i < T::kABlocks; ++i) direct_load16(ga, a_src[i], lds_a + stage * T::kAStage + i * 1024u);
+        moe_issue_weights<WAVES>((it < row_blocks ? gate_e : up_e) + blk * 144u, w_src, lds_w + stage * T::kWStage);
+      };
+#pragma unroll
+      for (int s = 0; s < S - 1; ++s) {
+        if (static_cast<uint32_t>(s) < total) issue(s, s);
+      }
+      moe_loader_barrier<(S - 2) * kLoads>(total >= static_cast<uint32_t>(S - 1));
+      uint32_t stage = 0;
+      for (uint32_t it = 0; it < total; ++it) {
+        const bool more = it + (S - 1) < total;
+        if (more) issue(it + (S - 1), stage == 0 ? S - 1 : stage - 1u);
+        moe_loader_barrier<(S - 2) * kLoads>(more);
+        stage = stage + 1u == S ? 0u : stage + 1u;
+      }
+    } else {
+      const uint32_t l32 = lane & 31u, kg = lane >> 5;
+      const uint8_t* w_lane = lds + S * T::kAStage + (wave * 32u + l32) * 144u;
+      const uint8_t* a_lane = lds + l32 * 512u;
+      float16_t acc, acc_gate;
+      uint32_t stage = 0;
+      moe_compute_barrier();
+      auto run = [&]() {   // one tensor
+        zero_acc(acc);
+        for (uint32_t blk = 0; blk < row_blocks; ++blk) {
+          moe_block_mma(w_lane + stage * T::kWStage, kg,
+                        [&](uint32_t c) { return a_lane + stage * T::kAStage + ((c ^ l32) * 16u); }, acc);
+          moe_compute_barrier();
+          stage = stage + 1u == S ? 0u : stage + 1u;
+        }
+      };
+      run();
+      acc_gate = acc;
+      run();
+
+      // lane holds column `col` and rows (e/4)*8 + kg*4 + e%4 of the pass
+      const uint32_t col = tile * T::kBN + wave * 32u + l32;
+#pragma unroll
+      for (int e16 = 0; e16 < 16; ++e16) {
+        const uint32_t row = (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
+        if (row < live) {
+          const float s = row_scale[row];
+          const float g = acc_gate[e16] * s, u = acc[e16] * s;
+          phi[static_cast<size_t>(row_dst[row]) * n + col] = (g / (1.0f + expf(-g))) * u;
+        }
+      }
+    }
+    __syncthreads();   // the row tables are rewritten by the next pass
+  }
+}
+
+// rows[p][c] = (down_e phi[p])(c) for the pairs of expert e, in pair order as fp32.  The 32 rows
+// of a pass stay in LDS for the whole pass as fp16 under a power-of-two row scale (phi can
+// exceed the fp16 range), converted here from the fp32 rows; the workgroup then streams the
+// weights of `tiles_per_chunk` column tiles past them without a break between tiles.
+// Dynamic LDS: S weight stages, the row tables, 32 rows of 2k + 16 bytes.
+template <int WAVES, int S>
+__global__ __launch_bounds__((WAVES + 1) * 64) void moe_down_kernel(
+    const float* __restrict__ phi, const uint8_t* __restrict__ down, uint64_t down_stride, float* __restrict__ rows,
+    const uint32_t* __restrict__ seg, const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t experts,
+    uint32_t chunks, uint32_t tiles_per_chunk) {
+  using T = MoeTile<WAVES>;
+  extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
+  float* row_scale = reinterpret_cast<float*>(dyn_lds + S * T::kWStage);
+  uint32_t* row_dst = reinterpret_cast<uint32_t*>(dyn_lds + S * T::kWStage + 128);
+  uint8_t* a_lds = dyn_lds + S * T::kWStage + 256;
+  const uint32_t a_stride = 2u * k + 16u;
+
+  const uint32_t tiles = n / T::kBN;
+  const uint32_t slot = blockIdx.x / 8u;
+  const uint32_t e = (slot / chunks) * 8u + blockIdx.x % 8u;
+  const uint32_t tile0 = (slot % chunks) * tiles_per_chunk;
+  if (e >= experts || tile0 >= tiles) return;
+  const uint32_t tile1 = tile0 + tiles_per_chunk < tiles ? tile0 + tiles_per_chunk : tiles;
+  const uint32_t r0 = seg[e], r1 = seg[e + 1];
+  if (r1 <= r0) return;
+
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t row_blocks = k / 256u, row_bytes = row_blocks * 144u;
+  const uint32_t total = (tile1 - tile0) * row_blocks;
+  const uint32_t lds_w = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)dyn_lds));
+
+  for (uint32_t m0 = r0; m0 < r1; m0 += 32u) {
+    const uint32_t live = r1 - m0 < 32u ? r1 - m0 : 32u;
+    // The fp16 copy of the pass's rows: the compute wavefronts' (WAVES * 2) threads a row take its
+    // largest magnitude, then write the groups of 8 in the order the decode yields.
+    if (wave < WAVES) {
+      constexpr uint32_t kPer = WAVES * 2u;
+      const uint32_t row = t / kPer, sub = t % kPer;
+      const uint32_t p = inv[m0 + (row < live ? row : live - 1u)];
+      const float4* src = reinterpret_cast<const float4*>(phi + static_cast<size_t>(p) * k);
+      float amax = 0.0f;
+      for (uint32_t c = sub; c < k / 4u; c += kPer) {
+        const float4 v = src[c];
+        amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), amax));
+      }
+#pragma unroll
+      for (uint32_t d = 1; d < kPer; d *= 2u) amax = fmaxf(amax, __shfl_xor(amax, d));
+      const float s = row_scale_for(amax), inv_s = 1.0f / s;
+      for (uint32_t c = sub; c < k / 8u; c += kPer) {
+        *reinterpret_cast<half8_t*>(a_lds + row * a_stride + c * 16u) = to_f16_group(src[2 * c], src[2 * c + 1], inv_s);
+      }
+      if (sub == 0) row_scale[row] = s, row_dst[row] = p;
+    }
+    __syncthreads();
+
+    // Iteration `it` is block it % row_blocks of tile tile0 + it / row_blocks; stages and waits
+    // as in moe_gate_up_kernel.
+    if (wave == WAVES) {
+      const uint8_t* down_e = down + e * down_stride;
+      uint32_t w_src[T::kWBlocks];
+      moe_weight_offsets<WAVES>(lane, row_bytes, w_src);
+      uint32_t tile_i = tile0, blk_i = 0;   // S - 1 iterations ahead
+      auto issue_next = [&](uint32_t stage) {
+        moe_issue_weights<WAVES>(down_e + static_cast<size_t>(tile_i) * T::kBN * row_bytes + blk_i * 144u, w_src,
+                                 lds_w + stage * T::kWStage);
+        if (++blk_i == row_blocks) blk_i = 0, ++tile_i;
+      };
+#pragma unroll
+      for (int s = 0; s < S - 1; ++s) {
+        if (static_cast<uint32_t>(s) < total) issue_next(s);
+      }
+      moe_loader_barrier<(S - 2) * T::kWBlocks>(total >= static_cast<uint32_t>(S - 1));
+      uint32_t stage = 0;
+      for (uint32_t it = 0; it < total; ++it) {
+        const bool more = it + (S - 1) < total;
+        if (more) issue_next(stage == 0 ? S - 1 : stage - 1u);
+        moe_loader_barrier<(S - 2) * T::kWBlocks>(more);
+        stage = stage + 1u == S ? 0u : stage + 1u;
+      }
+    } else {
+      const uint32_t l32 = lane & 31u, kg = lane >> 5;
+      const uint8_t* w_lane = dyn_lds + (wave * 32u + l32) * 144u;
+      const uint8_t* a_lane = a_lds + l32 * a_stride;
+      float16_t acc;
+      uint32_t stage = 0;
+      moe_compute_barrier();
+      for (uint32_t tile = tile0; tile < tile1; ++tile) {
+        zero_acc(acc);
+        for (uint32_t blk = 0; blk < row_blocks; ++blk) {
+          moe_block_mma(w_lane + stage * T::kWStage, kg, [&](uint32_t c) { return a_lane + (blk * 32u + c) * 16u; }, acc);
+          moe_compute_barrier();
+          stage = stage + 1u == S ? 0u : stage + 1u;
+        }
+        const uint32_t col = tile * T::kBN + wave * 32u + l32;
+#pragma unroll
+        for (int e16 = 0; e16 < 16; ++e16) {
+          const uint32_t row = (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
+          if (row < live) rows[static_cast<size_t>(row_dst[row]) * n + col] = acc[e16] * row_scale[row];
+        }
+      }
+    }
+    __syncthreads();   // the rows and their tables are rewritten by the next pass
+  }
+}
+
+// out[t][j] (+)= sum_slot wts[t][slot] * rows[t * top_k + slot][j], slots in order, four columns a thread.
+__global__ __launch_bounds__(256) void moe_combine_pairs_kernel(const float4* __restrict__ rows, const float* __restrict__ wts,
+                                                                float4* __restrict__ out, uint32_t tokens, uint32_t top_k,
+                                                                uint32_t hidden4, bool accumulate) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (i >= static_cast<uint64_t>(tokens) * hidden4) return;
+  const uint32_t t = static_cast<uint32_t>(i / hidden4), j = static_cast<uint32_t>(i % hidden4);
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  for (uint32_t s = 0; s < top_k; ++s) {
+    const float w = wts[t * top_k + s];
+    const float4 r = rows[static_cast<size_t>(t * top_k + s) * hidden4 + j];
+    acc.x += w * r.x, acc.y += w * r.y, acc.z += w * r.z, acc.w += w * r.w;
+  }
+  if (accumulate) {
+    const float4 o = out[i];
+    acc.x += o.x, acc.y += o.y, acc.z += o.z, acc.w += o.w;
+  }
+  out[i] = acc;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~size_t{255}; }
+
+constexpr size_t kMoeLdsLimit = 160 * 1024 - 64;
+template <int WAVES, int S>
+size_t moe_down_lds_bytes(uint32_t inter) {
+  return S * MoeTile<WAVES>::kWStage + 256 + 32 * (2 * static_cast<size_t>(inter) + 16);
+}
+
+// The two-kernel path needs an expert's 32 rows of phi in LDS next to the weight ring (eight
+// compute wavefronts and three stages up to an inner width of 768, four and two up to 1792),
+// whole column tiles, and 32-bit byte offsets into the fp16 token copy.
+bool moe_resident_path(uint32_t hidden, uint32_t inter, uint32_t tokens) {
+  return moe_down_lds_bytes<4, 2>(inter) <= kMoeLdsLimit && static_cast<uint64_t>(tokens) * hidden * 2 < (1ull << 32);
+}
+
+void launch_moe_gate_up_resident(const _Float16* a16, const float* a_scale, const uint8_t* gate, const uint8_t* up,
+                                 uint64_t gate_stride, uint64_t up_stride, float* phi, const uint32_t* seg,
+                                 const uint32_t* inv, uint32_t hidden, uint32_t inter, uint32_t experts, uint32_t top_k,
+                                 hipStream_t stream) {
+  const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
+  hipLaunchKernelGGL((moe_gate_up_kernel<8, 3>), dim3(expert_groups * (inter / 256u)), dim3(MoeTile<8>::kThreads), 0, stream, a16, a_scale,
+                     gate, up, gate_stride, up_stride, phi, seg, inv, inter, hidden, experts, top_k);
+}
+
+template <int WAVES, int S>
+void launch_moe_down_tiles(const float* phi, const uint8_t* down, uint64_t down_stride, float* rows, const uint32_t* seg,
+                           const uint32_t* inv, uint32_t hidden, uint32_t inter, uint32_t experts, uint32_t per_cu,
+                           hipStream_t stream) {
+  // As many column chunks per expert as give every CU its `per_cu` workgroups.
+  const uint32_t tiles = hidden / MoeTile<WAVES>::kBN;
+  const uint32_t want = (per_cu * static_cast<uint32_t>(num_cus()) + experts - 1u) / experts;
+  const uint32_t chunks = want < 1u ? 1u : want > tiles ? tiles : want;
+  const uint32_t tiles_per_chunk = (tiles + chunks - 1u) / chunks;
+  const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
+  const size_t lds_bytes = moe_down_lds_bytes<WAVES, S>(inter);
+  hipLaunchKernelGGL((moe_down_kernel<WAVES, S>), dim3(expert_groups * chunks), dim3(MoeTile<WAVES>::kThreads), lds_bytes, stream, phi,
+                     down, down_stride, rows, seg, inv, hidden, inter, experts, chunks, tiles_per_chunk);
+}
+
+void launch_moe_down_resident(const float* phi, const uint8_t* down, uint64_t down_stride, float* rows, const uint32_t* seg,
+                              const uint32_t* inv, uint32_t hidden, uint32_t inter, uint32_t experts, hipStream_t stream) {
+  if (moe_down_lds_bytes<8, 3>(inter) <= kMoeLdsLimit) {
+    launch_moe_down_tiles<8, 3>(phi, down, down_stride, rows, seg, inv, hidden, inter, experts, 1u, stream);
+  } else {
+    launch_moe_down_tiles<4, 2>(phi, down, down_stride, rows, seg, inv, hidden, inter, experts, 1u, stream);
+  }
+}
+
+}  // namespace
+
+bool moe_ffn_q4k_supported(uint64_t hidden, uint64_t inter, uint64_t experts) {
+  return hidden % 256 == 0 && inter % 256 == 0 && hidden <= (1u << 16) && inter <= (1u << 16) && experts >= 1 &&
+         experts <= 1024;
+}
+
+hipError_t moe_q4k_prepare() {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_down_kernel<8, 3>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMoeLdsLimit));
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_down_kernel<4, 2>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             static_cast<int>(kMoeLdsLimit));
+}
+
+namespace {
+
+// The workspace, carved the same way by the three entry points (each uses the parts it needs).
+struct MoeWorkspace {
+  uint32_t *seg, *pos, *inv;
+  float *x_scale, *phi_scale;
+  _Float16* a16;      // fp16 rows of x: one per token (resident path) or one per pair, gathered
+  float *g, *u;       // pairs x inter each; g doubles as phi (fp32, pair order) on the resident path
+  _Float16* phi16;
+  float* rows;        // pairs x hidden
+  size_t bytes;
+};
+MoeWorkspace carve_moe_workspace(void* workspace, uint64_t pairs, uint64_t hidden, uint64_t inter, uint64_t experts) {
+  uint8_t* const base = static_cast<uint8_t*>(workspace);
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    uint8_t* p = base + off;
+    off += align256(bytes);
+    return p;
+  };
+  MoeWorkspace w;
+  w.seg = reinterpret_cast<uint32_t*>(take((experts + 1) * 4));
+  w.pos = reinterpret_cast<uint32_t*>(take(pairs * 4));
+  w.inv = reinterpret_cast<uint32_t*>(take(pairs * 4));
+  w.x_scale = reinterpret_cast<float*>(take((pairs + 256) * 4));
+  w.phi_scale = reinterpret_cast<float*>(take((pairs + 256) * 4));
+  w.a16 = reinterpret_cast<_Float16*>(take(pairs * hidden * 2));
+  w.g = reinterpret_cast<float*>(take(pairs * inter * 4));
+  w.u = reinterpret_cast<float*>(take(pairs * inter * 4));
+  w.phi16 = reinterpret_cast<_Float16*>(take(pairs * inter * 2));
+  w.rows = reinterpret_cast<float*>(take(pairs * hidden * 4));
+  w.bytes = off;
+  return w;
+}
+
+void launch_grouped(const _Float16* a16, const float* a_scale, const uint8_t* w, float* c, const uint32_t* seg,
+                    uint64_t w_stride, uint32_t n, uint32_t k, uint32_t experts, const uint8_t* w2, float* c2,
+                    uint64_t w2_stride, hipStream_t stream) {
+  constexpr int BM = 32, BN = 64;
+  const uint32_t expert_groups = (experts + 7u) / 8u * 8u, tensors = w2 != nullptr ? 2u : 1u;
+  hipLaunchKernelGGL((q4k_gemm_grouped_kernel<BM, BN>), dim3(expert_groups * ((n + BN - 1) / BN) * tensors), dim3(BN * 2), 0,
+                     stream, a16, a_scale, w, c, seg, w_stride, n, k, experts, tensors, w2, c2, w2_stride);
+}
+
+void launch_combine(const float* rows, const float* wts, float* out, uint32_t tokens, uint32_t top_k, uint32_t hidden,
+                    bool accumulate, hipStream_t stream) {
+  const uint64_t outs = static_cast<uint64_t>(tokens) * (hidden / 4u);
+  hipLaunchKernelGGL(moe_combine_pairs_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream,
+                     reinterpret_cast<const float4*>(rows), wts, reinterpret_cast<float4*>(out), tokens, top_k, hidden / 4u,
+                     accumulate);
+}
+
+}  // namespace
+
+size_t moe_ffn_q4k_workspace_bytes(uint64_t pairs, uint64_t hidden, uint64_t inter, uint64_t experts) {
+  return carve_moe_workspace(nullptr, pairs, hidden, inter, experts).bytes;
+}
+
+// Two regimes.  Experts whose inner width fits LDS (moe_resident_path): x as one fp16 row per
+// token, moe_gate_up_kernel, moe_down_kernel, a combine over consecutive rows.  Wider experts:
+// the pairs' rows gathered as fp16, grouped GEMM tiles with the activations streamed in slices
+// (q4k_gemm_grouped_kernel), silu and the fp16 copy of phi as a pass of their own.
+hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                              const uint32_t* ids, const float* wts, float* out, void* workspace,
+                              uint32_t hidden, uint32_t inter, uint32_t top_k, uint64_t gate_stride,
+                              uint64_t up_stride, uint64_t down_stride, uint32_t experts, uint32_t tokens,
+                              bool accumulate, hipStream_t stream) {
+  const uint32_t pairs = tokens * top_k;
+  const MoeWorkspace ws = carve_moe_workspace(workspace, pairs, hidden, inter, experts);
+  if (moe_resident_path(hidden, inter, tokens)) {
+    hipLaunchKernelGGL(moe_prepare_kernel, dim3(1u + tokens), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos,
+                       ws.inv, x, ws.a16, ws.x_scale, hidden);
+    launch_moe_gate_up_resident(ws.a16, ws.x_scale, gate, up, gate_stride, up_stride, ws.g, ws.seg, ws.inv, hidden, inter,
+                                experts, top_k, stream);
+    launch_moe_down_resident(ws.g, down, down_stride, ws.rows, ws.seg, ws.inv, hidden, inter, experts, stream);
+    launch_combine(ws.rows, wts, out, tokens, top_k, hidden, accumulate, stream);
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos, ws.inv);
+  launch_rows_to_f16(x, ws.a16, ws.x_scale, pairs, hidden, ws.pos, top_k, stream);
+  launch_grouped(ws.a16, ws.x_scale, gate, ws.g, ws.seg, gate_stride, inter, hidden, experts, up, ws.u, up_stride, stream);
+  hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(pairs), dim3(256), 0, stream, ws.g, ws.u, ws.phi16, ws.phi_scale, inter);
+  launch_grouped(ws.phi16, ws.phi_scale, down, ws.rows, ws.seg, down_stride, hidden, inter, experts, nullptr, nullptr, 0,
+                 stream);
+  const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, ws.rows,
+                     ws.pos, wts, out, tokens, top_k, hidden, accumulate);
+  return hipGetLastError();
+}
+
+// The two halves of launch_moe_ffn_q4k behind the reference's own pair of ids
+// ("moe_experts_gate_up_q4k_rows" then "moe_experts_down_q4k_rows",
+// src/backends/rocm/rocm_kernels_moe.cpp:15-79) for a chunk of tokens: each sorts the pairs by
+// expert for itself, so an expert's weights are read once per launch instead of once per token
+// that chose it.  phi keeps the caller's layout (tokens x top_k x inter, fp32) between the two.
+// Workspace as for launch_moe_ffn_q4k.
+hipError_t launch_moe_gate_up_q4k_grouped(const float* x, const uint8_t* gate, const uint8_t* up, const uint32_t* ids,
+                                          float* phi, void* workspace, uint32_t hidden, uint32_t inter, uint32_t top_k,
+                                          uint64_t gate_stride, uint64_t up_stride, uint32_t experts, uint32_t tokens,
+                                          hipStream_t stream) {
+  const uint32_t pairs = tokens * top_k;
+  const MoeWorkspace ws = carve_moe_workspace(workspace, pairs, hidden, inter, experts);
+  if (moe_resident_path(hidden, inter, tokens)) {
+    hipLaunchKernelGGL(moe_prepare_kernel, dim3(1u + tokens), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos,
+                       ws.inv, x, ws.a16, ws.x_scale, hidden);
+    launch_moe_gate_up_resident(ws.a16, ws.x_scale, gate, up, gate_stride, up_stride, phi, ws.seg, ws.inv, hidden, inter,
+                                experts, top_k, stream);
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos, ws.inv);
+  launch_rows_to_f16(x, ws.a16, ws.x_scale, pairs, hidden, ws.pos, top_k, stream);
+  launch_grouped(ws.a16, ws.x_scale, gate, ws.g, ws.seg, gate_stride, inter, hidden, experts, up, ws.u, up_stride, stream);
+  hipLaunchKernelGGL(moe_silu_scatter_kernel, dim3(pairs), dim3(256), 0, stream, ws.g, ws.u, ws.pos, phi, inter);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_down_q4k_grouped(const float* phi, const uint8_t* down, const uint32_t* ids, const float* wts,
+                                       float* out, void* workspace, uint32_t hidden, uint32_t inter, uint32_t top_k,
+                                       uint64_t down_stride, uint32_t experts, uint32_t tokens, bool accumulate,
+                                       hipStream_t stream) {
+  const uint32_t pairs = tokens * top_k;
+  const MoeWorkspace ws = carve_moe_workspace(workspace, pairs, hidden, inter, experts);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos, ws.inv);
+  if (moe_resident_path(hidden, inter, tokens)) {
+    launch_moe_down_resident(phi, down, down_stride, ws.rows, ws.seg, ws.inv, hidden, inter, experts, stream);
+    launch_combine(ws.rows, wts, out, tokens, top_k, hidden, accumulate, stream);
+    return hipGetLastError();
+  }
+  // source row of pair p is p itself (phi is pair-major): top_k = 1 in the gather
+  launch_rows_to_f16(phi, ws.phi16, ws.phi_scale, pairs, inter, ws.pos, 1u, stream);
+  launch_grouped(ws.phi16, ws.phi_scale, down, ws.rows, ws.seg, down_stride, hidden, inter, experts, nullptr, nullptr, 0,
+                 stream);
+  const uint64_t outs = static_cast<uint64_t>(tokens) * hidden;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(static_cast<uint32_t>((outs + 255) / 256)), dim3(256), 0, stream, ws.rows,
+                     ws.pos, wts, out, tokens, top_k, hidden, accumulate);
+  return hipGetLastError();
+}
+
+}  // namespace qmm

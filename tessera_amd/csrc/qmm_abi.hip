@@ -1080,7 +1080,7 @@ qmm_status qmm_init(int device) {
     }
     g_static_scratch[device] = p;
   }
-  if ((e = qmm::gemv_q4k_rows16_prepare()) != hipSuccess) {
+  if ((e = qmm::gemv_q4k_rows16_prepare()) != hipSuccess || (e = qmm::moe_q4k_prepare()) != hipSuccess) {
     g_device = -1;
     return map_hip(e);
   }

@@ -94,8 +94,12 @@ size_t gemm_kquant_f16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k);
 hipError_t launch_kquant_f16_gemm(const float* a, const uint8_t* w, uint32_t block_bytes, float* c, void* workspace,
                                   uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
 
-// Routed experts for a chunk of tokens, grouped by expert (gemm_q4k.hip): out[t] (+)= sum over
+// Routed experts for a chunk of tokens, grouped by expert (moe_q4k.hip): out[t] (+)= sum over
 // the token's top_k experts of wts * down_e(silu(gate_e x) * up_e x), as grouped MFMA GEMMs.
+// fp16 copy of fp32 rows, each divided by a power-of-two scale written to scale[row] (gemm_q4k.hip).
+// With `pos`, destination row pos[p] takes source row p / top_k.
+void launch_rows_to_f16(const float* src, _Float16* dst, float* scale, uint32_t rows, uint32_t cols, const uint32_t* pos,
+                        uint32_t top_k, hipStream_t stream);
 bool moe_ffn_q4k_supported(uint64_t hidden, uint64_t inter, uint64_t experts);
 size_t moe_ffn_q4k_workspace_bytes(uint64_t pairs, uint64_t hidden, uint64_t inter, uint64_t experts);
 hipError_t launch_moe_gate_up_q4k_grouped(const float* x, const uint8_t* gate, const uint8_t* up, const uint32_t* ids,
@@ -129,6 +133,7 @@ hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
 // Q4_K x 2..16 activation rows in one pass over the weights on the 16x16x32 fp16 MFMA, exact on the
 // weight side (gemv_q4k_rows16.hip).  `workspace` holds the K parts' output regions.
 hipError_t gemv_q4k_rows16_prepare();   // once per device, from qmm_init
+hipError_t moe_q4k_prepare();           // once per device, from qmm_init (moe_q4k.hip)
 bool gemv_q4k_rows16_supported(uint64_t m, uint64_t n, uint64_t k);
 size_t gemv_q4k_rows16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k);
 hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,

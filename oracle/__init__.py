@@ -63,6 +63,7 @@ def _load() -> C.CDLL:
         "orc_gemm_mxfp4_ref_omp": (C.c_int, [f32p, u8p, u8p, f32p, sz, sz, sz]),
         "orc_dequantize_mxfp4": (C.c_int, [u8p, f32p, sz, sz]),
         "orc_gemm_fp8_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
+        "orc_gemm_fp8_block_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
         "orc_permute_mxfp4_to_wmma": (C.c_int, [u8p, u8p, sz, sz]),
         "orc_rope": (C.c_int, [f32p, sz, sz, sz, sz, C.c_uint64, C.c_double]),
         "orc_mrope": (C.c_int, [f32p, C.POINTER(C.c_uint64), sz, sz, sz, sz, sz, sz, sz, C.c_double]),
@@ -269,6 +270,18 @@ def gemm_fp8(a, w, s, m: int, n: int, k: int) -> np.ndarray:
     c = np.empty((m, n), dtype=np.float32)
     _check(_lib.orc_gemm_fp8_ref(_p(a, C.c_float), _p(w, C.c_uint8), _p(s, C.c_float),
                                  _p(c, C.c_float), m, n, k))
+    return c
+
+
+def gemm_fp8_block(a, w, s, m: int, n: int, k: int) -> np.ndarray:
+    """GemmFp8BlockRef: one scale per 128 x 128 block of W (s is (n/128) x (k/128))."""
+    a, w, s = _f32(a), _u8(w), _f32(s)
+    assert a.size == m * k and w.size == n * k
+    if n % 128 == 0 and k % 128 == 0:
+        assert s.size == (n // 128) * (k // 128)
+    c = np.empty((m, n), dtype=np.float32)
+    _check(_lib.orc_gemm_fp8_block_ref(_p(a, C.c_float), _p(w, C.c_uint8), _p(s, C.c_float),
+                                       _p(c, C.c_float), m, n, k))
     return c
 
 

@@ -594,6 +594,25 @@ int orc_gemm_fp8_ref(const float* a, const uint8_t* w, const float* s, float* c,
   return ORC_OK;
 }
 
+/* ---- the same with one fp32 scale per 128 x 128 block of W (gemm.cpp:282-309):
+ *      s is (n/128) x (k/128), n and k multiples of 128 ---- */
+int orc_gemm_fp8_block_ref(const float* a, const uint8_t* w, const float* s, float* c, size_t m,
+                           size_t n, size_t k) {
+  if (m == 0 || n == 0 || k == 0 || n % 128 != 0 || k % 128 != 0) return ORC_INVALID_ARGUMENT;
+  const size_t k_blocks = k / 128;
+  for (size_t i = 0; i < m; ++i) {
+    for (size_t j = 0; j < n; ++j) {
+      const float* s_row = s + (j / 128) * k_blocks;
+      float acc = 0.0f;
+      for (size_t t = 0; t < k; ++t) {
+        acc = fmaf(a[i * k + t], s_row[t / 128] * orc_fp8_e4m3_to_float(w[j * k + t]), acc);
+      }
+      c[i * n + j] = acc;
+    }
+  }
+  return ORC_OK;
+}
+
 /* e4m3 byte of (E2M1 magnitude code mag) * 2^-d, derived from the encoder with
  * round-to-nearest-even.  Agrees with the reference's literal table below except in
  * three tie entries (the tests list them). */

@@ -1070,7 +1070,10 @@ struct MxFp4A8Codec {
 // ----------------------------------------------------------------------------
 // NQ = 16-byte pieces per chunk: a lane takes 16 * NQ consecutive weights of a row.  One piece
 // for rows up to 16384 long, two beyond (a row must fit the 1024 threads of a workgroup).
-template <int NQ>
+// BLOCK: `s` holds one scale per 128 x 128 block of W instead ("gemm_fp8_block",
+// include/tessera/backend.hpp:183-186; src/core/numerics/gemm.cpp:282-309): a chunk lies inside
+// one block, so its partial dot product takes the block's scale before the lanes are summed.
+template <int NQ, bool BLOCK = false>
 struct Fp8CodecT {
   struct Args {
     const float* a;
@@ -1085,6 +1088,7 @@ struct Fp8CodecT {
   };
   struct Frag {
     uint4 q[NQ];
+    float bs;   // BLOCK: the scale of the chunk's block
   };
 
   static __host__ __device__ __forceinline__ uint32_t chunks_per_row(uint32_t k) { return k / kChunk; }
@@ -1108,9 +1112,10 @@ struct Fp8CodecT {
     }
   }
 
+  // off1 (BLOCK): the lane's row inside the group and the 128-wide K block of its chunk
   static __device__ __forceinline__ Lane make_lane(const Args&, uint32_t cpr, uint32_t chunk,
                                                    uint32_t prow) {
-    return Lane{(prow * cpr + chunk) * kChunk, 0u};
+    return Lane{(prow * cpr + chunk) * kChunk, BLOCK ? prow | ((chunk * kChunk / 128u) << 8) : 0u};
   }
 
   static __device__ __forceinline__ void load(const Args& p, const Lane& ln, uint32_t row,
@@ -1118,6 +1123,7 @@ struct Fp8CodecT {
     const uint8_t* base = p.w + static_cast<size_t>(row) * cpr * kChunk + ln.off0;
 #pragma unroll
     for (int j = 0; j < NQ; ++j) f.q[j] = load_u4(base + 16 * j);
+    if constexpr (BLOCK) f.bs = p.s[static_cast<size_t>((row + (ln.off1 & 0xFFu)) >> 7) * (p.k >> 7) + (ln.off1 >> 8)];
   }
 
   template <int R>
@@ -1144,12 +1150,12 @@ struct Fp8CodecT {
       }
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) out[r] = a0[r] + a1[r];
+    for (int r = 0; r < R; ++r) out[r] = BLOCK ? (a0[r] + a1[r]) * f.bs : a0[r] + a1[r];
   }
 
   template <int R>
   static __device__ __forceinline__ float finish(const Args& p, uint32_t row, int, float v) {
-    return v * p.s[row];
+    return BLOCK ? v : v * p.s[row];
   }
 };
 using Fp8Codec = Fp8CodecT<1>;
@@ -1850,11 +1856,16 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
   return hipSuccess;
 }
 
-hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
-                           uint32_t n, uint32_t k, hipStream_t stream) {
+namespace {
+template <bool BLOCK>
+hipError_t launch_fp8_gemv_as(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
+                              uint32_t n, uint32_t k, hipStream_t stream) {
+  using Fp8Codec = Fp8CodecT<1, BLOCK>;
+  using Fp8WideCodec = Fp8CodecT<2, BLOCK>;
+  using Fp8QuadCodec = Fp8CodecT<4, BLOCK>;
   if (k / 32u > 1024u || (k / 16u > 1024u && k % 32u != 0)) {
     for (uint32_t r = 0; r < m; ++r) {
-      const hipError_t e = launch_gemv_generic<Fp8Codec>(Fp8Codec::Args{a + static_cast<size_t>(r) * k, w, s, k},
+      const hipError_t e = launch_gemv_generic<Fp8Codec>(typename Fp8Codec::Args{a + static_cast<size_t>(r) * k, w, s, k},
                                                          c + static_cast<size_t>(r) * n, n, k, stream);
       if (e != hipSuccess) return e;
     }
@@ -1863,13 +1874,13 @@ hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, flo
   const uint32_t cpr4 = k / 64u;
   if (m == 1 && k % 64u == 0 && cpr4 >= 64u && cpr4 <= 768u) {
     // one row: 64 weights a lane, so the reduction and the loop overhead are paid once per 64
-    Fp8QuadCodec::Args args{a, w, s, k};
+    typename Fp8QuadCodec::Args args{a, w, s, k};
     return launch_gemv_r<Fp8QuadCodec, 1, 768, 2, 9>(args, c, n, k, n, stream);
   }
   if (k / 16u > 1024u) {
     // rows of 16385..32768 weights: 32 weights a lane, one or two activation rows per weight pass
     for (uint32_t r0 = 0; r0 < m;) {
-      Fp8WideCodec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
+      typename Fp8WideCodec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
       float* out = c + static_cast<size_t>(r0) * n;
       hipError_t e;
       uint32_t took;
@@ -1885,7 +1896,7 @@ hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, flo
   }
   for (uint32_t r0 = 0; r0 < m;) {
     const uint32_t left = m - r0;
-    Fp8Codec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
+    typename Fp8Codec::Args args{a + static_cast<size_t>(r0) * k, w, s, k};
     float* out = c + static_cast<size_t>(r0) * n;
     hipError_t e;
     uint32_t took;
@@ -1900,6 +1911,18 @@ hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, flo
     r0 += took;
   }
   return hipSuccess;
+}
+}  // namespace
+
+hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
+                           uint32_t n, uint32_t k, hipStream_t stream) {
+  return launch_fp8_gemv_as<false>(a, w, s, c, m, n, k, stream);
+}
+
+// One scale per 128 x 128 block of W (n and k multiples of 128).
+hipError_t launch_fp8_block_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
+                                 uint32_t n, uint32_t k, hipStream_t stream) {
+  return launch_fp8_gemv_as<true>(a, w, s, c, m, n, k, stream);
 }
 
 // ---- mixture-of-experts (Q4_K experts) ------------------------------------------------

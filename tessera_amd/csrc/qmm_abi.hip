@@ -788,6 +788,22 @@ qmm_status run_gemm_fp8(const LaunchCtx& c) {
                                       static_cast<uint32_t>(k), c.stream));
 }
 
+// "gemm_fp8_block": buffers A, W (n x k E4M3 bytes), S ((n/128) x (k/128) fp32 block scales), C;
+// scalars m, n, k with n and k multiples of 128 (include/tessera/backend.hpp:183-186,476-485;
+// reference kernel src/backends/rocm/rocm_kernels_basic.cpp:1066-1089).
+qmm_status run_gemm_fp8_block(const LaunchCtx& c) {
+  if (!counts(c, 4, 3)) return bad("gemm_fp8_block: expects 4 buffers and 3 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
+  if (!dims_ok(m, n, k) || n % 128 != 0 || k % 128 != 0) return bad("gemm_fp8_block: m, n, k must be non-zero, n and k multiples of 128");
+  if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, static_cast<u128>(n) * k) ||
+      !c.fits(2, static_cast<u128>(n / 128) * (k / 128) * 4) || !c.fits(3, static_cast<u128>(m) * n * 4)) {
+    return bad("gemm_fp8_block: a buffer is smaller than m, n, k require");
+  }
+  return map_hip(qmm::launch_fp8_block_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
+                                            c.ptr<float>(3), static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                            static_cast<uint32_t>(k), c.stream));
+}
+
 // "moe_scale_add": buffers a, b, f, o; scalars n, idx
 // (src/backends/rocm/rocm_kernels_basic.cpp:1932-1942).
 qmm_status run_moe_scale_add(const LaunchCtx& c) {
@@ -1015,6 +1031,7 @@ const Entry kTable[] = {
     {"quantize_fp8_pack", run_quantize_fp8_pack},
     {"quantize_fp8_pack_rows", run_quantize_fp8_pack},
     {"gemm_fp8", run_gemm_fp8},
+    {"gemm_fp8_block", run_gemm_fp8_block},
     {"moe_scale_add", run_moe_scale_add},
     {"moe_experts_gate_up_q4k", run_moe_gate_up},
     {"moe_experts_down_q4k", run_moe_down},

@@ -33,6 +33,8 @@ hipError_t launch_mxfp4_a8_gemv(const uint8_t* a8, const float* as, const uint8_
 // W = n x k E4M3 bytes, s = one fp32 scale per weight row.
 hipError_t launch_fp8_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
                            uint32_t n, uint32_t k, hipStream_t stream);
+hipError_t launch_fp8_block_gemv(const float* a, const uint8_t* w, const float* s, float* c, uint32_t m,
+                           uint32_t n, uint32_t k, hipStream_t stream);   // s: (n/128) x (k/128) block scales
 
 // Q4_K times 1..4 activation rows on the 4x4x4 fp16 MFMA (gemv_q4k_mfma.hip).  `workspace`
 // holds the fp16 hi/lo activation operand (gemv_q4k_mfma_workspace_bytes).

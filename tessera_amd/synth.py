@@ -125,6 +125,18 @@ def fp8_weights(g: np.random.Generator, n: int, k: int) -> tuple[np.ndarray, np.
     return codes.reshape(-1), scales
 
 
+def fp8_block_weights(g: np.random.Generator, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:
+    """E4M3 weights with one scale per 128 x 128 block (n and k multiples of 128): W ~ N(0, 0.02^2)
+    with a per-block gain, scale = amax(block) / 448, codes = e4m3(W / scale).  Returns
+    (codes n*k, scales (n/128)*(k/128) row-major)."""
+    nb, kb = n // 128, k // 128
+    gain = g.uniform(0.25, 4.0, size=(nb, kb)).astype(np.float32)
+    w = (g.standard_normal(size=(n, k)) * 0.02).astype(np.float32).reshape(nb, 128, kb, 128) * gain[:, None, :, None]
+    scales = (np.abs(w).max(axis=(1, 3)) / np.float32(448.0)).astype(np.float32)
+    codes = encode_e4m3((w / scales[:, None, :, None]).reshape(n, k))
+    return codes.reshape(-1), scales.reshape(-1)
+
+
 def activations_f32(g: np.random.Generator, m: int, k: int) -> np.ndarray:
     return g.standard_normal(size=(m, k)).astype(np.float32)
 

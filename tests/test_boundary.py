@@ -19,7 +19,7 @@ REFERENCE_IDS = [
     "gemm_q4k_rows5", "gemm_q4k_batched", "gemm_q4k_wmma", "gemm_vec_reduce", "gemm_mxfp4",
     "gemm_mxfp4_rows", "gemm_mxfp4_batched", "mxfp4_row_ref", "gemm_mxfp4_wmma",
     "gemm_mxfp4_wmma_reduce", "quantize_fp8", "quantize_fp8_pack", "quantize_fp8_pack_rows",
-    "gemm_fp8", "moe_scale_add", "moe_experts_gate_up_q4k", "moe_experts_down_q4k", "moe_gate",
+    "gemm_fp8", "gemm_fp8_block", "moe_scale_add", "moe_experts_gate_up_q4k", "moe_experts_down_q4k", "moe_gate",
     "top_k_rows", "gemm_q6k", "gemm_q6k_vec", "gemm_q6k_rows2", "gemm_q6k_rows3", "gemm_q6k_rows4",
     "gemm_q6k_rows5", "gemm_q6k_batched", "gemm_q5k", "gemm_q5k_vec", "gemm_q5k_rows2", "gemm_q5k_rows3",
     "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched", "moe_experts_down_q6k", "gemm_q5k_wmma", "gemm_q6k_wmma",

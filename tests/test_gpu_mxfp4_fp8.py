@@ -268,6 +268,35 @@ def test_gemm_fp8_matches_oracle(backend, n, k, m):
     assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
+# 16 weights a lane (several rows), 32 (rows past 16384 long), 64 (one row); a row band and a K
+# block boundary inside a workgroup's rows and inside a wavefront
+@pytest.mark.parametrize("n,k", [(128, 128), (256, 1024), (384, 5120), (128, 17408), (128, 32768)])
+@pytest.mark.parametrize("m", [1, 2, 5])
+def test_gemm_fp8_block_matches_oracle(backend, n, k, m):
+    """gemm_fp8_block: one scale per 128 x 128 block of W (GemmFp8BlockRef).  The device multiplies a
+    lane's partial dot product by the block's scale where the reference scales every weight: same
+    bound as gemm_fp8.  A one-hot row gives scale * weight bit for bit."""
+    g = synth.rng(4100 * m + n + k)
+    codes, scales = synth.fp8_block_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_fp8_block(a, codes, scales, m, n, k)
+    da, dw, ds = backend.Upload(a), backend.Upload(codes), backend.Upload(scales)
+    dc = backend.AllocateBuffer(4 * m * n)
+    run(backend, "gemm_fp8_block", [da, dw, ds, dc], [m, n, k], grid=((m * n + 255) // 256, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    pos = sorted({min(p, k - 1) for p in (0, 127, 128, k // 2 + 3, k - 1)})[:m]
+    hot = synth.one_hot_rows(k, pos)
+    run(backend, "gemm_fp8_block", [backend.Upload(hot), dw, ds, dc], [len(pos), n, k])
+    backend.Synchronize()
+    got = backend.CopyD2H(dc, dtype=np.float32)[: len(pos) * n].reshape(len(pos), n)
+    assert same_bits_zero_sign_free(got, oracle.gemm_fp8_block(hot, codes, scales, len(pos), n, k))
+    with pytest.raises(StatusError) as e:   # n and k must be multiples of 128
+        run(backend, "gemm_fp8_block", [da, dw, ds, dc], [m, n, k - 64])
+    assert e.value.code == StatusCode.InvalidArgument
+
+
 @pytest.mark.parametrize("k", [512, 17408])
 def test_gemm_fp8_one_hot_bit_exact(backend, k):
     g = synth.rng(77)

@@ -84,6 +84,35 @@ def test_gemm_fp8():
     assert np.allclose(c, ref, rtol=0, atol=1e-4 * np.abs(ref).max())
 
 
+def test_gemm_fp8_block():
+    """One scale per 128 x 128 block: a one-hot row returns scale[block] * weight bit for bit (torch's
+    E4M3 decode, block picked by integer division written out here), a dense row stays within the
+    float64 product's rounding bound, and with every block of a row band given that band's row
+    scale the result equals gemm_fp8's bit for bit."""
+    g = synth.rng(31)
+    n, k = 256, 384
+    codes, scales = synth.fp8_block_weights(g, n, k)
+    wv = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).to(torch.float64).numpy().reshape(n, k)
+    sc = scales.reshape(n // 128, k // 128)
+    pos = [0, 127, 128, 200, 383]
+    c = oracle.gemm_fp8_block(synth.one_hot_rows(k, pos), codes, scales, len(pos), n, k)
+    for r, t in enumerate(pos):
+        per_row = np.repeat(sc[:, t // 128], 128)
+        want = (per_row * wv[:, t].astype(np.float32)).astype(np.float32)
+        assert np.array_equal(c[r].view(np.uint32), want.view(np.uint32))
+    a = synth.activations_f32(g, 2, k)
+    c = oracle.gemm_fp8_block(a, codes, scales, 2, n, k)
+    full = np.repeat(np.repeat(sc, 128, axis=0), 128, axis=1).astype(np.float64)
+    ref = a.astype(np.float64) @ (wv * full).T
+    assert np.allclose(c, ref, rtol=0, atol=1e-4 * np.abs(ref).max())
+    band = g.uniform(0.5, 2.0, n // 128).astype(np.float32)
+    uniform = np.repeat(band[:, None], k // 128, axis=1).reshape(-1)
+    assert np.array_equal(oracle.gemm_fp8_block(a, codes, uniform, 2, n, k),
+                          oracle.gemm_fp8(a, codes, np.repeat(band, 128), 2, n, k))
+    with pytest.raises(oracle.OracleError):
+        oracle.gemm_fp8_block(a[:, :320], codes[: n * 320], scales, 2, n, 320)   # k not a multiple of 128
+
+
 def test_quantize_fp8_invariants():
     g = synth.rng(4)
     rows, cols = 6, 512

@@ -64,6 +64,10 @@ def _load() -> C.CDLL:
         "orc_dequantize_mxfp4": (C.c_int, [u8p, f32p, sz, sz]),
         "orc_gemm_fp8_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
         "orc_gemm_fp8_block_ref": (C.c_int, [f32p, u8p, f32p, f32p, sz, sz, sz]),
+        "orc_quantize_q8": (C.c_int, [f32p, u8p, f32p, sz, sz]),
+        "orc_quantize_q4": (C.c_int, [f32p, u8p, f32p, sz, sz]),
+        "orc_attention_quant": (C.c_int, [f32p, u8p, u8p, f32p, f32p, f32p, sz, sz, sz, sz, sz, C.c_uint64, sz, C.c_int]),
+        "orc_cast_f32_f16": (None, [f32p, C.POINTER(C.c_uint16), sz]),
         "orc_permute_mxfp4_to_wmma": (C.c_int, [u8p, u8p, sz, sz]),
         "orc_rope": (C.c_int, [f32p, sz, sz, sz, sz, C.c_uint64, C.c_double]),
         "orc_mrope": (C.c_int, [f32p, C.POINTER(C.c_uint64), sz, sz, sz, sz, sz, sz, sz, C.c_double]),
@@ -398,6 +402,40 @@ def attention(q, k, v, m: int, n: int, heads: int, kv_heads: int, head_dim: int,
     _check(_lib.orc_attention(_p(q, C.c_float), k.ctypes.data_as(C.c_void_p), v.ctypes.data_as(C.c_void_p),
                               _p(out, C.c_float), m, n, heads, kv_heads, head_dim, q_base, window, int(kv_f16), int(causal)))
     return out.reshape(m, heads * head_dim)
+
+
+def quantize_kv(data, rows: int, cols: int, bits: int) -> tuple[np.ndarray, np.ndarray]:
+    """QuantizeQ8Ref (bits = 8: rows x cols bytes) / QuantizeQ4Ref (bits = 4: rows x cols/2 bytes);
+    returns (codes, one scale per row)."""
+    data = _f32(data).reshape(-1)
+    assert data.size == rows * cols and bits in (4, 8)
+    out = np.empty(rows * cols * bits // 8, dtype=np.uint8)
+    scale = np.empty(rows, dtype=np.float32)
+    fn = _lib.orc_quantize_q8 if bits == 8 else _lib.orc_quantize_q4
+    _check(fn(_p(data, C.c_float), _p(out, C.c_uint8), _p(scale, C.c_float), rows, cols))
+    return out, scale
+
+
+KV_KINDS = {"q8": 0, "q4": 1, "fp8": 2}
+
+
+def attention_quant(q, k, v, k_scale, v_scale, m: int, n: int, heads: int, kv_heads: int, head_dim: int, kind: str,
+                    q_base: int = 0, window: int = 0) -> np.ndarray:
+    """AttentionQ8Ref / AttentionQ4Ref / AttentionFp8Ref: k, v hold codes, one scale per key row."""
+    q, k, v, ks, vs = _f32(q).reshape(-1), _u8(k), _u8(v), _f32(k_scale), _f32(v_scale)
+    out = np.empty(m * heads * head_dim, dtype=np.float32)
+    _check(_lib.orc_attention_quant(_p(q, C.c_float), _p(k, C.c_uint8), _p(v, C.c_uint8), _p(ks, C.c_float),
+                                    _p(vs, C.c_float), _p(out, C.c_float), m, n, heads, kv_heads, head_dim, q_base, window,
+                                    KV_KINDS[kind]))
+    return out.reshape(m, heads * head_dim)
+
+
+def cast_f32_f16(data) -> np.ndarray:
+    """The "cast_f32_f16" built-in's conversion (significand cut toward zero); returns uint16 bits."""
+    data = _f32(data).reshape(-1)
+    out = np.empty(data.size, dtype=np.uint16)
+    _lib.orc_cast_f32_f16(_p(data, C.c_float), out.ctypes.data_as(C.POINTER(C.c_uint16)), data.size)
+    return out
 
 
 def qgate_split(fused, heads: int, head_dim: int, rows: int) -> tuple[np.ndarray, np.ndarray]:

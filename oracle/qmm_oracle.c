@@ -43,6 +43,12 @@
  *                                             causal / window mask built independently; one key =
  *                                             its value row)
  *   qgate_split ............................. pinned (numpy reshape)
+ *   quantize_q8 / quantize_q4 ............... pinned (float64 half-away rounding written with floor,
+ *                                             |x - q s| <= s / 2, extremes map to +-127 / +-7)
+ *   attention over int8 / 4-bit / E4M3 keys . pinned (numpy / torch decode of the codes fed to torch
+ *                                             softmax attention)
+ *   cast_f32_f16 (significand cut) .......... pinned (numpy float16 stepped toward zero when the
+ *                                             nearest value lies above the input)
  *
  * Status codes mirror tessera::StatusCode (include/tessera/types.hpp:36-48).
  */
@@ -888,6 +894,103 @@ int orc_attention(const float* q, const void* k, const void* v, float* out, size
   }
   free(kf), free(vf), free(scores);
   return ORC_OK;
+}
+
+/* ---- quantized key/value caches: symmetric per-row int8 (scale amax / 127) and 4-bit (amax / 7,
+ *      two codes a byte, low nibble first) with round half away from zero, an all-zero row taking
+ *      scale 1 (quant.cpp:123-178) ---- */
+int orc_quantize_q8(const float* in, uint8_t* out, float* scale, size_t rows, size_t cols) {
+  if (rows == 0 || cols == 0 || cols % 4 != 0) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    float amax = 0.0f;
+    for (size_t c = 0; c < cols; ++c) amax = fmaxf(amax, fabsf(in[r * cols + c]));
+    const float s = amax > 0.0f ? amax / 127.0f : 1.0f;
+    scale[r] = s;
+    for (size_t c = 0; c < cols; ++c) {
+      long q = lroundf(in[r * cols + c] / s);
+      q = q < -127 ? -127 : (q > 127 ? 127 : q);
+      out[r * cols + c] = (uint8_t)(int8_t)q;
+    }
+  }
+  return ORC_OK;
+}
+
+int orc_quantize_q4(const float* in, uint8_t* out, float* scale, size_t rows, size_t cols) {
+  if (rows == 0 || cols == 0 || cols % 8 != 0) return ORC_INVALID_ARGUMENT;
+  for (size_t r = 0; r < rows; ++r) {
+    float amax = 0.0f;
+    for (size_t c = 0; c < cols; ++c) amax = fmaxf(amax, fabsf(in[r * cols + c]));
+    const float s = amax > 0.0f ? amax / 7.0f : 1.0f;
+    scale[r] = s;
+    for (size_t c = 0; c < cols; c += 2) {
+      uint8_t packed = 0;
+      for (size_t h = 0; h < 2; ++h) {
+        long q = lroundf(in[r * cols + c + h] / s);
+        q = q < -7 ? -7 : (q > 7 ? 7 : q);
+        packed |= (uint8_t)(((uint8_t)q & 0xFu) << (4 * h));
+      }
+      out[r * cols / 2 + c / 2] = packed;
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- attention over a quantized cache: every key / value element is code * scale of its key row
+ *      (kind 0: int8, 1: signed 4-bit, two a byte, 2: E4M3), then orc_attention, causal
+ *      (attention.cpp:45-121) ---- */
+int orc_attention_quant(const float* q, const uint8_t* k, const uint8_t* v, const float* k_scale, const float* v_scale,
+                        float* out, size_t m, size_t n, size_t heads, size_t kv_heads, size_t head_dim, uint64_t q_base,
+                        size_t window, int kind) {
+  if (m == 0 || n == 0 || heads == 0 || kv_heads == 0 || head_dim == 0 || heads % kv_heads != 0 || kind < 0 || kind > 2) {
+    return ORC_INVALID_ARGUMENT;
+  }
+  const size_t width = kv_heads * head_dim, count = n * width;
+  float* kf = (float*)malloc(count * sizeof(float));
+  float* vf = (float*)malloc(count * sizeof(float));
+  if (!kf || !vf) {
+    free(kf), free(vf);
+    return ORC_OOM;
+  }
+  for (size_t j = 0; j < n; ++j) {
+    for (size_t d = 0; d < width; ++d) {
+      const size_t i = j * width + d;
+      float kc, vc;
+      if (kind == 0) {
+        kc = (float)(int8_t)k[i], vc = (float)(int8_t)v[i];
+      } else if (kind == 1) {
+        int kn = (k[i / 2] >> ((i % 2) * 4)) & 0xF, vn = (v[i / 2] >> ((i % 2) * 4)) & 0xF;
+        kc = (float)((kn & 8) ? kn - 16 : kn), vc = (float)((vn & 8) ? vn - 16 : vn);
+      } else {
+        kc = orc_fp8_e4m3_to_float(k[i]), vc = orc_fp8_e4m3_to_float(v[i]);
+      }
+      kf[i] = kc * k_scale[j], vf[i] = vc * v_scale[j];
+    }
+  }
+  const int rc = orc_attention(q, kf, vf, out, m, n, heads, kv_heads, head_dim, q_base, window, 0, 1);
+  free(kf), free(vf);
+  return rc;
+}
+
+/* ---- fp32 -> binary16 as the "cast_f32_f16" built-in does it: the significand is cut, not rounded
+ *      (toward zero), magnitudes of 2^16 and more -- and NaN -- give infinity, magnitudes below
+ *      2^-24 give zero (src/backends/rocm/rocm_kernels.hpp:26-45) ---- */
+uint16_t orc_float_to_fp16_cut(float value) {
+  uint32_t bits;
+  memcpy(&bits, &value, sizeof(bits));
+  const uint32_t sign = (bits >> 16) & 0x8000u;
+  const int exponent = (int)((bits >> 23) & 0xFFu) - 127;
+  uint32_t mantissa = bits & 0x7FFFFFu;
+  if (exponent > 15) return (uint16_t)(sign | 0x7C00u);
+  if (exponent < -24) return (uint16_t)sign;
+  if (exponent < -14) {
+    mantissa |= 0x800000u;
+    return (uint16_t)(sign | (mantissa >> (uint32_t)(-exponent - 14 + 13)));
+  }
+  return (uint16_t)(sign | ((uint32_t)(exponent + 15) << 10) | (mantissa >> 13));
+}
+
+void orc_cast_f32_f16(const float* in, uint16_t* out, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = orc_float_to_fp16_cut(in[i]);
 }
 
 /* ---- fused gated-attention projection (rows x heads x [query | gate]) -> queries, gates

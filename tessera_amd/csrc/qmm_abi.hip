@@ -379,6 +379,66 @@ qmm_status run_attention(const LaunchCtx& c) {
                                        heads, kv_heads, head_dim, q_base, row_base, window, kv_f16 == 1, causal == 1, c.stream));
 }
 
+// "attention_q8", "attention_q4", "attention_fp8": buffers q, K and V codes (n x kv_heads*head_dim int8
+// / nibbles, two a byte / E4M3), one fp32 scale per key row for K and for V, out; scalars m, n, heads,
+// kv_heads, head_dim, q_base, row_base, window, kind (0..2; the id fixes the decode, as in the
+// reference's kernels) (include/tessera/backend.hpp:284-309,679-691; always causal).
+qmm_status run_attention_quant(const LaunchCtx& c, uint32_t kind) {
+  if (!counts(c, 6, 9)) return bad("attention_q8/q4/fp8: expects 6 buffers and 9 scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], heads = c.sc[2], kv_heads = c.sc[3], head_dim = c.sc[4], q_base = c.sc[5],
+                 row_base = c.sc[6], window = c.sc[7];
+  if (m == 0 || n == 0 || heads == 0 || kv_heads == 0 || head_dim == 0 || heads % kv_heads != 0 || c.sc[8] > 2) {
+    return bad("attention_q8/q4/fp8: m, n, heads, kv_heads, head_dim must be non-zero, heads a multiple of kv_heads, kind 0..2");
+  }
+  if (head_dim > 256) return bad("attention_q8/q4/fp8: head_dim must be at most 256");
+  if (kind == 1 && (kv_heads * head_dim) % 2 != 0) return bad("attention_q4: a key row must hold an even number of codes");
+  if (m > (1u << 24) || n > (1ull << 32) || heads > (1u << 16) || row_base > (1ull << 32) || q_base > (1ull << 40) ||
+      m * heads > 0x7FFFFFFFull) {
+    return bad("attention_q8/q4/fp8: a scalar is out of range");
+  }
+  const u128 q_bytes = static_cast<u128>(row_base + m) * heads * head_dim * 4;
+  const u128 codes = static_cast<u128>(n) * kv_heads * head_dim;
+  const u128 kv_bytes = kind == 1 ? codes / 2 : codes;
+  if (!c.fits(0, q_bytes) || !c.fits(1, kv_bytes) || !c.fits(2, kv_bytes) || !c.fits(3, static_cast<u128>(n) * 4) ||
+      !c.fits(4, static_cast<u128>(n) * 4) || !c.fits(5, q_bytes)) {
+    return bad("attention_q8/q4/fp8: a buffer is smaller than the scalars require");
+  }
+  return map_hip(qmm::launch_attention_quant(c.ptr<const float>(0), c.ptr<const void>(1), c.ptr<const void>(2),
+                                             c.ptr<const float>(3), c.ptr<const float>(4), c.ptr<float>(5), m, n, heads,
+                                             kv_heads, head_dim, q_base, row_base, window, kind, c.stream));
+}
+qmm_status run_attention_q8(const LaunchCtx& c) { return run_attention_quant(c, 0); }
+qmm_status run_attention_q4(const LaunchCtx& c) { return run_attention_quant(c, 1); }
+qmm_status run_attention_fp8(const LaunchCtx& c) { return run_attention_quant(c, 2); }
+
+// "quantize_q8" / "quantize_q4": buffers In (rows x cols fp32), Out (int8 codes / 4-bit codes, two a
+// byte), one fp32 scale per row; scalars rows, cols (a multiple of 4 / of 8)
+// (include/tessera/backend.hpp:280-283,292-295,670-678,706-714).
+qmm_status run_quantize_kv(const LaunchCtx& c, uint32_t bits) {
+  if (!counts(c, 3, 2)) return bad("quantize_q8/q4: expects 3 buffers and 2 scalars");
+  const uint64_t rows = c.sc[0], cols = c.sc[1];
+  if (rows == 0 || cols == 0 || cols % (bits == 8 ? 4 : 8) != 0 || rows > 0x7FFFFFFFull || cols > (1ull << 32)) {
+    return bad("quantize_q8/q4: rows and cols must be non-zero, cols a multiple of 4 (q8) or 8 (q4)");
+  }
+  if (!c.fits(0, static_cast<u128>(rows) * cols * 4) || !c.fits(1, static_cast<u128>(rows) * cols * bits / 8) ||
+      !c.fits(2, static_cast<u128>(rows) * 4)) {
+    return bad("quantize_q8/q4: a buffer is smaller than rows and cols require");
+  }
+  return map_hip(qmm::launch_quantize_kv(c.ptr<const float>(0), c.ptr<uint8_t>(1), c.ptr<float>(2), rows, cols, bits, c.stream));
+}
+qmm_status run_quantize_q8(const LaunchCtx& c) { return run_quantize_kv(c, 8); }
+qmm_status run_quantize_q4(const LaunchCtx& c) { return run_quantize_kv(c, 4); }
+
+// "cast_f32_f16": buffers In (n fp32), Out (n binary16, two per 32-bit word); scalar n, even
+// (include/tessera/backend.hpp:334-336,732-740).
+qmm_status run_cast_f32_f16(const LaunchCtx& c) {
+  if (!counts(c, 2, 1)) return bad("cast_f32_f16: expects 2 buffers and 1 scalar");
+  const uint64_t n = c.sc[0];
+  if (n == 0 || n % 2 != 0 || n > (1ull << 40)) return bad("cast_f32_f16: n must be non-zero and even");
+  if (!c.fits(0, static_cast<u128>(n) * 4) || !c.fits(1, static_cast<u128>(n) * 2)) return bad("cast_f32_f16: a buffer is smaller than n requires");
+  return map_hip(qmm::launch_cast_f32_f16(c.ptr<const float>(0), c.ptr<void>(1), n, c.stream));
+}
+
 // "qgate_split": buffers Fused (rows x heads x 2*head_dim: per head the query then the gate), Q, G
 // (rows x heads*head_dim each); scalars heads, head_dim, rows (include/tessera/backend.hpp:386-390,819-826).
 qmm_status run_qgate_split(const LaunchCtx& c) {
@@ -1015,6 +1075,12 @@ const Entry kTable[] = {
     {"rope", run_rope},
     {"mrope", run_mrope},
     {"attention", run_attention},
+    {"attention_q8", run_attention_q8},
+    {"attention_q4", run_attention_q4},
+    {"attention_fp8", run_attention_fp8},
+    {"quantize_q8", run_quantize_q8},
+    {"quantize_q4", run_quantize_q4},
+    {"cast_f32_f16", run_cast_f32_f16},
     {"qgate_split", run_qgate_split},
     {"embedding_f32", run_embedding_f32},
     {"embedding_bf16", run_embedding_bf16},

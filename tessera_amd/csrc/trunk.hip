@@ -37,9 +37,15 @@ __global__ __launch_bounds__(256) void rope_kernel(float* __restrict__ data, con
 // thread e accumulates weight * v[key][e] (coalesced value reads): the usual running softmax, so
 // the result differs from AttentionRef (src/core/numerics/attention.cpp:158-225) in summation
 // order only.
-template <bool F16>
+// KV: how keys and values are stored.  The quantized kinds hold codes and one fp32 scale per key
+// row (all kv heads of a position), and an element is code * scale as in AttentionQ8Ref /
+// AttentionQ4Ref / AttentionFp8Ref (src/core/numerics/attention.cpp:45-121).
+enum class KvKind { F32, F16, Q8, Q4, Fp8 };
+
+template <KvKind KV>
 __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ q, const void* __restrict__ k,
-                                                        const void* __restrict__ v, float* __restrict__ out, uint64_t n,
+                                                        const void* __restrict__ v, const float* __restrict__ k_scale,
+                                                        const float* __restrict__ v_scale, float* __restrict__ out, uint64_t n,
                                                         uint64_t heads, uint64_t kv_heads, uint64_t head_dim, uint64_t q_base,
                                                         uint64_t row_base, uint64_t window, uint64_t causal) {
   constexpr uint32_t kKeys = 64;
@@ -55,9 +61,19 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   }
   const float scale = 1.0f / sqrtf(static_cast<float>(head_dim));
   const uint64_t qb = ((row_base + i) * heads + h) * head_dim;
-  auto kv_at = [&](const void* base, uint64_t idx) {
-    if constexpr (F16) return half_bits_to_float(static_cast<const uint16_t*>(base)[idx]);
-    else return static_cast<const float*>(base)[idx];
+  auto kv_at = [&](const void* base, const float* row_scale, uint64_t key, uint64_t idx) {
+    if constexpr (KV == KvKind::F16) {
+      return half_bits_to_float(static_cast<const uint16_t*>(base)[idx]);
+    } else if constexpr (KV == KvKind::F32) {
+      return static_cast<const float*>(base)[idx];
+    } else if constexpr (KV == KvKind::Q8) {
+      return static_cast<float>(static_cast<const int8_t*>(base)[idx]) * row_scale[key];
+    } else if constexpr (KV == KvKind::Q4) {
+      const int nib = (static_cast<const uint8_t*>(base)[idx >> 1] >> ((idx & 1u) * 4u)) & 0xF;
+      return static_cast<float>((nib & 8) ? nib - 16 : nib) * row_scale[key];
+    } else {
+      return e4m3_to_float(static_cast<const uint8_t*>(base)[idx]) * row_scale[key];
+    }
   };
   float qr[4];                       // head_dim <= 256: up to four elements a lane
 #pragma unroll
@@ -72,7 +88,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
         const uint64_t kb = ((j0 + kk) * kv_heads + kv) * head_dim;
 #pragma unroll
         for (int cc = 0; cc < 4; ++cc) {
-          if (lane + 64u * cc < head_dim) dot = fmaf(qr[cc], kv_at(k, kb + lane + 64u * cc), dot);
+          if (lane + 64u * cc < head_dim) dot = fmaf(qr[cc], kv_at(k, k_scale, j0 + kk, kb + lane + 64u * cc), dot);
         }
       }
       dot = wave_sum(dot);
@@ -97,7 +113,9 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     run_max = m_new;
     if (t < head_dim) {
       float a = 0.0f;
-      for (uint32_t kk = 0; kk < count; ++kk) a = fmaf(wt[kk], kv_at(v, ((j0 + kk) * kv_heads + kv) * head_dim + t), a);
+      for (uint32_t kk = 0; kk < count; ++kk) {
+        a = fmaf(wt[kk], kv_at(v, v_scale, j0 + kk, ((j0 + kk) * kv_heads + kv) * head_dim + t), a);
+      }
       acc = fmaf(corr, acc, a);
     }
     __syncthreads();
@@ -112,6 +130,61 @@ __global__ __launch_bounds__(256) void qgate_split_kernel(const float* __restric
   const uint64_t rh = i / head_dim, e = i % head_dim;
   q[i] = fused[rh * 2 * head_dim + e];
   gate[i] = fused[rh * 2 * head_dim + head_dim + e];
+}
+
+// Per-row symmetric quantizer of the quantized key/value caches (QuantizeQ8Ref / QuantizeQ4Ref,
+// src/core/numerics/quant.cpp:123-178): scale = amax / QMAX (1 for an all-zero row), code =
+// x / scale rounded half away from zero and clamped to +-QMAX; int8 codes a byte each, 4-bit codes
+// two a byte, low nibble first.  One workgroup per row.
+template <int BITS>
+__global__ __launch_bounds__(256) void quantize_kv_kernel(const float* __restrict__ in, uint8_t* __restrict__ out,
+                                                          float* __restrict__ scale, uint64_t cols) {
+  constexpr float kMax = BITS == 8 ? 127.0f : 7.0f;
+  __shared__ float red[4];
+  const uint32_t t = threadIdx.x;
+  const float* row = in + static_cast<size_t>(blockIdx.x) * cols;
+  float amax = 0.0f;
+  for (uint64_t c = t; c < cols; c += 256u) amax = fmaxf(amax, fabsf(row[c]));
+  amax = wave_max(amax);
+  if ((t & 63u) == 0) red[t >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float s = amax > 0.0f ? amax / kMax : 1.0f;
+  if (t == 0) scale[blockIdx.x] = s;
+  auto code = [&](float x) {
+    const float r = roundf(x / s);                       // half away from zero, as lround
+    return static_cast<int>(fminf(fmaxf(r, -kMax), kMax));
+  };
+  if constexpr (BITS == 8) {
+    uint8_t* dst = out + static_cast<size_t>(blockIdx.x) * cols;
+    for (uint64_t c = t; c < cols; c += 256u) dst[c] = static_cast<uint8_t>(static_cast<int8_t>(code(row[c])));
+  } else {
+    uint8_t* dst = out + static_cast<size_t>(blockIdx.x) * (cols / 2);
+    for (uint64_t c = t; c < cols / 2; c += 256u) {
+      dst[c] = static_cast<uint8_t>((code(row[2 * c]) & 0xF) | ((code(row[2 * c + 1]) & 0xF) << 4));
+    }
+  }
+}
+
+// fp32 -> binary16 with the significand cut toward zero, magnitudes from 2^16 up (and NaN) to
+// infinity, below 2^-24 to zero: the conversion of the "cast_f32_f16" built-in
+// (src/backends/rocm/rocm_kernels.hpp:26-45), not the hardware's round-to-nearest.
+__device__ __forceinline__ uint32_t float_to_fp16_cut(float value) {
+  const uint32_t bits = bit_cast<uint32_t>(value);
+  const uint32_t sign = (bits >> 16) & 0x8000u;
+  const int exponent = static_cast<int>((bits >> 23) & 0xFFu) - 127;
+  const uint32_t mantissa = bits & 0x7FFFFFu;
+  if (exponent > 15) return sign | 0x7C00u;
+  if (exponent < -24) return sign;
+  if (exponent < -14) return sign | ((mantissa | 0x800000u) >> static_cast<uint32_t>(-exponent - 1));
+  return sign | (static_cast<uint32_t>(exponent + 15) << 10) | (mantissa >> 13);
+}
+
+__global__ __launch_bounds__(256) void cast_f32_f16_kernel(const float* __restrict__ in, uint32_t* __restrict__ out, uint64_t pairs) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (i >= pairs) return;
+  const float2 v = reinterpret_cast<const float2*>(in)[i];
+  out[i] = float_to_fp16_cut(v.x) | (float_to_fp16_cut(v.y) << 16);
 }
 
 dim3 blocks_for(uint64_t count) { return dim3(static_cast<uint32_t>((count + 255) / 256)); }
@@ -129,13 +202,44 @@ hipError_t launch_attention(const float* q, const void* k, const void* v, float*
                             uint64_t kv_heads, uint64_t head_dim, uint64_t q_base, uint64_t row_base, uint64_t window,
                             bool kv_f16, bool causal, hipStream_t stream) {
   const dim3 grid(static_cast<uint32_t>(m * heads));
+  const float* none = nullptr;
   if (kv_f16) {
-    hipLaunchKernelGGL(attention_kernel<true>, grid, dim3(256), 0, stream, q, k, v, out, n, heads, kv_heads, head_dim, q_base,
-                       row_base, window, causal ? 1ull : 0ull);
+    hipLaunchKernelGGL(attention_kernel<KvKind::F16>, grid, dim3(256), 0, stream, q, k, v, none, none, out, n, heads, kv_heads,
+                       head_dim, q_base, row_base, window, causal ? 1ull : 0ull);
   } else {
-    hipLaunchKernelGGL(attention_kernel<false>, grid, dim3(256), 0, stream, q, k, v, out, n, heads, kv_heads, head_dim, q_base,
-                       row_base, window, causal ? 1ull : 0ull);
+    hipLaunchKernelGGL(attention_kernel<KvKind::F32>, grid, dim3(256), 0, stream, q, k, v, none, none, out, n, heads, kv_heads,
+                       head_dim, q_base, row_base, window, causal ? 1ull : 0ull);
   }
+  return hipGetLastError();
+}
+
+// kind: 0 int8, 1 4-bit, 2 E4M3 keys and values with one scale per key row; always causal.
+hipError_t launch_attention_quant(const float* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                  float* out, uint64_t m, uint64_t n, uint64_t heads, uint64_t kv_heads, uint64_t head_dim,
+                                  uint64_t q_base, uint64_t row_base, uint64_t window, uint32_t kind, hipStream_t stream) {
+  const dim3 grid(static_cast<uint32_t>(m * heads));
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, q, k, v, k_scale, v_scale, out, n, heads, kv_heads, head_dim, q_base,
+                       row_base, window, 1ull);
+  };
+  if (kind == 0) go(attention_kernel<KvKind::Q8>);
+  else if (kind == 1) go(attention_kernel<KvKind::Q4>);
+  else go(attention_kernel<KvKind::Fp8>);
+  return hipGetLastError();
+}
+
+hipError_t launch_quantize_kv(const float* in, uint8_t* out, float* scale, uint64_t rows, uint64_t cols, uint32_t bits,
+                              hipStream_t stream) {
+  if (bits == 8) {
+    hipLaunchKernelGGL(quantize_kv_kernel<8>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, in, out, scale, cols);
+  } else {
+    hipLaunchKernelGGL(quantize_kv_kernel<4>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, in, out, scale, cols);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_cast_f32_f16(const float* in, void* out, uint64_t n, hipStream_t stream) {
+  hipLaunchKernelGGL(cast_f32_f16_kernel, blocks_for(n / 2), dim3(256), 0, stream, in, static_cast<uint32_t*>(out), n / 2);
   return hipGetLastError();
 }
 

@@ -173,7 +173,7 @@ int main(int argc, char** argv) {
     return 2;
   }
   // Error behaviour of the reference interface.
-  if (auto k = backend->LoadKernel("attention_q8"); k || k.error() != StatusCode::UnsupportedFeature) return 4;
+  if (auto k = backend->LoadKernel("delta_step_heads"); k || k.error() != StatusCode::UnsupportedFeature) return 4;
   const std::byte blob[4] = {};
   if (auto k = backend->LoadKernel("gemm_q4k", std::span<const std::byte>(blob)); k || k.error() != StatusCode::UnsupportedFeature) return 4;
   if (auto b = backend->AllocateBuffer(0); b || b.error() != StatusCode::InvalidArgument) return 4;

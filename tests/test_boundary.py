@@ -24,7 +24,8 @@ REFERENCE_IDS = [
     "gemm_q6k_rows5", "gemm_q6k_batched", "gemm_q5k", "gemm_q5k_vec", "gemm_q5k_rows2", "gemm_q5k_rows3",
     "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched", "moe_experts_down_q6k", "gemm_q5k_wmma", "gemm_q6k_wmma",
     "silu_mul", "round_bf16", "add", "fill", "rmsnorm", "embedding_f32", "embedding_bf16", "embedding_q4k",
-    "rope", "mrope", "attention", "qgate_split",
+    "rope", "mrope", "attention", "qgate_split", "attention_q8", "attention_q4", "attention_fp8", "quantize_q8",
+    "quantize_q4", "cast_f32_f16",
 ]
 
 
@@ -53,7 +54,7 @@ def test_kernel_table_and_unknown_ids_without_a_device():
     for kid in REFERENCE_IDS:
         assert kid in names
         assert b.LoadKernel(kid).Id() == kid
-    for kid in ("gemm_q3k", "attention_q8", "", "gemm_q4k "):
+    for kid in ("gemm_q3k", "delta_step_heads", "", "gemm_q4k "):
         with pytest.raises(StatusError) as e:
             b.LoadKernel(kid)
         assert e.value.code == StatusCode.UnsupportedFeature   # callers fall through on this code

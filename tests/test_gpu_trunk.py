@@ -100,3 +100,75 @@ def test_qgate_split(backend):
     want_q, want_g = oracle.qgate_split(fused, heads, head_dim, rows)
     assert np.array_equal(backend.CopyD2H(dq, dtype=np.float32), want_q)
     assert np.array_equal(backend.CopyD2H(dg, dtype=np.float32), want_g)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 1024), (33, 2056)])
+def test_quantize_kv_bit_exact(backend, bits, rows, cols):
+    """quantize_q8 / quantize_q4 (the quantized cache's per-row quantizers): codes and scales equal
+    QuantizeQ8Ref / QuantizeQ4Ref bit for bit, with an all-zero row, exact ties and an outlier."""
+    g = synth.rng(rows * 10 + cols + bits)
+    x = g.standard_normal((rows, cols)).astype(np.float32) * np.float32(2.5)
+    x[0] = 0.0
+    x[0, :8] = np.array([0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 127.0 if bits == 8 else 7.0, -1.0], np.float32)   # scale 1: exact ties
+    if rows > 2:
+        x[1] = 0.0
+        x[2, cols // 2] = 300.0
+    want_codes, want_scale = oracle.quantize_kv(x, rows, cols, bits)
+    din = backend.Upload(x)
+    dout, dscale = backend.AllocateBuffer(rows * cols * bits // 8), backend.AllocateBuffer(4 * rows)
+    run(backend, "quantize_q8" if bits == 8 else "quantize_q4", [din, dout, dscale], [rows, cols], grid=(rows, 1, 1))
+    backend.Synchronize()
+    assert np.array_equal(backend.CopyD2H(dscale, dtype=np.float32), want_scale)
+    assert np.array_equal(backend.CopyD2H(dout), want_codes)
+    with pytest.raises(StatusError) as e:
+        run(backend, "quantize_q8" if bits == 8 else "quantize_q4", [din, dout, dscale], [rows, cols + 2])
+    assert e.value.code == StatusCode.InvalidArgument
+
+
+@pytest.mark.parametrize("kind", ["q8", "q4", "fp8"])
+@pytest.mark.parametrize("m,n,heads,kv_heads,head_dim,q_base,window", [(5, 12, 4, 2, 32, 7, 0), (3, 200, 8, 8, 64, 197, 50),
+                                                                        (1, 130, 6, 2, 128, 129, 0), (2, 70, 2, 1, 256, 68, 0)])
+def test_attention_over_a_quantized_cache(backend, kind, m, n, heads, kv_heads, head_dim, q_base, window):
+    """attention_q8 / attention_q4 / attention_fp8: a cache written by the matching quantizer, read back
+    by the attention id, against AttentionQ8Ref / Q4Ref / Fp8Ref (summation order differs)."""
+    g = synth.rng(m * 7 + n + len(kind) * 1000)
+    width = kv_heads * head_dim
+    q = g.standard_normal((m, heads * head_dim)).astype(np.float32)
+    kf = g.standard_normal((n, width)).astype(np.float32)
+    vf = g.standard_normal((n, width)).astype(np.float32)
+    if kind == "fp8":
+        k, ks = oracle.quantize_fp8_pack(kf, n, width)
+        v, vs = oracle.quantize_fp8_pack(vf, n, width)
+    else:
+        k, ks = oracle.quantize_kv(kf, n, width, 8 if kind == "q8" else 4)
+        v, vs = oracle.quantize_kv(vf, n, width, 8 if kind == "q8" else 4)
+    want = oracle.attention_quant(q, k, v, ks, vs, m, n, heads, kv_heads, head_dim, kind, q_base, window)
+    row_base, total = 1, m + 3
+    qbuf = np.zeros((total, heads * head_dim), np.float32)
+    qbuf[row_base:row_base + m] = q
+    bufs = [backend.Upload(qbuf), backend.Upload(k), backend.Upload(v), backend.Upload(ks), backend.Upload(vs),
+            backend.Upload(np.full((total, heads * head_dim), 7.0, np.float32))]
+    run(backend, "attention_" + kind, bufs, [m, n, heads, kv_heads, head_dim, q_base, row_base, window, oracle.KV_KINDS[kind]],
+        grid=(m * heads, 1, 1))
+    backend.Synchronize()
+    got = backend.CopyD2H(bufs[5], dtype=np.float32).reshape(total, heads * head_dim)
+    assert np.max(np.abs(got[row_base:row_base + m] - want)) <= 2e-6 * max(1.0, np.max(np.abs(want)))
+    assert np.all(got[:row_base] == 7.0) and np.all(got[row_base + m:] == 7.0)
+    with pytest.raises(StatusError) as e:   # kind above 2
+        run(backend, "attention_" + kind, bufs, [m, n, heads, kv_heads, head_dim, q_base, row_base, window, 3])
+    assert e.value.code == StatusCode.InvalidArgument
+
+
+def test_cast_f32_f16_bit_exact(backend):
+    g = synth.rng(78)
+    x = np.concatenate([g.standard_normal(5000).astype(np.float32) * np.float32(10.0) ** g.integers(-9, 6, 5000).astype(np.float32),
+                        np.array([0.0, -0.0, 1.0, 65504.0, 65519.9, 65535.9, 65536.0, -70000.0, 2.0 ** -24, 2.0 ** -25,
+                                  2.0 ** -14, np.inf, -np.inf, np.nan], np.float32)])
+    din, dout = backend.Upload(x), backend.AllocateBuffer(2 * x.size)
+    run(backend, "cast_f32_f16", [din, dout], [x.size], grid=((x.size // 2 + 255) // 256, 1, 1))
+    backend.Synchronize()
+    assert np.array_equal(backend.CopyD2H(dout, dtype=np.uint16), oracle.cast_f32_f16(x))
+    with pytest.raises(StatusError) as e:   # n must be even
+        run(backend, "cast_f32_f16", [din, dout], [x.size - 1])
+    assert e.value.code == StatusCode.InvalidArgument

@@ -1,6 +1,7 @@
 """Pins the oracle's restatements of the non-matmul trunk pieces that sit around the projections:
-RopeRef, MropeRef, AttentionRef (fp32 and fp16 keys/values), QGateSplitRef
-(src/core/numerics/attention.cpp)."""
+RopeRef, MropeRef, AttentionRef (fp32 and fp16 keys/values), QGateSplitRef, the quantized key/value
+caches (QuantizeQ8Ref, QuantizeQ4Ref, AttentionQ8Ref / Q4Ref / Fp8Ref) and the cast_f32_f16 conversion
+(src/core/numerics/attention.cpp, quant.cpp:123-178, src/backends/rocm/rocm_kernels.hpp:26-45)."""
 import numpy as np
 import pytest
 import torch
@@ -109,3 +110,86 @@ def test_qgate_split():
     q, gate = oracle.qgate_split(fused, heads, head_dim, rows)
     assert np.array_equal(q.reshape(rows, heads, head_dim), fused[:, :, 0])
     assert np.array_equal(gate.reshape(rows, heads, head_dim), fused[:, :, 1])
+
+
+def half_away(x):
+    """Round half away from zero, float64, written with floor (not the library's round)."""
+    return np.sign(x) * np.floor(np.abs(x) + 0.5)
+
+
+@pytest.mark.parametrize("bits,qmax", [(8, 127), (4, 7)])
+def test_quantize_kv(bits, qmax):
+    g = synth.rng(40 + bits)
+    rows, cols = 7, 96
+    x = g.standard_normal((rows, cols)).astype(np.float32) * np.float32(3.0)
+    x[2] = 0.0                                                   # all-zero row: scale 1, codes 0
+    x[3, 5] = 50.0                                               # one outlier sets the scale
+    x[4, :8] = np.array([0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.49, -0.49], np.float32)
+    x[4, 8] = np.float32(qmax)                                   # amax = qmax: scale exactly 1, the values above are exact ties
+    x[4, 9:] = 0.0
+    codes, scale = oracle.quantize_kv(x, rows, cols, bits)
+    amax = np.abs(x).max(axis=1)
+    want_scale = np.where(amax > 0, (amax / np.float32(qmax)).astype(np.float32), np.float32(1.0))
+    assert np.array_equal(scale, want_scale)
+    if bits == 8:
+        q = codes.view(np.int8).reshape(rows, cols).astype(np.int64)
+    else:
+        nib = np.stack([codes & 0xF, codes >> 4], axis=-1).reshape(rows, cols).astype(np.int64)
+        q = np.where(nib >= 8, nib - 16, nib)
+    want = np.clip(half_away((x / scale[:, None]).astype(np.float32).astype(np.float64)), -qmax, qmax).astype(np.int64)
+    assert np.array_equal(q, want)
+    assert np.all(np.abs(q * scale[:, None].astype(np.float64) - x) <= scale[:, None] * 0.5000001)
+    assert np.all(np.abs(q).max(axis=1)[amax > 0] == qmax) and np.all(q[2] == 0)
+    assert scale[4] == 1.0 and q[4, :8].tolist() == [1, -1, 2, -2, 3, -3, 0, 0]
+    with pytest.raises(oracle.OracleError):
+        oracle.quantize_kv(x[:, :94], rows, 94, bits)           # cols not a multiple of 4 / 8
+
+
+@pytest.mark.parametrize("kind", ["q8", "q4", "fp8"])
+@pytest.mark.parametrize("m,n,heads,kv_heads,head_dim,q_base,window", [(4, 20, 4, 2, 32, 16, 0), (2, 33, 6, 6, 16, 40, 8)])
+def test_attention_quant(kind, m, n, heads, kv_heads, head_dim, q_base, window):
+    """The codes are decoded here with numpy / torch views (int8 view, nibble arithmetic, torch's E4M3) and
+    fed to the torch attention; the oracle must agree to summation order."""
+    g = synth.rng(m + n + len(kind))
+    width = kv_heads * head_dim
+    q = g.standard_normal((m, heads * head_dim)).astype(np.float32)
+    ks = g.uniform(0.005, 0.02, n).astype(np.float32)
+    vs = g.uniform(0.005, 0.02, n).astype(np.float32)
+    if kind == "q4":
+        k = g.integers(0, 256, n * width // 2, dtype=np.uint8)
+        v = g.integers(0, 256, n * width // 2, dtype=np.uint8)
+        def dec(c):
+            nib = np.stack([c & 0xF, c >> 4], axis=-1).reshape(n, width).astype(np.int64)
+            return np.where(nib >= 8, nib - 16, nib).astype(np.float64)
+    elif kind == "q8":
+        k = g.integers(0, 256, n * width, dtype=np.uint8)
+        v = g.integers(0, 256, n * width, dtype=np.uint8)
+        dec = lambda c: c.view(np.int8).reshape(n, width).astype(np.float64)
+    else:
+        k = g.integers(0, 0x7F, n * width, dtype=np.uint8) | (g.integers(0, 2, n * width, dtype=np.uint8) << 7)   # no NaN codes
+        v = g.integers(0, 0x7F, n * width, dtype=np.uint8) | (g.integers(0, 2, n * width, dtype=np.uint8) << 7)
+        dec = lambda c: torch.from_numpy(c.copy()).view(torch.float8_e4m3fn).to(torch.float64).numpy().reshape(n, width)
+    got = oracle.attention_quant(q, k, v, ks, vs, m, n, heads, kv_heads, head_dim, kind, q_base, window)
+    kf = (dec(k).astype(np.float32) * ks[:, None]).astype(np.float32)
+    vf = (dec(v).astype(np.float32) * vs[:, None]).astype(np.float32)
+    want = torch_attention(q, kf, vf, m, n, heads, kv_heads, head_dim, q_base, window, True)
+    assert np.max(np.abs(got - want)) <= 2e-6 * max(1.0, np.max(np.abs(want)))
+    assert np.array_equal(got, oracle.attention(q, kf, vf, m, n, heads, kv_heads, head_dim, q_base, window, False, True))
+
+
+def test_cast_f32_f16_cuts_the_significand():
+    """Toward zero: numpy's nearest binary16, stepped one value toward zero where it lies above the
+    input in magnitude; 2^16 and more (and NaN) give infinity, below 2^-24 zero."""
+    g = synth.rng(77)
+    x = np.concatenate([g.standard_normal(4000).astype(np.float32) * np.float32(10.0) ** g.integers(-9, 5, 4000).astype(np.float32),
+                        np.array([0.0, -0.0, 1.0, 65504.0, 65519.9, 65535.9, 65536.0, -70000.0, 2.0 ** -24, 2.0 ** -25,
+                                  -(2.0 ** -24) * 1.5, 2.0 ** -14, 2.0 ** -14 * 0.999, np.inf, -np.inf], np.float32)])
+    got = oracle.cast_f32_f16(x)
+    with np.errstate(over="ignore"):
+        near = x.astype(np.float16)
+    above = np.abs(near.astype(np.float64)) > np.abs(x.astype(np.float64))
+    cut = np.where(above, np.nextafter(near, np.float16(0.0)), near)
+    big = np.abs(x) >= 65536.0
+    want = np.where(big, np.where(np.signbit(x), np.float16(-np.inf), np.float16(np.inf)), cut).astype(np.float16)
+    assert np.array_equal(got, want.view(np.uint16))
+    assert oracle.cast_f32_f16(np.array([np.nan], np.float32))[0] & 0x7FFF == 0x7C00     # NaN becomes infinity

@@ -68,6 +68,8 @@ def _load() -> C.CDLL:
         "orc_quantize_q4": (C.c_int, [f32p, u8p, f32p, sz, sz]),
         "orc_attention_quant": (C.c_int, [f32p, u8p, u8p, f32p, f32p, f32p, sz, sz, sz, sz, sz, C.c_uint64, sz, C.c_int]),
         "orc_cast_f32_f16": (None, [f32p, C.POINTER(C.c_uint16), sz]),
+        "orc_attention_split": (C.c_int, [f32p, f32p, f32p, f32p, f32p, f32p, sz, sz, sz, sz, sz, C.c_uint64, sz, C.c_int, sz]),
+        "orc_attention_combine": (C.c_int, [f32p, f32p, f32p, f32p, sz, sz, sz, sz]),
         "orc_permute_mxfp4_to_wmma": (C.c_int, [u8p, u8p, sz, sz]),
         "orc_rope": (C.c_int, [f32p, sz, sz, sz, sz, C.c_uint64, C.c_double]),
         "orc_mrope": (C.c_int, [f32p, C.POINTER(C.c_uint64), sz, sz, sz, sz, sz, sz, sz, C.c_double]),
@@ -428,6 +430,41 @@ def attention_quant(q, k, v, k_scale, v_scale, m: int, n: int, heads: int, kv_he
                                     _p(vs, C.c_float), _p(out, C.c_float), m, n, heads, kv_heads, head_dim, q_base, window,
                                     KV_KINDS[kind]))
     return out.reshape(m, heads * head_dim)
+
+
+def attention_split(q, k, v, m: int, n: int, heads: int, kv_heads: int, head_dim: int, split: int, q_base: int = 0,
+                    window: int = 0, causal: bool = True) -> tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """Flash-decoding partials (pacc m*heads*split x head_dim, pmax, psum) over fp32 keys and values."""
+    q, k, v = _f32(q).reshape(-1), _f32(k).reshape(-1), _f32(v).reshape(-1)
+    parts = m * heads * split
+    pacc = np.empty(parts * head_dim, dtype=np.float32)
+    pmax, psum = np.empty(parts, dtype=np.float32), np.empty(parts, dtype=np.float32)
+    _check(_lib.orc_attention_split(_p(q, C.c_float), _p(k, C.c_float), _p(v, C.c_float), _p(pacc, C.c_float),
+                                    _p(pmax, C.c_float), _p(psum, C.c_float), m, n, heads, kv_heads, head_dim, q_base, window,
+                                    int(causal), split))
+    return pacc.reshape(parts, head_dim), pmax, psum
+
+
+def attention_combine(pacc, pmax, psum, m: int, heads: int, head_dim: int, split: int) -> np.ndarray:
+    pacc, pmax, psum = _f32(pacc).reshape(-1), _f32(pmax), _f32(psum)
+    out = np.empty(m * heads * head_dim, dtype=np.float32)
+    _check(_lib.orc_attention_combine(_p(pacc, C.c_float), _p(pmax, C.c_float), _p(psum, C.c_float), _p(out, C.c_float), m,
+                                      heads, head_dim, split))
+    return out.reshape(m, heads * head_dim)
+
+
+def dequant_kv(codes, scale, n: int, width: int, kind: str) -> np.ndarray:
+    """code * scale[key row] of a quantized cache as fp32 (n x width): the element decode of
+    AttentionQ8Ref / AttentionQ4Ref / AttentionFp8Ref, for tests that feed the fp32 routines."""
+    codes, scale = _u8(codes), _f32(scale)
+    if kind == "q8":
+        vals = codes.view(np.int8).astype(np.float32)
+    elif kind == "q4":
+        nib = np.stack([codes & 0xF, codes >> 4], axis=-1).reshape(-1).astype(np.int32)
+        vals = np.where(nib >= 8, nib - 16, nib).astype(np.float32)
+    else:
+        vals = np.array([fp8_e4m3_to_float(int(c)) for c in range(256)], np.float32)[codes]
+    return (vals.reshape(n, width) * scale[:, None]).astype(np.float32)
 
 
 def cast_f32_f16(data) -> np.ndarray:

@@ -47,6 +47,9 @@
  *                                             |x - q s| <= s / 2, extremes map to +-127 / +-7)
  *   attention over int8 / 4-bit / E4M3 keys . pinned (numpy / torch decode of the codes fed to torch
  *                                             softmax attention)
+ *   attention_split / attention_combine ..... pinned (each chunk's pacc / psum equals torch attention
+ *                                             over that chunk's keys alone, pmax the float64 maximum;
+ *                                             combine(split) equals the unsplit attention)
  *   cast_f32_f16 (significand cut) .......... pinned (numpy float16 stepped toward zero when the
  *                                             nearest value lies above the input)
  *
@@ -969,6 +972,88 @@ int orc_attention_quant(const float* q, const uint8_t* k, const uint8_t* v, cons
   const int rc = orc_attention(q, kf, vf, out, m, n, heads, kv_heads, head_dim, q_base, window, 0, 1);
   free(kf), free(vf);
   return rc;
+}
+
+/* ---- flash-decoding partials: the key range of (row, head) is cut into `split` chunks of
+ *      ceil(span / split) keys; chunk s leaves pacc = sum_j exp(score_j - pmax) v_j (not
+ *      normalised), pmax = its largest score, psum = sum_j exp(score_j - pmax) at index
+ *      (row * heads + head) * split + s; an empty chunk leaves 0, -1e30, 0
+ *      (src/backends/rocm/rocm_kernels_basic.cpp:275-440; sequential sums here).  k, v are fp32. ---- */
+int orc_attention_split(const float* q, const float* k, const float* v, float* pacc, float* pmax, float* psum, size_t m,
+                        size_t n, size_t heads, size_t kv_heads, size_t head_dim, uint64_t q_base, size_t window, int causal,
+                        size_t split) {
+  if (m == 0 || n == 0 || heads == 0 || kv_heads == 0 || head_dim == 0 || heads % kv_heads != 0 || split == 0) {
+    return ORC_INVALID_ARGUMENT;
+  }
+  float* scores = (float*)malloc(n * sizeof(float));
+  if (!scores) return ORC_OOM;
+  const size_t group = heads / kv_heads;
+  const float scale = 1.0f / sqrtf((float)head_dim);
+  for (size_t i = 0; i < m; ++i) {
+    const size_t pos = (size_t)(q_base + i);
+    const size_t last = causal ? (pos >= n ? n - 1 : pos) : n - 1;
+    size_t start = 0;
+    if (causal) {
+      start = window != 0 && pos + 1 > window ? pos + 1 - window : 0;
+      if (start > last) start = last;
+    }
+    const size_t chunk = (last + 1 - start + split - 1) / split;
+    for (size_t h = 0; h < heads; ++h) {
+      const size_t kv = h / group;
+      const float* q_row = q + (i * heads + h) * head_dim;
+      for (size_t sidx = 0; sidx < split; ++sidx) {
+        const size_t base = (i * heads + h) * split + sidx;
+        const size_t cstart = start + sidx * chunk;
+        if (cstart > last) {
+          for (size_t e = 0; e < head_dim; ++e) pacc[base * head_dim + e] = 0.0f;
+          pmax[base] = -1e30f, psum[base] = 0.0f;
+          continue;
+        }
+        const size_t cend = cstart + chunk - 1 < last ? cstart + chunk - 1 : last;
+        float top = 0.0f;
+        for (size_t j = cstart; j <= cend; ++j) {
+          float dot = 0.0f;
+          for (size_t e = 0; e < head_dim; ++e) dot = fmaf(q_row[e], k[(j * kv_heads + kv) * head_dim + e], dot);
+          scores[j] = dot * scale;
+          if (j == cstart || scores[j] > top) top = scores[j];
+        }
+        float denom = 0.0f;
+        for (size_t j = cstart; j <= cend; ++j) {
+          scores[j] = expf(scores[j] - top);
+          denom += scores[j];
+        }
+        for (size_t e = 0; e < head_dim; ++e) {
+          float acc = 0.0f;
+          for (size_t j = cstart; j <= cend; ++j) acc = fmaf(scores[j], v[(j * kv_heads + kv) * head_dim + e], acc);
+          pacc[base * head_dim + e] = acc;
+        }
+        pmax[base] = top, psum[base] = denom;
+      }
+    }
+  }
+  free(scores);
+  return ORC_OK;
+}
+
+/* ---- merge of the partials (rocm_kernels_basic.cpp:664-690) ---- */
+int orc_attention_combine(const float* pacc, const float* pmax, const float* psum, float* out, size_t m, size_t heads,
+                          size_t head_dim, size_t split) {
+  if (m == 0 || heads == 0 || head_dim == 0 || split == 0) return ORC_INVALID_ARGUMENT;
+  for (size_t g = 0; g < m * heads; ++g) {
+    const size_t base = g * split;
+    float top = -1e30f;
+    for (size_t s = 0; s < split; ++s) top = fmaxf(top, pmax[base + s]);
+    for (size_t e = 0; e < head_dim; ++e) {
+      float num = 0.0f, den = 0.0f;
+      for (size_t s = 0; s < split; ++s) {
+        const float w = expf(pmax[base + s] - top);
+        num = fmaf(w, pacc[(base + s) * head_dim + e], num);
+        den = fmaf(w, psum[base + s], den);
+      }
+      out[g * head_dim + e] = num / den;
+    }
+  }
+  return ORC_OK;
 }
 
 /* ---- fp32 -> binary16 as the "cast_f32_f16" built-in does it: the significand is cut, not rounded

@@ -411,6 +411,68 @@ qmm_status run_attention_q8(const LaunchCtx& c) { return run_attention_quant(c, 
 qmm_status run_attention_q4(const LaunchCtx& c) { return run_attention_quant(c, 1); }
 qmm_status run_attention_fp8(const LaunchCtx& c) { return run_attention_quant(c, 2); }
 
+// The flash-decoding forms.  "attention_split" / "attention_split_gqa": buffers q, k, v, pacc
+// (m*heads*split x head_dim), pmax, psum (m*heads*split each); scalars m, n, heads, kv_heads,
+// head_dim, q_base, window, kv_f16, causal, split (the gqa id: m = 1 and at most 6 heads a kv head;
+// same partials, so this backend runs it as the plain split).  "attention_q8_split" / "_q4_split" /
+// "_fp8_split": buffers q, k, v, ks, vs, pacc, pmax, psum; scalars m, n, heads, kv_heads, head_dim,
+// q_base, window, kind, split (include/tessera/backend.hpp:310-329,441-466,692-705).
+qmm_status run_attention_split_common(const LaunchCtx& c, const char* id, bool quant, uint32_t kind, bool gqa) {
+  if (!counts(c, quant ? 8 : 6, quant ? 9 : 10)) return bad(std::string(id) + ": wrong number of buffers or scalars");
+  const uint64_t m = c.sc[0], n = c.sc[1], heads = c.sc[2], kv_heads = c.sc[3], head_dim = c.sc[4], q_base = c.sc[5],
+                 window = c.sc[6];
+  const uint64_t split = quant ? c.sc[8] : c.sc[9];
+  if (m == 0 || n == 0 || heads == 0 || kv_heads == 0 || head_dim == 0 || heads % kv_heads != 0 || split == 0) {
+    return bad(std::string(id) + ": m, n, heads, kv_heads, head_dim, split must be non-zero and heads a multiple of kv_heads");
+  }
+  if (quant ? c.sc[7] > 2 : (c.sc[7] > 1 || c.sc[8] > 1)) return bad(std::string(id) + ": kind, kv_f16 or causal out of range");
+  if (gqa && (m != 1 || heads / kv_heads > 6)) return bad(std::string(id) + ": m must be 1 and heads / kv_heads at most 6");
+  if (head_dim > 256) return bad(std::string(id) + ": head_dim must be at most 256");
+  if (quant && kind == 1 && (kv_heads * head_dim) % 2 != 0) return bad(std::string(id) + ": a key row must hold an even number of codes");
+  if (m > (1u << 24) || n > (1ull << 32) || heads > (1u << 16) || q_base > (1ull << 40) || split > (1u << 16) ||
+      static_cast<u128>(m) * heads * split > 0x7FFFFFFFull) {
+    return bad(std::string(id) + ": a scalar is out of range");
+  }
+  const u128 q_bytes = static_cast<u128>(m) * heads * head_dim * 4;
+  const u128 codes = static_cast<u128>(n) * kv_heads * head_dim;
+  const u128 kv_bytes = !quant ? codes * (c.sc[7] ? 2 : 4) : kind == 1 ? codes / 2 : codes;
+  const u128 parts = static_cast<u128>(m) * heads * split;
+  const size_t p0 = quant ? 5 : 3;
+  bool ok = c.fits(0, q_bytes) && c.fits(1, kv_bytes) && c.fits(2, kv_bytes) && c.fits(p0, parts * head_dim * 4) &&
+            c.fits(p0 + 1, parts * 4) && c.fits(p0 + 2, parts * 4);
+  if (quant) ok = ok && c.fits(3, static_cast<u128>(n) * 4) && c.fits(4, static_cast<u128>(n) * 4);
+  if (!ok) return bad(std::string(id) + ": a buffer is smaller than the scalars require");
+  const uint32_t kv_kind = quant ? 2u + kind : static_cast<uint32_t>(c.sc[7]);
+  const bool causal = quant ? true : c.sc[8] == 1;
+  return map_hip(qmm::launch_attention_split(c.ptr<const float>(0), c.ptr<const void>(1), c.ptr<const void>(2),
+                                             quant ? c.ptr<const float>(3) : nullptr, quant ? c.ptr<const float>(4) : nullptr,
+                                             c.ptr<float>(p0), c.ptr<float>(p0 + 1), c.ptr<float>(p0 + 2), m, n, heads, kv_heads,
+                                             head_dim, q_base, window, kv_kind, causal, split, c.stream));
+}
+qmm_status run_attention_split(const LaunchCtx& c) { return run_attention_split_common(c, "attention_split", false, 0, false); }
+qmm_status run_attention_split_gqa(const LaunchCtx& c) { return run_attention_split_common(c, "attention_split_gqa", false, 0, true); }
+qmm_status run_attention_q8_split(const LaunchCtx& c) { return run_attention_split_common(c, "attention_q8_split", true, 0, false); }
+qmm_status run_attention_q4_split(const LaunchCtx& c) { return run_attention_split_common(c, "attention_q4_split", true, 1, false); }
+qmm_status run_attention_fp8_split(const LaunchCtx& c) { return run_attention_split_common(c, "attention_fp8_split", true, 2, false); }
+
+// "attention_combine": buffers pacc, pmax, psum, out (m x heads*head_dim); scalars m, heads, head_dim,
+// split (include/tessera/backend.hpp:330-333,467-475).
+qmm_status run_attention_combine(const LaunchCtx& c) {
+  if (!counts(c, 4, 4)) return bad("attention_combine: expects 4 buffers and 4 scalars");
+  const uint64_t m = c.sc[0], heads = c.sc[1], head_dim = c.sc[2], split = c.sc[3];
+  if (m == 0 || heads == 0 || head_dim == 0 || split == 0) return bad("attention_combine: m, heads, head_dim, split must be non-zero");
+  if (head_dim > 256 || m > (1u << 24) || heads > (1u << 16) || split > (1u << 16) || m * heads > 0x7FFFFFFFull) {
+    return bad("attention_combine: a scalar is out of range");
+  }
+  const u128 parts = static_cast<u128>(m) * heads * split;
+  if (!c.fits(0, parts * head_dim * 4) || !c.fits(1, parts * 4) || !c.fits(2, parts * 4) ||
+      !c.fits(3, static_cast<u128>(m) * heads * head_dim * 4)) {
+    return bad("attention_combine: a buffer is smaller than the scalars require");
+  }
+  return map_hip(qmm::launch_attention_combine(c.ptr<const float>(0), c.ptr<const float>(1), c.ptr<const float>(2), c.ptr<float>(3),
+                                               m, heads, head_dim, split, c.stream));
+}
+
 // "quantize_q8" / "quantize_q4": buffers In (rows x cols fp32), Out (int8 codes / 4-bit codes, two a
 // byte), one fp32 scale per row; scalars rows, cols (a multiple of 4 / of 8)
 // (include/tessera/backend.hpp:280-283,292-295,670-678,706-714).
@@ -1078,6 +1140,12 @@ const Entry kTable[] = {
     {"attention_q8", run_attention_q8},
     {"attention_q4", run_attention_q4},
     {"attention_fp8", run_attention_fp8},
+    {"attention_split", run_attention_split},
+    {"attention_split_gqa", run_attention_split_gqa},
+    {"attention_q8_split", run_attention_q8_split},
+    {"attention_q4_split", run_attention_q4_split},
+    {"attention_fp8_split", run_attention_fp8_split},
+    {"attention_combine", run_attention_combine},
     {"quantize_q8", run_quantize_q8},
     {"quantize_q4", run_quantize_q4},
     {"cast_f32_f16", run_cast_f32_f16},

@@ -182,6 +182,12 @@ hipError_t launch_attention(const float* q, const void* k, const void* v, float*
 hipError_t launch_attention_quant(const float* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                                   float* out, uint64_t m, uint64_t n, uint64_t heads, uint64_t kv_heads, uint64_t head_dim,
                                   uint64_t q_base, uint64_t row_base, uint64_t window, uint32_t kind, hipStream_t stream);
+hipError_t launch_attention_split(const float* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                  float* pacc, float* pmax, float* psum, uint64_t m, uint64_t n, uint64_t heads,
+                                  uint64_t kv_heads, uint64_t head_dim, uint64_t q_base, uint64_t window, uint32_t kv_kind,
+                                  bool causal, uint64_t split, hipStream_t stream);
+hipError_t launch_attention_combine(const float* pacc, const float* pmax, const float* psum, float* out, uint64_t m,
+                                    uint64_t heads, uint64_t head_dim, uint64_t split, hipStream_t stream);
 hipError_t launch_quantize_kv(const float* in, uint8_t* out, float* scale, uint64_t rows, uint64_t cols, uint32_t bits,
                               hipStream_t stream);
 hipError_t launch_cast_f32_f16(const float* in, void* out, uint64_t n, hipStream_t stream);

@@ -42,22 +42,45 @@ __global__ __launch_bounds__(256) void rope_kernel(float* __restrict__ data, con
 // AttentionQ4Ref / AttentionFp8Ref (src/core/numerics/attention.cpp:45-121).
 enum class KvKind { F32, F16, Q8, Q4, Fp8 };
 
-template <KvKind KV>
+// SPLIT (the flash-decoding ids, src/backends/rocm/rocm_kernels_basic.cpp:275-440): workgroup
+// (row, head, s) covers chunk s of ceil(span / split) keys of the row's key range and leaves the
+// unnormalized sum, the chunk's largest score and its sum of weights in pacc / pmax / psum at
+// index (row * heads + head) * split + s (an empty chunk: 0, -1e30, 0); attention_combine_kernel
+// merges them.
+struct SplitOut {
+  float *pacc, *pmax, *psum;
+  uint64_t split;
+};
+
+template <KvKind KV, bool SPLIT>
 __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ q, const void* __restrict__ k,
                                                         const void* __restrict__ v, const float* __restrict__ k_scale,
-                                                        const float* __restrict__ v_scale, float* __restrict__ out, uint64_t n,
-                                                        uint64_t heads, uint64_t kv_heads, uint64_t head_dim, uint64_t q_base,
-                                                        uint64_t row_base, uint64_t window, uint64_t causal) {
+                                                        const float* __restrict__ v_scale, float* __restrict__ out,
+                                                        SplitOut part, uint64_t n, uint64_t heads, uint64_t kv_heads,
+                                                        uint64_t head_dim, uint64_t q_base, uint64_t row_base, uint64_t window,
+                                                        uint64_t causal) {
   constexpr uint32_t kKeys = 64;
   __shared__ float sc[kKeys], wt[kKeys], bc[2];
   const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-  const uint64_t i = blockIdx.x / heads, h = blockIdx.x % heads, kv = h / (heads / kv_heads);
+  const uint64_t g = blockIdx.x, rest = SPLIT ? g / part.split : g;
+  const uint64_t i = rest / heads, h = rest % heads, kv = h / (heads / kv_heads);
   const uint64_t pos = q_base + i;
-  const uint64_t last = causal != 0 ? (pos >= n ? n - 1 : pos) : n - 1;
+  uint64_t last = causal != 0 ? (pos >= n ? n - 1 : pos) : n - 1;
   uint64_t start = 0;
   if (causal != 0) {
     start = (window != 0 && pos + 1 > window) ? pos + 1 - window : 0;
     if (start > last) start = last;
+  }
+  if constexpr (SPLIT) {
+    const uint64_t chunk = (last + 1 - start + part.split - 1) / part.split;
+    const uint64_t cstart = start + (g % part.split) * chunk;
+    if (cstart > last) {   // workgroup-uniform
+      if (t < head_dim) part.pacc[g * head_dim + t] = 0.0f;
+      if (t == 0) part.pmax[g] = -1e30f, part.psum[g] = 0.0f;
+      return;
+    }
+    last = cstart + chunk - 1 < last ? cstart + chunk - 1 : last;
+    start = cstart;
   }
   const float scale = 1.0f / sqrtf(static_cast<float>(head_dim));
   const uint64_t qb = ((row_base + i) * heads + h) * head_dim;
@@ -120,7 +143,32 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     }
     __syncthreads();
   }
-  if (t < head_dim) out[qb + t] = acc / run_sum;
+  if constexpr (SPLIT) {
+    if (t < head_dim) part.pacc[g * head_dim + t] = acc;
+    if (t == 0) part.pmax[g] = run_max, part.psum[g] = run_sum;
+  } else {
+    if (t < head_dim) out[qb + t] = acc / run_sum;
+  }
+}
+
+// out[row][head] = sum_s w_s pacc_s / sum_s w_s psum_s with w_s = exp(pmax_s - max_s pmax_s)
+// (src/backends/rocm/rocm_kernels_basic.cpp:664-690).  One workgroup per (row, head).
+__global__ __launch_bounds__(256) void attention_combine_kernel(const float* __restrict__ pacc, const float* __restrict__ pmax,
+                                                                const float* __restrict__ psum, float* __restrict__ out,
+                                                                uint64_t head_dim, uint64_t split) {
+  const uint64_t g = blockIdx.x, base = g * split;
+  const uint32_t e = threadIdx.x;
+  float top = -1e30f;
+  for (uint64_t s = 0; s < split; ++s) top = fmaxf(top, pmax[base + s]);
+  if (e < head_dim) {
+    float num = 0.0f, den = 0.0f;
+    for (uint64_t s = 0; s < split; ++s) {
+      const float w = expf(pmax[base + s] - top);
+      num = fmaf(w, pacc[(base + s) * head_dim + e], num);
+      den = fmaf(w, psum[base + s], den);
+    }
+    out[g * head_dim + e] = num / den;
+  }
 }
 
 __global__ __launch_bounds__(256) void qgate_split_kernel(const float* __restrict__ fused, float* __restrict__ q,
@@ -198,33 +246,57 @@ hipError_t launch_rope(float* data, const uint64_t* pos3, uint64_t rows, uint64_
   return hipGetLastError();
 }
 
+namespace {
+// kind: 0 fp32, 1 fp16 keys and values; 2 int8, 3 4-bit, 4 E4M3 codes with one scale per key row.
+template <bool SPLIT>
+hipError_t launch_attention_as(uint32_t kind, dim3 grid, const float* q, const void* k, const void* v, const float* k_scale,
+                               const float* v_scale, float* out, SplitOut part, uint64_t n, uint64_t heads, uint64_t kv_heads,
+                               uint64_t head_dim, uint64_t q_base, uint64_t row_base, uint64_t window, bool causal,
+                               hipStream_t stream) {
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, q, k, v, k_scale, v_scale, out, part, n, heads, kv_heads, head_dim,
+                       q_base, row_base, window, causal ? 1ull : 0ull);
+  };
+  switch (kind) {
+    case 0: go(attention_kernel<KvKind::F32, SPLIT>); break;
+    case 1: go(attention_kernel<KvKind::F16, SPLIT>); break;
+    case 2: go(attention_kernel<KvKind::Q8, SPLIT>); break;
+    case 3: go(attention_kernel<KvKind::Q4, SPLIT>); break;
+    default: go(attention_kernel<KvKind::Fp8, SPLIT>); break;
+  }
+  return hipGetLastError();
+}
+}  // namespace
+
 hipError_t launch_attention(const float* q, const void* k, const void* v, float* out, uint64_t m, uint64_t n, uint64_t heads,
                             uint64_t kv_heads, uint64_t head_dim, uint64_t q_base, uint64_t row_base, uint64_t window,
                             bool kv_f16, bool causal, hipStream_t stream) {
-  const dim3 grid(static_cast<uint32_t>(m * heads));
-  const float* none = nullptr;
-  if (kv_f16) {
-    hipLaunchKernelGGL(attention_kernel<KvKind::F16>, grid, dim3(256), 0, stream, q, k, v, none, none, out, n, heads, kv_heads,
-                       head_dim, q_base, row_base, window, causal ? 1ull : 0ull);
-  } else {
-    hipLaunchKernelGGL(attention_kernel<KvKind::F32>, grid, dim3(256), 0, stream, q, k, v, none, none, out, n, heads, kv_heads,
-                       head_dim, q_base, row_base, window, causal ? 1ull : 0ull);
-  }
-  return hipGetLastError();
+  return launch_attention_as<false>(kv_f16 ? 1u : 0u, dim3(static_cast<uint32_t>(m * heads)), q, k, v, nullptr, nullptr, out,
+                                    SplitOut{}, n, heads, kv_heads, head_dim, q_base, row_base, window, causal, stream);
 }
 
 // kind: 0 int8, 1 4-bit, 2 E4M3 keys and values with one scale per key row; always causal.
 hipError_t launch_attention_quant(const float* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                                   float* out, uint64_t m, uint64_t n, uint64_t heads, uint64_t kv_heads, uint64_t head_dim,
                                   uint64_t q_base, uint64_t row_base, uint64_t window, uint32_t kind, hipStream_t stream) {
-  const dim3 grid(static_cast<uint32_t>(m * heads));
-  auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, q, k, v, k_scale, v_scale, out, n, heads, kv_heads, head_dim, q_base,
-                       row_base, window, 1ull);
-  };
-  if (kind == 0) go(attention_kernel<KvKind::Q8>);
-  else if (kind == 1) go(attention_kernel<KvKind::Q4>);
-  else go(attention_kernel<KvKind::Fp8>);
+  return launch_attention_as<false>(2u + kind, dim3(static_cast<uint32_t>(m * heads)), q, k, v, k_scale, v_scale, out, SplitOut{},
+                                    n, heads, kv_heads, head_dim, q_base, row_base, window, true, stream);
+}
+
+// The split-N form: kv_kind as launch_attention_as (0 fp32, 1 fp16, 2.. quantized with scales).
+hipError_t launch_attention_split(const float* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                  float* pacc, float* pmax, float* psum, uint64_t m, uint64_t n, uint64_t heads,
+                                  uint64_t kv_heads, uint64_t head_dim, uint64_t q_base, uint64_t window, uint32_t kv_kind,
+                                  bool causal, uint64_t split, hipStream_t stream) {
+  return launch_attention_as<true>(kv_kind, dim3(static_cast<uint32_t>(m * heads * split)), q, k, v, k_scale, v_scale, nullptr,
+                                   SplitOut{pacc, pmax, psum, split}, n, heads, kv_heads, head_dim, q_base, 0, window, causal,
+                                   stream);
+}
+
+hipError_t launch_attention_combine(const float* pacc, const float* pmax, const float* psum, float* out, uint64_t m,
+                                    uint64_t heads, uint64_t head_dim, uint64_t split, hipStream_t stream) {
+  hipLaunchKernelGGL(attention_combine_kernel, dim3(static_cast<uint32_t>(m * heads)), dim3(256), 0, stream, pacc, pmax, psum, out,
+                     head_dim, split);
   return hipGetLastError();
 }
 

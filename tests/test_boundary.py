@@ -25,7 +25,8 @@ REFERENCE_IDS = [
     "gemm_q5k_rows4", "gemm_q5k_rows5", "gemm_q5k_batched", "moe_experts_down_q6k", "gemm_q5k_wmma", "gemm_q6k_wmma",
     "silu_mul", "round_bf16", "add", "fill", "rmsnorm", "embedding_f32", "embedding_bf16", "embedding_q4k",
     "rope", "mrope", "attention", "qgate_split", "attention_q8", "attention_q4", "attention_fp8", "quantize_q8",
-    "quantize_q4", "cast_f32_f16",
+    "quantize_q4", "cast_f32_f16", "attention_split", "attention_split_gqa", "attention_combine", "attention_q8_split",
+    "attention_q4_split", "attention_fp8_split",
 ]
 
 

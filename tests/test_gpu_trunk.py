@@ -172,3 +172,72 @@ def test_cast_f32_f16_bit_exact(backend):
     with pytest.raises(StatusError) as e:   # n must be even
         run(backend, "cast_f32_f16", [din, dout], [x.size - 1])
     assert e.value.code == StatusCode.InvalidArgument
+
+
+@pytest.mark.parametrize("m,n,heads,kv_heads,head_dim,q_base,window,kv_f16,causal,split,gqa", [
+    (1, 300, 8, 2, 64, 299, 0, 0, 1, 4, True), (1, 77, 6, 1, 128, 76, 0, 1, 1, 8, True), (3, 90, 4, 4, 32, 80, 25, 0, 1, 3, False),
+    (2, 11, 2, 1, 16, 0, 0, 0, 0, 16, False), (1, 5, 2, 2, 256, 4, 0, 0, 1, 1, False)])
+def test_attention_split_and_combine(backend, m, n, heads, kv_heads, head_dim, q_base, window, kv_f16, causal, split, gqa):
+    """attention_split / attention_split_gqa then attention_combine: the partials against the oracle's
+    (chunks of ceil(span / split) keys, empty chunks 0 / -1e30 / 0), the merged rows against the unsplit
+    attention."""
+    g = synth.rng(m * 13 + n + split)
+    q = g.standard_normal((m, heads * head_dim)).astype(np.float32)
+    k = g.standard_normal((n, kv_heads * head_dim)).astype(np.float32)
+    v = g.standard_normal((n, kv_heads * head_dim)).astype(np.float32)
+    if kv_f16:
+        k, v = k.astype(np.float16), v.astype(np.float16)
+    kf, vf = np.asarray(k, np.float32), np.asarray(v, np.float32)
+    want_acc, want_max, want_sum = oracle.attention_split(q, kf, vf, m, n, heads, kv_heads, head_dim, split, q_base, window, bool(causal))
+    parts = m * heads * split
+    dq, dk, dv = backend.Upload(q), backend.Upload(k), backend.Upload(v)
+    dacc, dmax, dsum = backend.AllocateBuffer(4 * parts * head_dim), backend.AllocateBuffer(4 * parts), backend.AllocateBuffer(4 * parts)
+    run(backend, "attention_split_gqa" if gqa else "attention_split", [dq, dk, dv, dacc, dmax, dsum],
+        [m, n, heads, kv_heads, head_dim, q_base, window, kv_f16, causal, split], grid=(parts, 1, 1))
+    dout = backend.AllocateBuffer(4 * m * heads * head_dim)
+    run(backend, "attention_combine", [dacc, dmax, dsum, dout], [m, heads, head_dim, split], grid=(m * heads, 1, 1))
+    backend.Synchronize()
+    got_max, got_sum = backend.CopyD2H(dmax, dtype=np.float32), backend.CopyD2H(dsum, dtype=np.float32)
+    got_acc = backend.CopyD2H(dacc, dtype=np.float32).reshape(parts, head_dim)
+    empty = want_sum == 0
+    assert np.array_equal(got_sum == 0, empty) and np.all(got_max[empty] == np.float32(-1e30)) and not got_acc[empty].any()
+    assert np.max(np.abs(got_max[~empty] - want_max[~empty])) <= 2e-6 * max(1.0, np.max(np.abs(want_max[~empty])))
+    assert np.max(np.abs(got_sum - want_sum)) <= 4e-6 * np.max(want_sum)
+    assert np.max(np.abs(got_acc - want_acc)) <= 4e-6 * max(1.0, np.max(np.abs(want_acc)))
+    want = oracle.attention(q, k, v, m, n, heads, kv_heads, head_dim, q_base, window, bool(kv_f16), bool(causal))
+    got = backend.CopyD2H(dout, dtype=np.float32).reshape(m, heads * head_dim)
+    assert np.max(np.abs(got - want)) <= 3e-6 * max(1.0, np.max(np.abs(want)))
+    if gqa:
+        with pytest.raises(StatusError) as e:   # the gqa form serves one row
+            run(backend, "attention_split_gqa", [dq, dk, dv, dacc, dmax, dsum], [2, n, heads, kv_heads, head_dim, q_base, window, kv_f16, causal, split])
+        assert e.value.code == StatusCode.InvalidArgument
+
+
+@pytest.mark.parametrize("kind", ["q8", "q4", "fp8"])
+def test_attention_split_over_a_quantized_cache(backend, kind):
+    m, n, heads, kv_heads, head_dim, q_base, window, split = 1, 150, 8, 2, 64, 149, 0, 5
+    g = synth.rng(len(kind) + 500)
+    width = kv_heads * head_dim
+    q = g.standard_normal((m, heads * head_dim)).astype(np.float32)
+    kf = g.standard_normal((n, width)).astype(np.float32)
+    vf = g.standard_normal((n, width)).astype(np.float32)
+    if kind == "fp8":
+        (k, ks), (v, vs) = oracle.quantize_fp8_pack(kf, n, width), oracle.quantize_fp8_pack(vf, n, width)
+    else:
+        bits = 8 if kind == "q8" else 4
+        (k, ks), (v, vs) = oracle.quantize_kv(kf, n, width, bits), oracle.quantize_kv(vf, n, width, bits)
+    kd, vd = oracle.dequant_kv(k, ks, n, width, kind), oracle.dequant_kv(v, vs, n, width, kind)
+    want_acc, want_max, want_sum = oracle.attention_split(q, kd, vd, m, n, heads, kv_heads, head_dim, split, q_base, window, True)
+    parts = m * heads * split
+    bufs = [backend.Upload(q), backend.Upload(k), backend.Upload(v), backend.Upload(ks), backend.Upload(vs),
+            backend.AllocateBuffer(4 * parts * head_dim), backend.AllocateBuffer(4 * parts), backend.AllocateBuffer(4 * parts)]
+    run(backend, f"attention_{kind}_split", bufs, [m, n, heads, kv_heads, head_dim, q_base, window, oracle.KV_KINDS[kind], split],
+        grid=(parts, 1, 1))
+    dout = backend.AllocateBuffer(4 * m * heads * head_dim)
+    run(backend, "attention_combine", bufs[5:] + [dout], [m, heads, head_dim, split], grid=(m * heads, 1, 1))
+    backend.Synchronize()
+    assert np.max(np.abs(backend.CopyD2H(bufs[5], dtype=np.float32).reshape(parts, head_dim) - want_acc)) <= 4e-6 * max(1.0, np.max(np.abs(want_acc)))
+    assert np.max(np.abs(backend.CopyD2H(bufs[7], dtype=np.float32) - want_sum)) <= 4e-6 * np.max(want_sum)
+    want = oracle.attention_quant(q, k, v, ks, vs, m, n, heads, kv_heads, head_dim, kind, q_base, window)
+    got = backend.CopyD2H(dout, dtype=np.float32).reshape(m, heads * head_dim)
+    assert np.max(np.abs(got - want)) <= 3e-6 * max(1.0, np.max(np.abs(want)))

@@ -193,3 +193,43 @@ def test_cast_f32_f16_cuts_the_significand():
     want = np.where(big, np.where(np.signbit(x), np.float16(-np.inf), np.float16(np.inf)), cut).astype(np.float16)
     assert np.array_equal(got, want.view(np.uint16))
     assert oracle.cast_f32_f16(np.array([np.nan], np.float32))[0] & 0x7FFF == 0x7C00     # NaN becomes infinity
+
+
+@pytest.mark.parametrize("m,n,heads,kv_heads,head_dim,q_base,window,causal,split", [
+    (1, 50, 4, 2, 32, 49, 0, True, 4), (3, 40, 6, 6, 16, 30, 12, True, 5), (2, 9, 2, 1, 8, 0, 0, False, 16), (1, 7, 2, 2, 8, 6, 0, True, 1)])
+def test_attention_split_and_combine(m, n, heads, kv_heads, head_dim, q_base, window, causal, split):
+    """Every chunk on its own is an attention over that chunk's keys (torch, float64): pacc / psum is its
+    output, pmax its largest score; merged, the chunks give the unsplit attention."""
+    g = synth.rng(m * 31 + n + split)
+    q = g.standard_normal((m, heads * head_dim)).astype(np.float32)
+    k = g.standard_normal((n, kv_heads * head_dim)).astype(np.float32)
+    v = g.standard_normal((n, kv_heads * head_dim)).astype(np.float32)
+    pacc, pmax, psum = oracle.attention_split(q, k, v, m, n, heads, kv_heads, head_dim, split, q_base, window, causal)
+    group = heads // kv_heads
+    empties = 0
+    for i in range(m):
+        pos = q_base + i
+        last = min(pos, n - 1) if causal else n - 1
+        start = min(max(0, pos + 1 - window) if (causal and window) else 0, last)
+        chunk = -(-(last + 1 - start) // split)
+        for h in range(heads):
+            for s in range(split):
+                base = (i * heads + h) * split + s
+                lo = start + s * chunk
+                if lo > last:
+                    assert pmax[base] == np.float32(-1e30) and psum[base] == 0 and not pacc[base].any()
+                    empties += 1
+                    continue
+                hi = min(lo + chunk - 1, last)
+                kk = k[lo:hi + 1].reshape(-1, kv_heads, head_dim)[:, h // group].astype(np.float64)
+                vv = v[lo:hi + 1].reshape(-1, kv_heads, head_dim)[:, h // group].astype(np.float64)
+                sc = kk @ q[i].reshape(heads, head_dim)[h].astype(np.float64) / np.sqrt(np.float32(head_dim)).astype(np.float64)
+                w = np.exp(sc - sc.max())
+                assert abs(pmax[base] - sc.max()) <= 2e-6 * max(1.0, abs(sc.max()))
+                assert abs(psum[base] - w.sum()) <= 2e-6 * w.sum() and psum[base] >= 1.0
+                assert np.max(np.abs(pacc[base] - w @ vv)) <= 4e-6 * max(1.0, np.max(np.abs(w @ vv)))
+    if split > n:
+        assert empties > 0
+    merged = oracle.attention_combine(pacc, pmax, psum, m, heads, head_dim, split)
+    want = torch_attention(q, k, v, m, n, heads, kv_heads, head_dim, q_base, window, causal)
+    assert np.max(np.abs(merged - want)) <= 3e-6 * max(1.0, np.max(np.abs(want)))

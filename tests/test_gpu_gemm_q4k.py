@@ -73,7 +73,7 @@ def f16_operands_product(a, w, m, n, k):
     return a16 @ w16.T
 
 
-def rel_err_survey(got, ref):
+def rel_err_floored(got, ref):
     """max |got - ref| / max(|ref|, eps), eps = 1e-3 rms(ref): the per-element figure with the
     small floor, reported (not asserted: an output that cancels to 1e-3 of the rms cannot be
     reproduced to 1e-3 of itself by any operand rounding)."""
@@ -90,7 +90,7 @@ def check(got, a, w, m, n, k, ref, what):
     sim_rms, sim_norm = rms_err(sim, ref), norm_err(sim, ref)
     got_rms, got_norm = rms_err(got, ref), norm_err(got, ref)
     print(f"{what}: vs fp32 oracle max|d|/rms {got_rms:.2e} (fp16-operand product {sim_rms:.2e}), "
-          f"2-norm {got_norm:.2e} ({sim_norm:.2e}), max|d|/max(|ref|,1e-3 rms) {rel_err_survey(got, ref):.2e}")
+          f"2-norm {got_norm:.2e} ({sim_norm:.2e}), max|d|/max(|ref|,1e-3 rms) {rel_err_floored(got, ref):.2e}")
     assert got_rms <= 1.2 * sim_rms + ACC_TOL, (what, got_rms, sim_rms)
     assert got_norm <= 1.2 * sim_norm + ACC_TOL, (what, got_norm, sim_norm)
     assert got_rms <= 4e-3 and got_norm <= 1e-3, (what, got_rms, got_norm)     # absolute ceiling of the path (fp32 rows, short K)

@@ -235,11 +235,13 @@ __device__ __forceinline__ void moe_loader_barrier(bool ring_full) {
 }
 __device__ __forceinline__ void moe_compute_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// One super-block (256 K values) of the 32 x 32 product of a wavefront: `raw` is the lane's
+// One super-block (256 K values) of the (32 RT) x 32 product of a wavefront: `raw` is the lane's
 // weight row in the raw stage, a_chunk(c) the address of 16-byte chunk c (8 K values) of the
-// lane's activation row.
-template <typename AChunk>
-__device__ __forceinline__ void moe_block_mma(const uint8_t* raw, uint32_t kg, AChunk&& a_chunk, float16_t& acc) {
+// lane's activation row in the first 32 rows, `tile_bytes` the distance to the same row of the
+// next 32.  The weights are decoded once for all RT row tiles.
+template <int RT, typename AChunk>
+__device__ __forceinline__ void moe_block_mma(const uint8_t* raw, uint32_t kg, AChunk&& a_chunk, uint32_t tile_bytes,
+                                              float16_t (&acc)[RT]) {
   const BlockHead head = load_block_head(raw);
   uint32_t qw[4], qs8[4];
   unrolled<8>([&](auto step) {
@@ -248,32 +250,160 @@ __device__ __forceinline__ void moe_block_mma(const uint8_t* raw, uint32_t kg, A
     decode_subblock<sb, true>(raw, kg, head, qw, qs8, b);
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      const half8_t af = *reinterpret_cast<const half8_t*>(a_chunk(sb * 4u + tt * 2u + kg));
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[tt], acc, 0, 0, 0);
+      const uint8_t* a = a_chunk(sb * 4u + tt * 2u + kg);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const half8_t af = *reinterpret_cast<const half8_t*>(a + rt * tile_bytes);
+        acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[tt], acc[rt], 0, 0, 0);
+      }
     }
+    // Two row tiles: keep the scheduler from gathering the whole block's activation reads ahead
+    // of the first matrix instruction, which costs more registers than a wavefront has.
+    if constexpr (RT > 1) __builtin_amdgcn_sched_barrier(0);
   });
 }
 
-__device__ __forceinline__ void zero_acc(float16_t& acc) {
+template <int RT>
+__device__ __forceinline__ void zero_acc(float16_t (&acc)[RT]) {
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[rt][e] = 0.0f;
+  }
+}
+
+// LDS of the gate/up kernel: a ring of three stages for passes of 32 rows, of two for 64.
+template <int WAVES>
+constexpr uint32_t moe_gate_up_ring_bytes() {
+  using T = MoeTile<WAVES>;
+  constexpr uint32_t one = 3u * (T::kAStage + T::kWStage), two = 2u * (2u * T::kAStage + T::kWStage);
+  return one > two ? one : two;
+}
+
+struct MoeRowTables {
+  uint32_t tok[64], dst[64];
+  float scale[64];
+};
+
+// One pass of moe_gate_up_kernel: rows m0 .. m0 + live of the sorted pairs (live <= 32 RT) against
+// the workgroup's column tile, gate over all of K and then up, through a ring of S stages.
+template <int WAVES, int S, int RT>
+__device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& rows, const _Float16* __restrict__ a16,
+                                                 const float* __restrict__ a_scale, const uint8_t* __restrict__ gate_e,
+                                                 const uint8_t* __restrict__ up_e, float* __restrict__ phi,
+                                                 const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t top_k,
+                                                 uint32_t col0, uint32_t m0, uint32_t live) {
+  using T = MoeTile<WAVES>;
+  constexpr int kABlocks = T::kABlocks * RT;
+  constexpr uint32_t kAStage = T::kAStage * RT;
+  constexpr int kLoads = kABlocks + T::kWBlocks;   // of one stage
+  static_assert(S == 2 || (S - 2) * kLoads < 64, "the loader's wait counts at most 63 loads");
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t row_blocks = k / 256u, row_bytes = row_blocks * 144u;
+  const uint32_t total = 2u * row_blocks;
+  const uint32_t lds_a = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds));
+  const uint32_t lds_w = lds_a + S * kAStage;
+
+  if (t < 32u * RT) {   // rows past the segment repeat its last row (computed, never stored)
+    const uint32_t p = inv[m0 + (t < live ? t : live - 1u)];
+    rows.tok[t] = p / top_k;
+    rows.dst[t] = p;
+    rows.scale[t] = a_scale[p / top_k];
+  }
+  __syncthreads();
+
+  // Stage of iteration `it` is it % S.  Before iteration `it` the loads of it .. it + S - 2 are
+  // issued and stage it has landed; during it the loader issues it + S - 1 into the stage every
+  // wavefront left at the last barrier, then waits for it + 1.
+  if (wave == WAVES) {
+    // The offsets are the same in every pass; computed again behind an opaque copy of the lane
+    // number, they do not sit in registers (of every wavefront) from one pass to the next.
+    uint32_t ll = lane;
+    asm volatile("" : "+v"(ll));
+    uint32_t w_src[T::kWBlocks], a_src[kABlocks];
+    moe_weight_offsets<WAVES>(ll, row_bytes, w_src);
+    // Activation stage = 32 RT rows x 512 bytes, loaded as blocks of two rows; chunk c of row r
+    // sits at position c ^ (r % 32) of the row, so that the 32 lanes of an MFMA operand read
+    // (same chunk, 32 rows) touch every bank once.
+#pragma unroll
+    for (int i = 0; i < kABlocks; ++i) {
+      const uint32_t row = 2u * i + ll / 32u;
+      a_src[i] = rows.tok[row] * (k * 2u) + (((ll % 32u) ^ (row & 31u)) * 16u);
+    }
+    auto issue = [&](uint32_t it, uint32_t stage) {
+      const uint32_t blk = it < row_blocks ? it : it - row_blocks;
+      const uint8_t* ga = reinterpret_cast<const uint8_t*>(a16) + blk * 512u;
+#pragma unroll
+      for (int i = 0; i < kABlocks; ++i) direct_load16(ga, a_src[i], lds_a + stage * kAStage + i * 1024u);
+      moe_issue_weights<WAVES>((it < row_blocks ? gate_e : up_e) + blk * 144u, w_src, lds_w + stage * T::kWStage);
+    };
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+      if (static_cast<uint32_t>(s) < total) issue(s, s);
+    }
+    moe_loader_barrier<(S - 2) * kLoads>(total >= static_cast<uint32_t>(S - 1));
+    uint32_t stage = 0;
+    for (uint32_t it = 0; it < total; ++it) {
+      const bool more = it + (S - 1) < total;
+      if (more) issue(it + (S - 1), stage == 0 ? S - 1 : stage - 1u);
+      moe_loader_barrier<(S - 2) * kLoads>(more);
+      stage = stage + 1u == S ? 0u : stage + 1u;
+    }
+  } else {
+    const uint32_t l32 = lane & 31u, kg = lane >> 5;
+    const uint8_t* w_lane = lds + S * kAStage + (wave * 32u + l32) * 144u;
+    const uint8_t* a_lane = lds + l32 * 512u;
+    float16_t acc[RT], acc_gate[RT];
+    uint32_t stage = 0;
+    moe_compute_barrier();
+    auto run = [&]() {   // one tensor
+      zero_acc<RT>(acc);
+      for (uint32_t blk = 0; blk < row_blocks; ++blk) {
+        moe_block_mma<RT>(w_lane + stage * T::kWStage, kg,
+                          [&](uint32_t c) { return a_lane + stage * kAStage + ((c ^ l32) * 16u); }, T::kAStage, acc);
+        moe_compute_barrier();
+        stage = stage + 1u == S ? 0u : stage + 1u;
+      }
+    };
+    run();
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc_gate[rt] = acc[rt];
+    run();
+
+    // lane holds column `col` and rows 32 rt + (e/4)*8 + kg*4 + e%4 of the pass
+    const uint32_t col = col0 + wave * 32u + l32;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+      for (int e16 = 0; e16 < 16; ++e16) {
+        const uint32_t row = rt * 32u + (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
+        if (row < live) {
+          const float s = rows.scale[row];
+          const float g = acc_gate[rt][e16] * s, u = acc[rt][e16] * s;
+          phi[static_cast<size_t>(rows.dst[row]) * n + col] = (g / (1.0f + expf(-g))) * u;
+        }
+      }
+    }
+  }
+  __syncthreads();   // the row tables and the ring are rewritten by the next pass
 }
 
 // phi[p][c] = silu((gate_e x_t)(c)) * (up_e x_t)(c) for the pairs p = (t, slot) of expert e and
 // the columns of the workgroup's tile, written in pair order as fp32.  x comes as one fp16 copy
-// per token (a16, scale a_scale): the direct loads of a pass fetch the tokens of its 32 pairs.
-// Gate runs over all of K, then up; the gate sums wait in registers.
-template <int WAVES, int S>
+// per token (a16, scale a_scale): the direct loads of a pass fetch the tokens of its pairs.
+// Gate runs over all of K, then up; the gate sums wait in registers.  An expert with more than
+// 32 pairs left takes 64 a pass (two row tiles against one decode of the weights, ring of two
+// stages), so that its weights are read and decoded once for up to 64 pairs.
+template <int WAVES>
 __global__ __launch_bounds__((WAVES + 1) * 64) void moe_gate_up_kernel(
     const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ gate,
     const uint8_t* __restrict__ up, uint64_t gate_stride, uint64_t up_stride, float* __restrict__ phi,
     const uint32_t* __restrict__ seg, const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t experts,
     uint32_t top_k) {
   using T = MoeTile<WAVES>;
-  constexpr int kLoads = T::kABlocks + T::kWBlocks;   // of one stage
-  __shared__ __attribute__((aligned(16))) uint8_t lds[S * (T::kAStage + T::kWStage)];
-  __shared__ uint32_t row_tok[32], row_dst[32];
-  __shared__ float row_scale[32];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[moe_gate_up_ring_bytes<WAVES>()];
+  __shared__ MoeRowTables rows;
   // Grid as in q4k_gemm_grouped_kernel: an expert's tiles on one XCD, adjacent in dispatch order.
   const uint32_t tiles = n / T::kBN;
   const uint32_t slot = blockIdx.x / 8u;
@@ -281,135 +411,54 @@ __global__ __launch_bounds__((WAVES + 1) * 64) void moe_gate_up_kernel(
   if (e >= experts) return;
   const uint32_t r0 = seg[e], r1 = seg[e + 1];
   if (r1 <= r0) return;
-
-  const uint32_t t = threadIdx.x, lane = t & 63u;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const uint32_t row_blocks = k / 256u, row_bytes = row_blocks * 144u;
-  const uint32_t total = 2u * row_blocks;
-  const uint32_t lds_a = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds));
-  const uint32_t lds_w = lds_a + S * T::kAStage;
-
-  for (uint32_t m0 = r0; m0 < r1; m0 += 32u) {
-    const uint32_t live = r1 - m0 < 32u ? r1 - m0 : 32u;
-    if (t < 32u) {   // rows past the segment repeat its last row (computed, never stored)
-      const uint32_t p = inv[m0 + (t < live ? t : live - 1u)];
-      row_tok[t] = p / top_k;
-      row_dst[t] = p;
-      row_scale[t] = a_scale[p / top_k];
-    }
-    __syncthreads();
-
-    // Stage of iteration `it` is it % S.  Before iteration `it` the loads of it .. it + S - 2 are
-    // issued and stage it has landed; during it the loader issues it + S - 1 into the stage every
-    // wavefront left at the last barrier, then waits for it + 1.
-    if (wave == WAVES) {
-      const size_t tile_off = static_cast<size_t>(tile) * T::kBN * row_bytes;
-      const uint8_t* gate_e = gate + e * gate_stride + tile_off;
-      const uint8_t* up_e = up + e * up_stride + tile_off;
-      uint32_t w_src[T::kWBlocks], a_src[T::kABlocks];
-      moe_weight_offsets<WAVES>(lane, row_bytes, w_src);
-      // Activation stage = 32 rows x 512 bytes, loaded as 16 blocks of two rows; chunk c of row r
-      // sits at position c ^ r of the row, so that the 32 lanes of an MFMA operand read (same
-      // chunk, 32 rows) touch every bank once.
-#pragma unroll
-      for (int i = 0; i < T::kABlocks; ++i) {
-        const uint32_t row = 2u * i + lane / 32u;
-        a_src[i] = row_tok[row] * (k * 2u) + (((lane % 32u) ^ row) * 16u);
-      }
-      auto issue = [&](uint32_t it, uint32_t stage) {
-        const uint32_t blk = it < row_blocks ? it : it - row_blocks;
-        const uint8_t* ga = reinterpret_cast<const uint8_t*>(a16) + blk * 512u;
-#pragma unroll
-        for (int i = 0; i < T::kABlocks; ++i) direct_load16(ga, a_src[i], lds_a + stage * T::kAStage + i * 1024u);
-        moe_issue_weights<WAVES>((it < row_blocks ? gate_e : up_e) + blk * 144u, w_src, lds_w + stage * T::kWStage);
-      };
-#pragma unroll
-      for (int s = 0; s < S - 1; ++s) {
-        if (static_cast<uint32_t>(s) < total) issue(s, s);
-      }
-      moe_loader_barrier<(S - 2) * kLoads>(total >= static_cast<uint32_t>(S - 1));
-      uint32_t stage = 0;
-      for (uint32_t it = 0; it < total; ++it) {
-        const bool more = it + (S - 1) < total;
-        if (more) issue(it + (S - 1), stage == 0 ? S - 1 : stage - 1u);
-        moe_loader_barrier<(S - 2) * kLoads>(more);
-        stage = stage + 1u == S ? 0u : stage + 1u;
-      }
+  const size_t tile_off = static_cast<size_t>(tile) * T::kBN * (k / 256u * 144u);
+  const uint8_t* gate_e = gate + e * gate_stride + tile_off;
+  const uint8_t* up_e = up + e * up_stride + tile_off;
+  for (uint32_t m0 = r0; m0 < r1;) {
+    const uint32_t left = r1 - m0;
+    if (left > 32u) {
+      moe_gate_up_pass<WAVES, 2, 2>(lds, rows, a16, a_scale, gate_e, up_e, phi, inv, n, k, top_k, tile * T::kBN, m0,
+                                    left < 64u ? left : 64u);
+      m0 += 64u;
     } else {
-      const uint32_t l32 = lane & 31u, kg = lane >> 5;
-      const uint8_t* w_lane = lds + S * T::kAStage + (wave * 32u + l32) * 144u;
-      const uint8_t* a_lane = lds + l32 * 512u;
-      float16_t acc, acc_gate;
-      uint32_t stage = 0;
-      moe_compute_barrier();
-      auto run = [&]() {   // one tensor
-        zero_acc(acc);
-        for (uint32_t blk = 0; blk < row_blocks; ++blk) {
-          moe_block_mma(w_lane + stage * T::kWStage, kg,
-                        [&](uint32_t c) { return a_lane + stage * T::kAStage + ((c ^ l32) * 16u); }, acc);
-          moe_compute_barrier();
-          stage = stage + 1u == S ? 0u : stage + 1u;
-        }
-      };
-      run();
-      acc_gate = acc;
-      run();
-
-      // lane holds column `col` and rows (e/4)*8 + kg*4 + e%4 of the pass
-      const uint32_t col = tile * T::kBN + wave * 32u + l32;
-#pragma unroll
-      for (int e16 = 0; e16 < 16; ++e16) {
-        const uint32_t row = (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
-        if (row < live) {
-          const float s = row_scale[row];
-          const float g = acc_gate[e16] * s, u = acc[e16] * s;
-          phi[static_cast<size_t>(row_dst[row]) * n + col] = (g / (1.0f + expf(-g))) * u;
-        }
-      }
+      moe_gate_up_pass<WAVES, 3, 1>(lds, rows, a16, a_scale, gate_e, up_e, phi, inv, n, k, top_k, tile * T::kBN, m0, left);
+      m0 += 32u;
     }
-    __syncthreads();   // the row tables are rewritten by the next pass
   }
 }
 
-// rows[p][c] = (down_e phi[p])(c) for the pairs of expert e, in pair order as fp32.  The 32 rows
-// of a pass stay in LDS for the whole pass as fp16 under a power-of-two row scale (phi can
-// exceed the fp16 range), converted here from the fp32 rows; the workgroup then streams the
-// weights of `tiles_per_chunk` column tiles past them without a break between tiles.
-// Dynamic LDS: S weight stages, the row tables, 32 rows of 2k + 16 bytes.
-template <int WAVES, int S>
-__global__ __launch_bounds__((WAVES + 1) * 64) void moe_down_kernel(
-    const float* __restrict__ phi, const uint8_t* __restrict__ down, uint64_t down_stride, float* __restrict__ rows,
-    const uint32_t* __restrict__ seg, const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t experts,
-    uint32_t chunks, uint32_t tiles_per_chunk) {
+// Dynamic LDS of the down kernel for passes of 32 RT rows: S weight stages, the row tables, the
+// rows as fp16 (2k + 16 bytes each).
+template <int WAVES>
+__host__ __device__ constexpr size_t moe_down_lds_bytes(int stages, int rt, uint32_t inter) {
+  return static_cast<size_t>(stages) * MoeTile<WAVES>::kWStage + 512u + 32u * rt * (2u * static_cast<size_t>(inter) + 16u);
+}
+
+// One pass of moe_down_kernel: rows m0 .. m0 + live of the sorted pairs (live <= 32 RT) against
+// column tiles tile0 .. tile1 of expert e.
+template <int WAVES, int S, int RT>
+__device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __restrict__ phi,
+                                              const uint8_t* __restrict__ down_e, float* __restrict__ rows,
+                                              const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t tile0,
+                                              uint32_t tile1, uint32_t m0, uint32_t live) {
   using T = MoeTile<WAVES>;
-  extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
   float* row_scale = reinterpret_cast<float*>(dyn_lds + S * T::kWStage);
-  uint32_t* row_dst = reinterpret_cast<uint32_t*>(dyn_lds + S * T::kWStage + 128);
-  uint8_t* a_lds = dyn_lds + S * T::kWStage + 256;
+  uint32_t* row_dst = reinterpret_cast<uint32_t*>(dyn_lds + S * T::kWStage + 256);
+  uint8_t* a_lds = dyn_lds + S * T::kWStage + 512;
   const uint32_t a_stride = 2u * k + 16u;
-
-  const uint32_t tiles = n / T::kBN;
-  const uint32_t slot = blockIdx.x / 8u;
-  const uint32_t e = (slot / chunks) * 8u + blockIdx.x % 8u;
-  const uint32_t tile0 = (slot % chunks) * tiles_per_chunk;
-  if (e >= experts || tile0 >= tiles) return;
-  const uint32_t tile1 = tile0 + tiles_per_chunk < tiles ? tile0 + tiles_per_chunk : tiles;
-  const uint32_t r0 = seg[e], r1 = seg[e + 1];
-  if (r1 <= r0) return;
-
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t row_blocks = k / 256u, row_bytes = row_blocks * 144u;
   const uint32_t total = (tile1 - tile0) * row_blocks;
   const uint32_t lds_w = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)dyn_lds));
 
-  for (uint32_t m0 = r0; m0 < r1; m0 += 32u) {
-    const uint32_t live = r1 - m0 < 32u ? r1 - m0 : 32u;
-    // The fp16 copy of the pass's rows: the compute wavefronts' (WAVES * 2) threads a row take its
-    // largest magnitude, then write the groups of 8 in the order the decode yields.
-    if (wave < WAVES) {
-      constexpr uint32_t kPer = WAVES * 2u;
-      const uint32_t row = t / kPer, sub = t % kPer;
+  // The fp16 copy of the pass's rows: the compute wavefronts' (WAVES * 2) threads a row take its
+  // largest magnitude, then write the groups of 8 in the order the decode yields.
+  if (wave < WAVES) {
+    constexpr uint32_t kPer = WAVES * 2u;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const uint32_t row = rt * 32u + t / kPer, sub = t % kPer;
       const uint32_t p = inv[m0 + (row < live ? row : live - 1u)];
       const float4* src = reinterpret_cast<const float4*>(phi + static_cast<size_t>(p) * k);
       float amax = 0.0f;
@@ -425,55 +474,96 @@ __global__ __launch_bounds__((WAVES + 1) * 64) void moe_down_kernel(
       }
       if (sub == 0) row_scale[row] = s, row_dst[row] = p;
     }
-    __syncthreads();
+  }
+  __syncthreads();
 
-    // Iteration `it` is block it % row_blocks of tile tile0 + it / row_blocks; stages and waits
-    // as in moe_gate_up_kernel.
-    if (wave == WAVES) {
-      const uint8_t* down_e = down + e * down_stride;
-      uint32_t w_src[T::kWBlocks];
-      moe_weight_offsets<WAVES>(lane, row_bytes, w_src);
-      uint32_t tile_i = tile0, blk_i = 0;   // S - 1 iterations ahead
-      auto issue_next = [&](uint32_t stage) {
-        moe_issue_weights<WAVES>(down_e + static_cast<size_t>(tile_i) * T::kBN * row_bytes + blk_i * 144u, w_src,
-                                 lds_w + stage * T::kWStage);
-        if (++blk_i == row_blocks) blk_i = 0, ++tile_i;
-      };
+  // Iteration `it` is block it % row_blocks of tile tile0 + it / row_blocks; stages and waits
+  // as in moe_gate_up_pass.
+  if (wave == WAVES) {
+    uint32_t ll = lane;   // as in moe_gate_up_pass
+    asm volatile("" : "+v"(ll));
+    uint32_t w_src[T::kWBlocks];
+    moe_weight_offsets<WAVES>(ll, row_bytes, w_src);
+    uint32_t tile_i = tile0, blk_i = 0;   // S - 1 iterations ahead
+    auto issue_next = [&](uint32_t stage) {
+      moe_issue_weights<WAVES>(down_e + static_cast<size_t>(tile_i) * T::kBN * row_bytes + blk_i * 144u, w_src,
+                               lds_w + stage * T::kWStage);
+      if (++blk_i == row_blocks) blk_i = 0, ++tile_i;
+    };
 #pragma unroll
-      for (int s = 0; s < S - 1; ++s) {
-        if (static_cast<uint32_t>(s) < total) issue_next(s);
-      }
-      moe_loader_barrier<(S - 2) * T::kWBlocks>(total >= static_cast<uint32_t>(S - 1));
-      uint32_t stage = 0;
-      for (uint32_t it = 0; it < total; ++it) {
-        const bool more = it + (S - 1) < total;
-        if (more) issue_next(stage == 0 ? S - 1 : stage - 1u);
-        moe_loader_barrier<(S - 2) * T::kWBlocks>(more);
+    for (int s = 0; s < S - 1; ++s) {
+      if (static_cast<uint32_t>(s) < total) issue_next(s);
+    }
+    moe_loader_barrier<(S - 2) * T::kWBlocks>(total >= static_cast<uint32_t>(S - 1));
+    uint32_t stage = 0;
+    for (uint32_t it = 0; it < total; ++it) {
+      const bool more = it + (S - 1) < total;
+      if (more) issue_next(stage == 0 ? S - 1 : stage - 1u);
+      moe_loader_barrier<(S - 2) * T::kWBlocks>(more);
+      stage = stage + 1u == S ? 0u : stage + 1u;
+    }
+  } else {
+    uint32_t lc = lane;   // as the loader's copy
+    asm volatile("" : "+v"(lc));
+    const uint32_t l32 = lc & 31u, kg = lc >> 5;
+    const uint8_t* w_lane = dyn_lds + (wave * 32u + l32) * 144u;
+    const uint8_t* a_lane = a_lds + l32 * a_stride;
+    float16_t acc[RT];
+    uint32_t stage = 0;
+    moe_compute_barrier();
+    for (uint32_t tile = tile0; tile < tile1; ++tile) {
+      zero_acc<RT>(acc);
+      for (uint32_t blk = 0; blk < row_blocks; ++blk) {
+        moe_block_mma<RT>(w_lane + stage * T::kWStage, kg, [&](uint32_t c) { return a_lane + (blk * 32u + c) * 16u; },
+                          32u * a_stride, acc);
+        moe_compute_barrier();
         stage = stage + 1u == S ? 0u : stage + 1u;
       }
-    } else {
-      const uint32_t l32 = lane & 31u, kg = lane >> 5;
-      const uint8_t* w_lane = dyn_lds + (wave * 32u + l32) * 144u;
-      const uint8_t* a_lane = a_lds + l32 * a_stride;
-      float16_t acc;
-      uint32_t stage = 0;
-      moe_compute_barrier();
-      for (uint32_t tile = tile0; tile < tile1; ++tile) {
-        zero_acc(acc);
-        for (uint32_t blk = 0; blk < row_blocks; ++blk) {
-          moe_block_mma(w_lane + stage * T::kWStage, kg, [&](uint32_t c) { return a_lane + (blk * 32u + c) * 16u; }, acc);
-          moe_compute_barrier();
-          stage = stage + 1u == S ? 0u : stage + 1u;
-        }
-        const uint32_t col = tile * T::kBN + wave * 32u + l32;
+      const uint32_t col = tile * T::kBN + wave * 32u + l32;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
         for (int e16 = 0; e16 < 16; ++e16) {
-          const uint32_t row = (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
-          if (row < live) rows[static_cast<size_t>(row_dst[row]) * n + col] = acc[e16] * row_scale[row];
+          const uint32_t row = rt * 32u + (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
+          if (row < live) rows[static_cast<size_t>(row_dst[row]) * n + col] = acc[rt][e16] * row_scale[row];
         }
       }
     }
-    __syncthreads();   // the rows and their tables are rewritten by the next pass
+  }
+  __syncthreads();   // the rows, their tables and the ring are rewritten by the next pass
+}
+
+// rows[p][c] = (down_e phi[p])(c) for the pairs of expert e, in pair order as fp32.  The rows
+// of a pass stay in LDS for the whole pass as fp16 under a power-of-two row scale (phi can
+// exceed the fp16 range), converted here from the fp32 rows; the workgroup then streams the
+// weights of `tiles_per_chunk` column tiles past them without a break between tiles.  A pass is
+// 32 rows behind a ring of S stages, or (`wide`: the launch reserved the LDS for it) 64 rows
+// behind a ring of two when the expert has more than 32 pairs left.
+template <int WAVES, int S>
+__global__ __launch_bounds__((WAVES + 1) * 64) void moe_down_kernel(
+    const float* __restrict__ phi, const uint8_t* __restrict__ down, uint64_t down_stride, float* __restrict__ rows,
+    const uint32_t* __restrict__ seg, const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t experts,
+    uint32_t chunks, uint32_t tiles_per_chunk, bool wide) {
+  using T = MoeTile<WAVES>;
+  extern __shared__ __attribute__((aligned(16))) uint8_t dyn_lds[];
+  const uint32_t tiles = n / T::kBN;
+  const uint32_t slot = blockIdx.x / 8u;
+  const uint32_t e = (slot / chunks) * 8u + blockIdx.x % 8u;
+  const uint32_t tile0 = (slot % chunks) * tiles_per_chunk;
+  if (e >= experts || tile0 >= tiles) return;
+  const uint32_t tile1 = tile0 + tiles_per_chunk < tiles ? tile0 + tiles_per_chunk : tiles;
+  const uint32_t r0 = seg[e], r1 = seg[e + 1];
+  if (r1 <= r0) return;
+  const uint8_t* down_e = down + e * down_stride;
+  for (uint32_t m0 = r0; m0 < r1;) {
+    const uint32_t left = r1 - m0;
+    if (wide && left > 32u) {
+      moe_down_pass<WAVES, 2, 2>(dyn_lds, phi, down_e, rows, inv, n, k, tile0, tile1, m0, left < 64u ? left : 64u);
+      m0 += 64u;
+    } else {
+      moe_down_pass<WAVES, S, 1>(dyn_lds, phi, down_e, rows, inv, n, k, tile0, tile1, m0, left < 32u ? left : 32u);
+      m0 += 32u;
+    }
   }
 }
 
@@ -500,16 +590,12 @@ __global__ __launch_bounds__(256) void moe_combine_pairs_kernel(const float4* __
 size_t align256(size_t v) { return (v + 255) & ~size_t{255}; }
 
 constexpr size_t kMoeLdsLimit = 160 * 1024 - 64;
-template <int WAVES, int S>
-size_t moe_down_lds_bytes(uint32_t inter) {
-  return S * MoeTile<WAVES>::kWStage + 256 + 32 * (2 * static_cast<size_t>(inter) + 16);
-}
 
 // The two-kernel path needs an expert's 32 rows of phi in LDS next to the weight ring (eight
 // compute wavefronts and three stages up to an inner width of 768, four and two up to 1792),
 // whole column tiles, and 32-bit byte offsets into the fp16 token copy.
 bool moe_resident_path(uint32_t hidden, uint32_t inter, uint32_t tokens) {
-  return moe_down_lds_bytes<4, 2>(inter) <= kMoeLdsLimit && static_cast<uint64_t>(tokens) * hidden * 2 < (1ull << 32);
+  return moe_down_lds_bytes<4>(2, 1, inter) <= kMoeLdsLimit && static_cast<uint64_t>(tokens) * hidden * 2 < (1ull << 32);
 }
 
 void launch_moe_gate_up_resident(const _Float16* a16, const float* a_scale, const uint8_t* gate, const uint8_t* up,
@@ -517,7 +603,7 @@ void launch_moe_gate_up_resident(const _Float16* a16, const float* a_scale, cons
                                  const uint32_t* inv, uint32_t hidden, uint32_t inter, uint32_t experts, uint32_t top_k,
                                  hipStream_t stream) {
   const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
-  hipLaunchKernelGGL((moe_gate_up_kernel<8, 3>), dim3(expert_groups * (inter / 256u)), dim3(MoeTile<8>::kThreads), 0, stream, a16, a_scale,
+  hipLaunchKernelGGL((moe_gate_up_kernel<8>), dim3(expert_groups * (inter / 256u)), dim3(MoeTile<8>::kThreads), 0, stream, a16, a_scale,
                      gate, up, gate_stride, up_stride, phi, seg, inv, inter, hidden, experts, top_k);
 }
 
@@ -531,14 +617,17 @@ void launch_moe_down_tiles(const float* phi, const uint8_t* down, uint64_t down_
   const uint32_t chunks = want < 1u ? 1u : want > tiles ? tiles : want;
   const uint32_t tiles_per_chunk = (tiles + chunks - 1u) / chunks;
   const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
-  const size_t lds_bytes = moe_down_lds_bytes<WAVES, S>(inter);
+  // 64-row passes where their rows fit next to a ring of two stages
+  const size_t narrow = moe_down_lds_bytes<WAVES>(S, 1, inter), wide_bytes = moe_down_lds_bytes<WAVES>(2, 2, inter);
+  const bool wide = wide_bytes <= kMoeLdsLimit;
+  const size_t lds_bytes = wide && wide_bytes > narrow ? wide_bytes : narrow;
   hipLaunchKernelGGL((moe_down_kernel<WAVES, S>), dim3(expert_groups * chunks), dim3(MoeTile<WAVES>::kThreads), lds_bytes, stream, phi,
-                     down, down_stride, rows, seg, inv, hidden, inter, experts, chunks, tiles_per_chunk);
+                     down, down_stride, rows, seg, inv, hidden, inter, experts, chunks, tiles_per_chunk, wide);
 }
 
 void launch_moe_down_resident(const float* phi, const uint8_t* down, uint64_t down_stride, float* rows, const uint32_t* seg,
                               const uint32_t* inv, uint32_t hidden, uint32_t inter, uint32_t experts, hipStream_t stream) {
-  if (moe_down_lds_bytes<8, 3>(inter) <= kMoeLdsLimit) {
+  if (moe_down_lds_bytes<8>(3, 1, inter) <= kMoeLdsLimit) {
     launch_moe_down_tiles<8, 3>(phi, down, down_stride, rows, seg, inv, hidden, inter, experts, 1u, stream);
   } else {
     launch_moe_down_tiles<4, 2>(phi, down, down_stride, rows, seg, inv, hidden, inter, experts, 1u, stream);

@@ -186,13 +186,15 @@ def forward_grouped(backend, x, ids, wts, gate, up, down, hidden, inter, experts
 
 @pytest.mark.parametrize("rows,experts,hidden,inter,top_k", [(1, 8, 256, 256, 2), (40, 16, 512, 256, 4),
                                                              (130, 6, 256, 512, 3), (64, 3, 768, 256, 1), (90, 12, 256, 256, 2),
-                                                             (48, 4, 256, 1024, 2), (40, 3, 256, 2048, 2)])
+                                                             (48, 4, 256, 1024, 2), (40, 3, 256, 2048, 2),
+                                                             (200, 4, 512, 512, 2)])
 def test_grouped_ffn_matches_oracle(backend, rows, experts, hidden, inter, top_k):
     """moe_experts_ffn_q4k_rows: tokens grouped by expert, three grouped fp16-MFMA GEMMs.  The
     operands are rounded to fp16 twice along the way (weights as in the Q4_K prefill GEMM, and
     phi before the down projection), so the bound is the prefill GEMM's, loosened for the chain:
     largest error at most 8e-3 of the rms output, 2e-3 in the 2-norm.  Experts that receive more
-    than 32 tokens (the kernel's row tile) and experts that receive none both occur here.  An inner
+    than 32 tokens (they take 64 rows a pass, then what is left: about 65 and about 100 tokens an
+    expert both occur) and experts that receive none both occur here.  An inner
     width of 1024 takes the narrower of the two row-resident kernels, 2048 the streamed grouped
     tiles (the rows of phi no longer fit LDS)."""
     g = synth.rng(rows * 3 + experts + hidden + inter)

@@ -93,6 +93,26 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
   moe_sort_pairs(ids, pairs, experts, seg, pos, inv);
 }
 
+// Half the sum of the 32 fp16 values of a Q4_K sub-block as an fp16 pair (hi, lo), for the
+// min term of the routed-expert kernels (see moe_block_mma).  `v` is group g (8 values) of a row,
+// held by four neighbouring lanes per sub-block; the row's sums live at `sums`, 16 halves a
+// super-block: hi of sub-blocks 0..7, then lo.  Halved so that 32 values below 2048 stay below
+// the largest fp16 number.
+__device__ __forceinline__ void store_subblock_sum(const half8_t& v, uint32_t g, _Float16* sums) {
+  float part = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) part += static_cast<float>(v[e]);
+  part += __shfl_xor(part, 1);
+  part += __shfl_xor(part, 2);
+  if ((g & 3u) == 0) {
+    const float half_sum = 0.5f * part;
+    const _Float16 hi = static_cast<_Float16>(half_sum);
+    const uint32_t at = (g >> 5) * 16u + ((g >> 2) & 7u);
+    sums[at] = hi;
+    sums[at + 8u] = static_cast<_Float16>(half_sum - static_cast<float>(hi));
+  }
+}
+
 // The sort and the fp16 copy of the token rows do not depend on each other: workgroup 0 sorts,
 // workgroup 1 + r converts row r of x (as rows_to_f16_kernel does: divided by the row's
 // power-of-two scale, groups of 8 in the order the weight decode yields).
@@ -100,7 +120,8 @@ __global__ __launch_bounds__(1024) void moe_prepare_kernel(const uint32_t* __res
                                                            uint32_t experts, uint32_t* __restrict__ seg,
                                                            uint32_t* __restrict__ pos, uint32_t* __restrict__ inv,
                                                            const float* __restrict__ x, _Float16* __restrict__ a16,
-                                                           float* __restrict__ a_scale, uint32_t cols) {
+                                                           _Float16* __restrict__ a_sums, float* __restrict__ a_scale,
+                                                           uint32_t cols) {
   if (blockIdx.x == 0) {
     moe_sort_pairs(ids, pairs, experts, seg, pos, inv);
     return;
@@ -121,7 +142,12 @@ __global__ __launch_bounds__(1024) void moe_prepare_kernel(const uint32_t* __res
   for (int w = 1; w < 16; ++w) amax = fmaxf(amax, red[w]);
   const float s = row_scale_for(amax), inv_s = 1.0f / s;
   half8_t* out = reinterpret_cast<half8_t*>(a16 + static_cast<size_t>(row) * cols);
-  for (uint32_t g = t; g < cols / 8u; g += 1024u) out[g] = to_f16_group(in[2 * g], in[2 * g + 1], inv_s);
+  _Float16* sums = a_sums + static_cast<size_t>(row) * (cols / 16u);
+  for (uint32_t g = t; g < cols / 8u; g += 1024u) {
+    const half8_t v = to_f16_group(in[2 * g], in[2 * g + 1], inv_s);
+    out[g] = v;
+    store_subblock_sum(v, g, sums);
+  }
   if (t == 0) a_scale[row] = s;
 }
 
@@ -197,8 +223,9 @@ struct MoeTile {
   static constexpr uint32_t kBN = WAVES * 32u;                   // columns of a workgroup's tile
   static constexpr int kWBlocks = kBN * 144u / 1024u;            // 1 KB loads of a weight stage (exact)
   static constexpr uint32_t kWStage = kWBlocks * 1024u;
-  static constexpr int kABlocks = 16;                            // 1 KB loads of an activation stage
-  static constexpr uint32_t kAStage = 32u * 512u;                // one super-block of K for 32 rows, fp16
+  static constexpr int kABlocks = 17;                            // 1 KB loads of an activation stage
+  static constexpr uint32_t kARows = 32u * 512u;                 // one super-block of K for 32 rows, fp16 ...
+  static constexpr uint32_t kAStage = kARows + 1024u;            // ... and the rows' 16 sub-block sums
   static constexpr uint32_t kThreads = (WAVES + 1) * 64u;        // compute wavefronts and the loader
   static_assert(kBN * 144u % 1024u == 0, "tile shape");
 };
@@ -235,32 +262,107 @@ __device__ __forceinline__ void moe_loader_barrier(bool ring_full) {
 }
 __device__ __forceinline__ void moe_compute_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// One super-block (256 K values) of the (32 RT) x 32 product of a wavefront: `raw` is the lane's
-// weight row in the raw stage, a_chunk(c) the address of 16-byte chunk c (8 K values) of the
-// lane's activation row in the first 32 rows, `tile_bytes` the distance to the same row of the
-// next 32.  The weights are decoded once for all RT row tiles.
+// One super-block (256 K values) of the (32 RT) x 32 product of a wavefront, added to `acc`.
+//
+// A Q4_K weight is d sc q - dmin mn (src/core/numerics/quant.cpp:656-675).  The matrix cores take
+// q sc undecoded: an integer n < 2048 written into a 16-bit half IS the fp16 number n 2^-24
+// (subnormal below 1024, the first normal binade above), so one 24-bit multiply of a masked
+// nibble pair by the 6-bit scale makes two exact operands (q sc <= 945), and d is applied once to
+// the block's sums.  The min term leaves the K loop: sum_k a_k dmin mn = sum_sb (dmin mn_sb) S_sb
+// with S_sb the sum of the row's activations over sub-block sb, a 16-deep product of the rows'
+// sums (fp16 hi/lo pairs, half the sum each, made where the fp16 rows are made) with 2 dmin mn
+// (fp16 hi/lo pairs, exact: 11 x 6 bits); the lo x lo products (2^-22 of the term) are dropped.
+// No weight is rounded, and the vector work per weight pair is a mask and a multiply (the
+// v_fma_mixlo/hi_f16 pair that forms a rounded fp16 weight issues at half rate).
+//
+// `raw` is the lane's weight row in the raw stage, a_chunk(c) the address of 16-byte chunk c
+// (8 K values) of the lane's activation row in the first 32 rows, `tile_bytes` the distance to
+// the same row of the next 32; `sums` the lane's 16 bytes of its row's sums (hi for kg 0, lo for
+// kg 1), `sums_tile_bytes` the distance to the next 32 rows' sums.  Every LDS read is requested
+// well before its use: the lane's 80 bytes of the weight row, the sums and the first activation
+// fragments up front, the fragments and quant words of a step one step before it (the scheduling
+// barrier keeps them there).
 template <int RT, typename AChunk>
 __device__ __forceinline__ void moe_block_mma(const uint8_t* raw, uint32_t kg, AChunk&& a_chunk, uint32_t tile_bytes,
-                                              float16_t (&acc)[RT]) {
-  const BlockHead head = load_block_head(raw);
-  uint32_t qw[4], qs8[4];
-  unrolled<8>([&](auto step) {
-    constexpr int sb = decltype(step)::value;
-    half8_t b[2];
-    decode_subblock<sb, true>(raw, kg, head, qw, qs8, b);
+                                              const uint8_t* sums, uint32_t sums_tile_bytes, float16_t (&acc)[RT]) {
+  const uint4 head_words = *reinterpret_cast<const uint4*>(raw);
+  half8_t row_sums[RT];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const uint8_t* a = a_chunk(sb * 4u + tt * 2u + kg);
+  for (int rt = 0; rt < RT; ++rt) row_sums[rt] = *reinterpret_cast<const half8_t*>(sums + rt * sums_tile_bytes);
+  // Quant words of sub-block pair g (bytes 32 g + 8 kg + [0,8) and the same + 16 of the row's
+  // quants) and the activation fragments of step j = 2 sb + tt, both fetched one step ahead.
+  uint32_t q_next[4];
+  auto load_q = [&](int g) {
+    const uint8_t* qp = raw + 16 + g * 32 + kg * 8u;
+    const uint2 q0 = *reinterpret_cast<const uint2*>(qp), q1 = *reinterpret_cast<const uint2*>(qp + 16);
+    q_next[0] = q0.x, q_next[1] = q0.y, q_next[2] = q1.x, q_next[3] = q1.y;
+  };
+  half8_t a_next[RT];
+  auto load_a = [&](int j) {
+    const uint8_t* a = a_chunk((j >> 1) * 4u + (j & 1) * 2u + kg);
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const half8_t af = *reinterpret_cast<const half8_t*>(a + rt * tile_bytes);
-        acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[tt], acc[rt], 0, 0, 0);
-      }
+    for (int rt = 0; rt < RT; ++rt) a_next[rt] = *reinterpret_cast<const half8_t*>(a + rt * tile_bytes);
+  };
+  load_q(0);
+  load_a(0);
+
+  const float d24 = half_bits_to_float(head_words.x & 0xFFFFu) * 0x1p24f;
+  const float ndmin2 = -2.0f * half_bits_to_float(head_words.x >> 16);
+  const ScaleBytes sbytes = unpack_scales(head_words.y, head_words.z, head_words.w);
+
+  // The min term: -2 dmin mn_sb as hi + lo (exact), hi against the sums' hi and lo, lo against
+  // the sums' hi only (lanes of K half 1 hold the sums' lo and get zeros).
+  {
+    half8_t min_hi, min_lo;
+#pragma unroll
+    for (int sb = 0; sb < 8; ++sb) {
+      const float p = static_cast<float>((sbytes.mn[sb >> 2] >> (8 * (sb & 3))) & 0xFFu) * ndmin2;
+      const _Float16 hi = static_cast<_Float16>(p);
+      min_hi[sb] = hi;
+      min_lo[sb] = kg == 0 ? static_cast<_Float16>(p - static_cast<float>(hi)) : static_cast<_Float16>(0.0f);
     }
-    // Two row tiles: keep the scheduler from gathering the whole block's activation reads ahead
-    // of the first matrix instruction, which costs more registers than a wavefront has.
-    if constexpr (RT > 1) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(row_sums[rt], min_hi, acc[rt], 0, 0, 0);
+      acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(row_sums[rt], min_lo, acc[rt], 0, 0, 0);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // The main term: sum_k a_k (q sc)_k 2^-24 over the block, then times d 2^24.
+  float16_t blk[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) blk[rt][e] = 0.0f;
+  }
+  uint32_t qw[4];
+  unrolled<16>([&](auto step) {
+    constexpr int j = decltype(step)::value, sb = j >> 1, tt = j & 1;
+    half8_t a_cur[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) a_cur[rt] = a_next[rt];
+    if (j % 4 == 0) {   // an even sub-block brings the words; its odd successor takes their high nibbles
+#pragma unroll
+      for (int x = 0; x < 4; ++x) qw[x] = q_next[x];
+      if (j < 12) load_q(j / 4 + 1);
+    }
+    if (j < 15) load_a(j + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t sc = (sbytes.sc[sb >> 2] >> (8 * (sb & 3))) & 0xFFu;
+    // bytes 0 and 2 of a word are weights (k0, k2), bytes 1 and 3 (the word shifted down a byte)
+    // (k1, k3): the order the fp16 rows are stored in
+    auto pair = [&](uint32_t x, uint32_t down) { return __umul24((x >> (down + ((sb & 1) ? 4u : 0u))) & 0x000F000Fu, sc); };
+    const uint4 words = make_uint4(pair(qw[2 * tt], 0u), pair(qw[2 * tt], 8u), pair(qw[2 * tt + 1], 0u), pair(qw[2 * tt + 1], 8u));
+    const half8_t b = bit_cast<half8_t>(words);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) blk[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[rt], b, blk[rt], 0, 0, 0);
   });
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[rt][e] = fmaf(d24, blk[rt][e], acc[rt][e]);
+  }
 }
 
 template <int RT>
@@ -281,20 +383,22 @@ constexpr uint32_t moe_gate_up_ring_bytes() {
 }
 
 struct MoeRowTables {
-  uint32_t tok[64], dst[64];
-  float scale[64];
+  alignas(16) uint32_t tok[64];
+  alignas(16) uint32_t dst[64];
+  alignas(16) float scale[64];
 };
 
 // One pass of moe_gate_up_kernel: rows m0 .. m0 + live of the sorted pairs (live <= 32 RT) against
 // the workgroup's column tile, gate over all of K and then up, through a ring of S stages.
 template <int WAVES, int S, int RT>
 __device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& rows, const _Float16* __restrict__ a16,
-                                                 const float* __restrict__ a_scale, const uint8_t* __restrict__ gate_e,
+                                                 const _Float16* __restrict__ a_sums, const float* __restrict__ a_scale,
+                                                 const uint8_t* __restrict__ gate_e,
                                                  const uint8_t* __restrict__ up_e, float* __restrict__ phi,
                                                  const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t top_k,
                                                  uint32_t col0, uint32_t m0, uint32_t live) {
   using T = MoeTile<WAVES>;
-  constexpr int kABlocks = T::kABlocks * RT;
+  constexpr int kABlocks = T::kABlocks * RT, kRowBlocks = 16 * RT;   // 1 KB loads of a stage: all, rows only
   constexpr uint32_t kAStage = T::kAStage * RT;
   constexpr int kLoads = kABlocks + T::kWBlocks;   // of one stage
   static_assert(S == 2 || (S - 2) * kLoads < 64, "the loader's wait counts at most 63 loads");
@@ -325,17 +429,23 @@ __device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& row
     moe_weight_offsets<WAVES>(ll, row_bytes, w_src);
     // Activation stage = 32 RT rows x 512 bytes, loaded as blocks of two rows; chunk c of row r
     // sits at position c ^ (r % 32) of the row, so that the 32 lanes of an MFMA operand read
-    // (same chunk, 32 rows) touch every bank once.
+    // (same chunk, 32 rows) touch every bank once.  Then the rows' sub-block sums, 32 bytes a
+    // row: one load per 32 rows.
 #pragma unroll
-    for (int i = 0; i < kABlocks; ++i) {
+    for (int i = 0; i < kRowBlocks; ++i) {
       const uint32_t row = 2u * i + ll / 32u;
       a_src[i] = rows.tok[row] * (k * 2u) + (((ll % 32u) ^ (row & 31u)) * 16u);
     }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) a_src[kRowBlocks + rt] = rows.tok[rt * 32u + ll / 2u] * (row_blocks * 32u) + (ll % 2u) * 16u;
     auto issue = [&](uint32_t it, uint32_t stage) {
       const uint32_t blk = it < row_blocks ? it : it - row_blocks;
       const uint8_t* ga = reinterpret_cast<const uint8_t*>(a16) + blk * 512u;
+      const uint8_t* gs = reinterpret_cast<const uint8_t*>(a_sums) + blk * 32u;
 #pragma unroll
-      for (int i = 0; i < kABlocks; ++i) direct_load16(ga, a_src[i], lds_a + stage * kAStage + i * 1024u);
+      for (int i = 0; i < kRowBlocks; ++i) direct_load16(ga, a_src[i], lds_a + stage * kAStage + i * 1024u);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) direct_load16(gs, a_src[kRowBlocks + rt], lds_a + stage * kAStage + (kRowBlocks + rt) * 1024u);
       moe_issue_weights<WAVES>((it < row_blocks ? gate_e : up_e) + blk * 144u, w_src, lds_w + stage * T::kWStage);
     };
 #pragma unroll
@@ -354,6 +464,7 @@ __device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& row
     const uint32_t l32 = lane & 31u, kg = lane >> 5;
     const uint8_t* w_lane = lds + S * kAStage + (wave * 32u + l32) * 144u;
     const uint8_t* a_lane = lds + l32 * 512u;
+    const uint8_t* s_lane = lds + kRowBlocks * 1024u + l32 * 32u + kg * 16u;
     float16_t acc[RT], acc_gate[RT];
     uint32_t stage = 0;
     moe_compute_barrier();
@@ -361,7 +472,8 @@ __device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& row
       zero_acc<RT>(acc);
       for (uint32_t blk = 0; blk < row_blocks; ++blk) {
         moe_block_mma<RT>(w_lane + stage * T::kWStage, kg,
-                          [&](uint32_t c) { return a_lane + stage * kAStage + ((c ^ l32) * 16u); }, T::kAStage, acc);
+                          [&](uint32_t c) { return a_lane + stage * kAStage + ((c ^ l32) * 16u); }, T::kARows,
+                          s_lane + stage * kAStage, 1024u, acc);
         moe_compute_barrier();
         stage = stage + 1u == S ? 0u : stage + 1u;
       }
@@ -371,17 +483,23 @@ __device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& row
     for (int rt = 0; rt < RT; ++rt) acc_gate[rt] = acc[rt];
     run();
 
-    // lane holds column `col` and rows 32 rt + (e/4)*8 + kg*4 + e%4 of the pass
+    // lane holds column `col` and rows 32 rt + 8 g + 4 kg + [0,4), g = 0..3: four table entries a read
     const uint32_t col = col0 + wave * 32u + l32;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-      for (int e16 = 0; e16 < 16; ++e16) {
-        const uint32_t row = rt * 32u + (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
-        if (row < live) {
-          const float s = rows.scale[row];
-          const float g = acc_gate[rt][e16] * s, u = acc[rt][e16] * s;
-          phi[static_cast<size_t>(rows.dst[row]) * n + col] = (g / (1.0f + expf(-g))) * u;
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const uint32_t row0 = rt * 32u + g4 * 8u + kg * 4u;
+        const uint4 dst4 = *reinterpret_cast<const uint4*>(rows.dst + row0);
+        const float4 sc4 = *reinterpret_cast<const float4*>(rows.scale + row0);
+        const uint32_t dst[4] = {dst4.x, dst4.y, dst4.z, dst4.w};
+        const float sc[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (row0 + i < live) {
+            const float g = acc_gate[rt][g4 * 4 + i] * sc[i], u = acc[rt][g4 * 4 + i] * sc[i];
+            phi[static_cast<size_t>(dst[i]) * n + col] = (g / (1.0f + expf(-g))) * u;
+          }
         }
       }
     }
@@ -397,8 +515,9 @@ __device__ __forceinline__ void moe_gate_up_pass(uint8_t* lds, MoeRowTables& row
 // stages), so that its weights are read and decoded once for up to 64 pairs.
 template <int WAVES>
 __global__ __launch_bounds__((WAVES + 1) * 64) void moe_gate_up_kernel(
-    const _Float16* __restrict__ a16, const float* __restrict__ a_scale, const uint8_t* __restrict__ gate,
-    const uint8_t* __restrict__ up, uint64_t gate_stride, uint64_t up_stride, float* __restrict__ phi,
+    const _Float16* __restrict__ a16, const _Float16* __restrict__ a_sums, const float* __restrict__ a_scale,
+    const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, uint64_t gate_stride, uint64_t up_stride,
+    float* __restrict__ phi,
     const uint32_t* __restrict__ seg, const uint32_t* __restrict__ inv, uint32_t n, uint32_t k, uint32_t experts,
     uint32_t top_k) {
   using T = MoeTile<WAVES>;
@@ -417,21 +536,22 @@ __global__ __launch_bounds__((WAVES + 1) * 64) void moe_gate_up_kernel(
   for (uint32_t m0 = r0; m0 < r1;) {
     const uint32_t left = r1 - m0;
     if (left > 32u) {
-      moe_gate_up_pass<WAVES, 2, 2>(lds, rows, a16, a_scale, gate_e, up_e, phi, inv, n, k, top_k, tile * T::kBN, m0,
+      moe_gate_up_pass<WAVES, 2, 2>(lds, rows, a16, a_sums, a_scale, gate_e, up_e, phi, inv, n, k, top_k, tile * T::kBN, m0,
                                     left < 64u ? left : 64u);
       m0 += 64u;
     } else {
-      moe_gate_up_pass<WAVES, 3, 1>(lds, rows, a16, a_scale, gate_e, up_e, phi, inv, n, k, top_k, tile * T::kBN, m0, left);
+      moe_gate_up_pass<WAVES, 3, 1>(lds, rows, a16, a_sums, a_scale, gate_e, up_e, phi, inv, n, k, top_k, tile * T::kBN, m0, left);
       m0 += 32u;
     }
   }
 }
 
 // Dynamic LDS of the down kernel for passes of 32 RT rows: S weight stages, the row tables, the
-// rows as fp16 (2k + 16 bytes each).
+// rows as fp16 (2k + 16 bytes each), their sub-block sums (k / 8 bytes each).
 template <int WAVES>
 __host__ __device__ constexpr size_t moe_down_lds_bytes(int stages, int rt, uint32_t inter) {
-  return static_cast<size_t>(stages) * MoeTile<WAVES>::kWStage + 512u + 32u * rt * (2u * static_cast<size_t>(inter) + 16u);
+  return static_cast<size_t>(stages) * MoeTile<WAVES>::kWStage + 256u * rt +
+         32u * rt * (2u * static_cast<size_t>(inter) + 16u + inter / 8u);
 }
 
 // One pass of moe_down_kernel: rows m0 .. m0 + live of the sorted pairs (live <= 32 RT) against
@@ -443,9 +563,10 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
                                               uint32_t tile1, uint32_t m0, uint32_t live) {
   using T = MoeTile<WAVES>;
   float* row_scale = reinterpret_cast<float*>(dyn_lds + S * T::kWStage);
-  uint32_t* row_dst = reinterpret_cast<uint32_t*>(dyn_lds + S * T::kWStage + 256);
-  uint8_t* a_lds = dyn_lds + S * T::kWStage + 512;
-  const uint32_t a_stride = 2u * k + 16u;
+  uint32_t* row_dst = reinterpret_cast<uint32_t*>(dyn_lds + S * T::kWStage + 128 * RT);
+  uint8_t* a_lds = dyn_lds + S * T::kWStage + 256 * RT;
+  const uint32_t a_stride = 2u * k + 16u, sums_stride = k / 8u;
+  uint8_t* sums_lds = a_lds + 32u * RT * a_stride;
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t row_blocks = k / 256u, row_bytes = row_blocks * 144u;
@@ -456,9 +577,11 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
   // largest magnitude, then write the groups of 8 in the order the decode yields.
   if (wave < WAVES) {
     constexpr uint32_t kPer = WAVES * 2u;
-#pragma unroll
+    uint32_t tc = t;   // opaque, so that nothing derived from it is kept in registers between passes
+    asm volatile("" : "+v"(tc));
+#pragma nounroll
     for (int rt = 0; rt < RT; ++rt) {
-      const uint32_t row = rt * 32u + t / kPer, sub = t % kPer;
+      const uint32_t row = rt * 32u + tc / kPer, sub = tc % kPer;
       const uint32_t p = inv[m0 + (row < live ? row : live - 1u)];
       const float4* src = reinterpret_cast<const float4*>(phi + static_cast<size_t>(p) * k);
       float amax = 0.0f;
@@ -469,8 +592,10 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
 #pragma unroll
       for (uint32_t d = 1; d < kPer; d *= 2u) amax = fmaxf(amax, __shfl_xor(amax, d));
       const float s = row_scale_for(amax), inv_s = 1.0f / s;
-      for (uint32_t c = sub; c < k / 8u; c += kPer) {
-        *reinterpret_cast<half8_t*>(a_lds + row * a_stride + c * 16u) = to_f16_group(src[2 * c], src[2 * c + 1], inv_s);
+      for (uint32_t c = sub; c < k / 8u; c += kPer) {   // neighbouring threads hold neighbouring groups
+        const half8_t v = to_f16_group(src[2 * c], src[2 * c + 1], inv_s);
+        *reinterpret_cast<half8_t*>(a_lds + row * a_stride + c * 16u) = v;
+        store_subblock_sum(v, c, reinterpret_cast<_Float16*>(sums_lds + row * sums_stride));
       }
       if (sub == 0) row_scale[row] = s, row_dst[row] = p;
     }
@@ -508,6 +633,7 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
     const uint32_t l32 = lc & 31u, kg = lc >> 5;
     const uint8_t* w_lane = dyn_lds + (wave * 32u + l32) * 144u;
     const uint8_t* a_lane = a_lds + l32 * a_stride;
+    const uint8_t* s_lane = sums_lds + l32 * sums_stride + kg * 16u;
     float16_t acc[RT];
     uint32_t stage = 0;
     moe_compute_barrier();
@@ -515,17 +641,25 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
       zero_acc<RT>(acc);
       for (uint32_t blk = 0; blk < row_blocks; ++blk) {
         moe_block_mma<RT>(w_lane + stage * T::kWStage, kg, [&](uint32_t c) { return a_lane + (blk * 32u + c) * 16u; },
-                          32u * a_stride, acc);
+                          32u * a_stride, s_lane + blk * 32u, 32u * sums_stride, acc);
         moe_compute_barrier();
         stage = stage + 1u == S ? 0u : stage + 1u;
       }
+      // lane holds column `col` and rows 32 rt + 8 g + 4 kg + [0,4), g = 0..3: four table entries a read
       const uint32_t col = tile * T::kBN + wave * 32u + l32;
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-        for (int e16 = 0; e16 < 16; ++e16) {
-          const uint32_t row = rt * 32u + (e16 >> 2) * 8u + kg * 4u + (e16 & 3u);
-          if (row < live) rows[static_cast<size_t>(row_dst[row]) * n + col] = acc[rt][e16] * row_scale[row];
+        for (int g = 0; g < 4; ++g) {
+          const uint32_t row0 = rt * 32u + g * 8u + kg * 4u;
+          const uint4 dst4 = *reinterpret_cast<const uint4*>(row_dst + row0);
+          const float4 sc4 = *reinterpret_cast<const float4*>(row_scale + row0);
+          const uint32_t dst[4] = {dst4.x, dst4.y, dst4.z, dst4.w};
+          const float sc[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (row0 + i < live) rows[static_cast<size_t>(dst[i]) * n + col] = acc[rt][g * 4 + i] * sc[i];
+          }
         }
       }
     }
@@ -598,12 +732,13 @@ bool moe_resident_path(uint32_t hidden, uint32_t inter, uint32_t tokens) {
   return moe_down_lds_bytes<4>(2, 1, inter) <= kMoeLdsLimit && static_cast<uint64_t>(tokens) * hidden * 2 < (1ull << 32);
 }
 
-void launch_moe_gate_up_resident(const _Float16* a16, const float* a_scale, const uint8_t* gate, const uint8_t* up,
+void launch_moe_gate_up_resident(const _Float16* a16, const _Float16* a_sums, const float* a_scale, const uint8_t* gate,
+                                 const uint8_t* up,
                                  uint64_t gate_stride, uint64_t up_stride, float* phi, const uint32_t* seg,
                                  const uint32_t* inv, uint32_t hidden, uint32_t inter, uint32_t experts, uint32_t top_k,
                                  hipStream_t stream) {
   const uint32_t expert_groups = (experts + 7u) / 8u * 8u;
-  hipLaunchKernelGGL((moe_gate_up_kernel<8>), dim3(expert_groups * (inter / 256u)), dim3(MoeTile<8>::kThreads), 0, stream, a16, a_scale,
+  hipLaunchKernelGGL((moe_gate_up_kernel<8>), dim3(expert_groups * (inter / 256u)), dim3(MoeTile<8>::kThreads), 0, stream, a16, a_sums, a_scale,
                      gate, up, gate_stride, up_stride, phi, seg, inv, inter, hidden, experts, top_k);
 }
 
@@ -656,6 +791,7 @@ struct MoeWorkspace {
   uint32_t *seg, *pos, *inv;
   float *x_scale, *phi_scale;
   _Float16* a16;      // fp16 rows of x: one per token (resident path) or one per pair, gathered
+  _Float16* a_sums;   // resident path: the token rows' sub-block sums, hidden / 16 halves a row
   float *g, *u;       // pairs x inter each; g doubles as phi (fp32, pair order) on the resident path
   _Float16* phi16;
   float* rows;        // pairs x hidden
@@ -676,6 +812,7 @@ MoeWorkspace carve_moe_workspace(void* workspace, uint64_t pairs, uint64_t hidde
   w.x_scale = reinterpret_cast<float*>(take((pairs + 256) * 4));
   w.phi_scale = reinterpret_cast<float*>(take((pairs + 256) * 4));
   w.a16 = reinterpret_cast<_Float16*>(take(pairs * hidden * 2));
+  w.a_sums = reinterpret_cast<_Float16*>(take(pairs * hidden / 8));
   w.g = reinterpret_cast<float*>(take(pairs * inter * 4));
   w.u = reinterpret_cast<float*>(take(pairs * inter * 4));
   w.phi16 = reinterpret_cast<_Float16*>(take(pairs * inter * 2));
@@ -720,8 +857,8 @@ hipError_t launch_moe_ffn_q4k(const float* x, const uint8_t* gate, const uint8_t
   const MoeWorkspace ws = carve_moe_workspace(workspace, pairs, hidden, inter, experts);
   if (moe_resident_path(hidden, inter, tokens)) {
     hipLaunchKernelGGL(moe_prepare_kernel, dim3(1u + tokens), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos,
-                       ws.inv, x, ws.a16, ws.x_scale, hidden);
-    launch_moe_gate_up_resident(ws.a16, ws.x_scale, gate, up, gate_stride, up_stride, ws.g, ws.seg, ws.inv, hidden, inter,
+                       ws.inv, x, ws.a16, ws.a_sums, ws.x_scale, hidden);
+    launch_moe_gate_up_resident(ws.a16, ws.a_sums, ws.x_scale, gate, up, gate_stride, up_stride, ws.g, ws.seg, ws.inv, hidden, inter,
                                 experts, top_k, stream);
     launch_moe_down_resident(ws.g, down, down_stride, ws.rows, ws.seg, ws.inv, hidden, inter, experts, stream);
     launch_combine(ws.rows, wts, out, tokens, top_k, hidden, accumulate, stream);
@@ -753,8 +890,8 @@ hipError_t launch_moe_gate_up_q4k_grouped(const float* x, const uint8_t* gate, c
   const MoeWorkspace ws = carve_moe_workspace(workspace, pairs, hidden, inter, experts);
   if (moe_resident_path(hidden, inter, tokens)) {
     hipLaunchKernelGGL(moe_prepare_kernel, dim3(1u + tokens), dim3(1024), 0, stream, ids, pairs, experts, ws.seg, ws.pos,
-                       ws.inv, x, ws.a16, ws.x_scale, hidden);
-    launch_moe_gate_up_resident(ws.a16, ws.x_scale, gate, up, gate_stride, up_stride, phi, ws.seg, ws.inv, hidden, inter,
+                       ws.inv, x, ws.a16, ws.a_sums, ws.x_scale, hidden);
+    launch_moe_gate_up_resident(ws.a16, ws.a_sums, ws.x_scale, gate, up, gate_stride, up_stride, phi, ws.seg, ws.inv, hidden, inter,
                                 experts, top_k, stream);
     return hipGetLastError();
   }

@@ -124,14 +124,11 @@ __device__ __forceinline__ BlockHead load_block_head(const uint8_t* raw) {
 // same shifted down one byte, for bytes 1 and 3) are carried from that call.  MIX selects
 // decode_pair_mix.
 template <int SB, bool MIX = false>
-__device__ __forceinline__ void decode_subblock(const uint8_t* raw, uint32_t kg, const BlockHead& h, uint32_t (&qw)[4],
-                                                uint32_t (&qs8)[4], half8_t (&b)[2]) {
+__device__ __forceinline__ void decode_subblock_words(const uint2& q0, const uint2& q1, const BlockHead& h, uint32_t (&qw)[4],
+                                                      uint32_t (&qs8)[4], half8_t (&b)[2]) {
   constexpr int kHi = SB & 1;
   const ScaleMin sm = scale_min_f32<SB>(h.sbytes, h.d, h.ndmin);
-  if (kHi == 0) {
-    const uint8_t* qp = raw + 16 + (SB >> 1) * 32 + kg * 8u;
-    const uint2 q0 = *reinterpret_cast<const uint2*>(qp);
-    const uint2 q1 = *reinterpret_cast<const uint2*>(qp + 16);
+  if (kHi == 0) {   // q0, q1: bytes (SB/2)*32 + 8 kg + [0,8) and the same + 16 of the row's quants
     qw[0] = q0.x, qw[1] = q0.y, qw[2] = q1.x, qw[3] = q1.y;
 #pragma unroll
     for (int x = 0; x < 4; ++x) qs8[x] = qw[x] >> 8;
@@ -142,6 +139,20 @@ __device__ __forceinline__ void decode_subblock(const uint8_t* raw, uint32_t kg,
     const half2_t p0 = pair(qw[2 * tt]), p1 = pair(qs8[2 * tt]), p2 = pair(qw[2 * tt + 1]), p3 = pair(qs8[2 * tt + 1]);
     b[tt] = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
   }
+}
+
+// The same with the quant words read from the raw row (an even SB reads, its odd successor
+// reuses).
+template <int SB, bool MIX = false>
+__device__ __forceinline__ void decode_subblock(const uint8_t* raw, uint32_t kg, const BlockHead& h, uint32_t (&qw)[4],
+                                                uint32_t (&qs8)[4], half8_t (&b)[2]) {
+  uint2 q0 = make_uint2(0u, 0u), q1 = q0;
+  if ((SB & 1) == 0) {
+    const uint8_t* qp = raw + 16 + (SB >> 1) * 32 + kg * 8u;
+    q0 = *reinterpret_cast<const uint2*>(qp);
+    q1 = *reinterpret_cast<const uint2*>(qp + 16);
+  }
+  decode_subblock_words<SB, MIX>(q0, q1, h, qw, qs8, b);
 }
 
 // Wavefronts of a BM x BN tile whose wavefronts each own WM rows x WN columns.

@@ -573,9 +573,36 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
   const uint32_t total = (tile1 - tile0) * row_blocks;
   const uint32_t lds_w = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)dyn_lds));
 
-  // The fp16 copy of the pass's rows: the compute wavefronts' (WAVES * 2) threads a row take its
-  // largest magnitude, then write the groups of 8 in the order the decode yields.
-  if (wave < WAVES) {
+  // Iteration `it` is block it % row_blocks of tile tile0 + it / row_blocks; stages and waits
+  // as in moe_gate_up_pass.  The loader requests the first weight stages while the other
+  // wavefronts stage the rows.
+  if (wave == WAVES) {
+    uint32_t ll = lane;   // as in moe_gate_up_pass
+    asm volatile("" : "+v"(ll));
+    uint32_t w_src[T::kWBlocks];
+    moe_weight_offsets<WAVES>(ll, row_bytes, w_src);
+    uint32_t tile_i = tile0, blk_i = 0;   // S - 1 iterations ahead
+    auto issue_next = [&](uint32_t stage) {
+      moe_issue_weights<WAVES>(down_e + static_cast<size_t>(tile_i) * T::kBN * row_bytes + blk_i * 144u, w_src,
+                               lds_w + stage * T::kWStage);
+      if (++blk_i == row_blocks) blk_i = 0, ++tile_i;
+    };
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+      if (static_cast<uint32_t>(s) < total) issue_next(s);
+    }
+    asm volatile("s_barrier" ::: "memory");   // the rows are staged; the weight loads stay in flight
+    moe_loader_barrier<(S - 2) * T::kWBlocks>(total >= static_cast<uint32_t>(S - 1));
+    uint32_t stage = 0;
+    for (uint32_t it = 0; it < total; ++it) {
+      const bool more = it + (S - 1) < total;
+      if (more) issue_next(stage == 0 ? S - 1 : stage - 1u);
+      moe_loader_barrier<(S - 2) * T::kWBlocks>(more);
+      stage = stage + 1u == S ? 0u : stage + 1u;
+    }
+  } else {
+    // The fp16 copy of the pass's rows: the compute wavefronts' (WAVES * 2) threads a row take its
+    // largest magnitude, then write the groups of 8 in the order the decode yields.
     constexpr uint32_t kPer = WAVES * 2u;
     uint32_t tc = t;   // opaque, so that nothing derived from it is kept in registers between passes
     asm volatile("" : "+v"(tc));
@@ -599,35 +626,7 @@ __device__ __forceinline__ void moe_down_pass(uint8_t* dyn_lds, const float* __r
       }
       if (sub == 0) row_scale[row] = s, row_dst[row] = p;
     }
-  }
-  __syncthreads();
-
-  // Iteration `it` is block it % row_blocks of tile tile0 + it / row_blocks; stages and waits
-  // as in moe_gate_up_pass.
-  if (wave == WAVES) {
-    uint32_t ll = lane;   // as in moe_gate_up_pass
-    asm volatile("" : "+v"(ll));
-    uint32_t w_src[T::kWBlocks];
-    moe_weight_offsets<WAVES>(ll, row_bytes, w_src);
-    uint32_t tile_i = tile0, blk_i = 0;   // S - 1 iterations ahead
-    auto issue_next = [&](uint32_t stage) {
-      moe_issue_weights<WAVES>(down_e + static_cast<size_t>(tile_i) * T::kBN * row_bytes + blk_i * 144u, w_src,
-                               lds_w + stage * T::kWStage);
-      if (++blk_i == row_blocks) blk_i = 0, ++tile_i;
-    };
-#pragma unroll
-    for (int s = 0; s < S - 1; ++s) {
-      if (static_cast<uint32_t>(s) < total) issue_next(s);
-    }
-    moe_loader_barrier<(S - 2) * T::kWBlocks>(total >= static_cast<uint32_t>(S - 1));
-    uint32_t stage = 0;
-    for (uint32_t it = 0; it < total; ++it) {
-      const bool more = it + (S - 1) < total;
-      if (more) issue_next(stage == 0 ? S - 1 : stage - 1u);
-      moe_loader_barrier<(S - 2) * T::kWBlocks>(more);
-      stage = stage + 1u == S ? 0u : stage + 1u;
-    }
-  } else {
+    moe_compute_barrier();   // the staged rows
     uint32_t lc = lane;   // as the loader's copy
     asm volatile("" : "+v"(lc));
     const uint32_t l32 = lc & 31u, kg = lc >> 5;

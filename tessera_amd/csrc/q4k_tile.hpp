@@ -66,18 +66,6 @@ __device__ __forceinline__ half2_t decode_pair(uint32_t x, float dsc24, float nd
                  static_cast<_Float16>(fmaf(static_cast<float>(q[1]), dsc24, ndmm))};
 }
 
-// decode_pair with the two instructions spelled out (the result's halves are written in place by
-// v_fma_mixlo_f16 / v_fma_mixhi_f16): for kernels where the compiler picks v_fma_mix_f32 and a
-// separate pack instead, which costs a third instruction per pair.
-template <int HI>
-__device__ __forceinline__ half2_t decode_pair_mix(uint32_t x, float dsc24, float ndmm) {
-  const uint32_t q = x & (HI ? 0x00F000F0u : 0x000F000Fu);
-  uint32_t d;
-  asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(d) : "v"(q), "v"(dsc24), "v"(ndmm));
-  asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(d) : "v"(q), "v"(dsc24), "v"(ndmm));
-  return bit_cast<half2_t>(d);
-}
-
 // The 6-bit scales and mins of a super-block, one byte each (src/core/numerics/quant.cpp:58-70):
 // sc[0], mn[0] hold sub-blocks 0..3, sc[1], mn[1] sub-blocks 4..7.
 struct ScaleBytes {
@@ -121,38 +109,26 @@ __device__ __forceinline__ BlockHead load_block_head(const uint8_t* raw) {
 // the weights 16t + 8kg + [0,8) in the order 0,2,1,3,4,6,5,7.  Sub-block SB lives in the low
 // (even SB) or high nibbles of bytes (SB/2)*32 + [0,32) (src/core/numerics/quant.cpp:656-675);
 // an odd SB decodes the bytes its even predecessor loaded, so `qw` (the words) and `qs8` (the
-// same shifted down one byte, for bytes 1 and 3) are carried from that call.  MIX selects
-// decode_pair_mix.
-template <int SB, bool MIX = false>
-__device__ __forceinline__ void decode_subblock_words(const uint2& q0, const uint2& q1, const BlockHead& h, uint32_t (&qw)[4],
-                                                      uint32_t (&qs8)[4], half8_t (&b)[2]) {
+// same shifted down one byte, for bytes 1 and 3) are carried from that call.
+template <int SB>
+__device__ __forceinline__ void decode_subblock(const uint8_t* raw, uint32_t kg, const BlockHead& h, uint32_t (&qw)[4],
+                                                uint32_t (&qs8)[4], half8_t (&b)[2]) {
   constexpr int kHi = SB & 1;
   const ScaleMin sm = scale_min_f32<SB>(h.sbytes, h.d, h.ndmin);
-  if (kHi == 0) {   // q0, q1: bytes (SB/2)*32 + 8 kg + [0,8) and the same + 16 of the row's quants
+  if (kHi == 0) {
+    const uint8_t* qp = raw + 16 + (SB >> 1) * 32 + kg * 8u;
+    const uint2 q0 = *reinterpret_cast<const uint2*>(qp);
+    const uint2 q1 = *reinterpret_cast<const uint2*>(qp + 16);
     qw[0] = q0.x, qw[1] = q0.y, qw[2] = q1.x, qw[3] = q1.y;
 #pragma unroll
     for (int x = 0; x < 4; ++x) qs8[x] = qw[x] >> 8;
   }
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt) {
-    auto pair = [&](uint32_t x) { return MIX ? decode_pair_mix<kHi>(x, sm.dsc, sm.ndmm) : decode_pair<kHi>(x, sm.dsc, sm.ndmm); };
-    const half2_t p0 = pair(qw[2 * tt]), p1 = pair(qs8[2 * tt]), p2 = pair(qw[2 * tt + 1]), p3 = pair(qs8[2 * tt + 1]);
+    const half2_t p0 = decode_pair<kHi>(qw[2 * tt], sm.dsc, sm.ndmm), p1 = decode_pair<kHi>(qs8[2 * tt], sm.dsc, sm.ndmm);
+    const half2_t p2 = decode_pair<kHi>(qw[2 * tt + 1], sm.dsc, sm.ndmm), p3 = decode_pair<kHi>(qs8[2 * tt + 1], sm.dsc, sm.ndmm);
     b[tt] = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
   }
-}
-
-// The same with the quant words read from the raw row (an even SB reads, its odd successor
-// reuses).
-template <int SB, bool MIX = false>
-__device__ __forceinline__ void decode_subblock(const uint8_t* raw, uint32_t kg, const BlockHead& h, uint32_t (&qw)[4],
-                                                uint32_t (&qs8)[4], half8_t (&b)[2]) {
-  uint2 q0 = make_uint2(0u, 0u), q1 = q0;
-  if ((SB & 1) == 0) {
-    const uint8_t* qp = raw + 16 + (SB >> 1) * 32 + kg * 8u;
-    q0 = *reinterpret_cast<const uint2*>(qp);
-    q1 = *reinterpret_cast<const uint2*>(qp + 16);
-  }
-  decode_subblock_words<SB, MIX>(q0, q1, h, qw, qs8, b);
 }
 
 // Wavefronts of a BM x BN tile whose wavefronts each own WM rows x WN columns.

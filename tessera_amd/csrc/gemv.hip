@@ -1182,6 +1182,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // when rows are long.
   constexpr int kMaxWaves = MAXT / kWave;
   __shared__ float red[2][D][P][R][LR ? 1 : kMaxWaves];
+  // Rows whose chunk count is a multiple of 16: an aligned run of 16 lanes never straddles two
+  // rows, so one four-step sum per run replaces the two masked six-step sums over the wavefront,
+  // and the threads that store add a row's runs instead of its wavefronts.
+  __shared__ float red16[2][D][R][LR ? 1 : MAXT / 16];
   __shared__ float part[2][D][R][LR ? MAXT : 1];
 
   if constexpr (k_slices<Codec>::value) {     // blockIdx.y = K slice and output region
@@ -1205,6 +1209,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // infinity among one row's weights must not reach its neighbour's sum (0 * inf = NaN), nor may
   // what an idle lane computed from the chunk it loaded for company.
   const bool to_a = valid && prow == row_a, to_b = valid && prow != row_a;
+  const bool by16 = (cpr & 15u) == 0u;   // uniform
 
   // Groups [g0, g1) belong to this workgroup.  A group index past its end is clamped to its
   // last group for the loads (a prefetch must not pull the next workgroup's rows, which would
@@ -1308,7 +1313,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       if constexpr (decltype(refill)::value) fetch(g + kGroupsPerRound, d, frag[d]);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        if (two) {
+        if (by16) {
+          const float s16 = row16_sum(valid ? v[r] : 0.0f);
+          if ((lane & 15u) == 0u) red16[buf][d][r][t >> 4] = s16;
+        } else if (two) {
           const float sa = wave_sum_last(to_a ? v[r] : 0.0f);
           const float sb = wave_sum_last(to_b ? v[r] : 0.0f);
           if (lane == 63u) {
@@ -1327,9 +1335,13 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       const uint32_t row = (g + d) * PR + po;
       if (g + d < g1 && row < n) {
         auto slot_sum = [&](uint32_t stage) {
-          const uint32_t w_lo = (po * cpr) >> 6, w_hi = ((po + 1u) * cpr - 1u) >> 6;
           float sum = 0.0f;
-          for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][stage][po][r][w];
+          if (by16) {
+            for (uint32_t q = (po * cpr) >> 4; q < ((po + 1u) * cpr) >> 4; ++q) sum += red16[buf][stage][r][q];
+          } else {
+            const uint32_t w_lo = (po * cpr) >> 6, w_hi = ((po + 1u) * cpr - 1u) >> 6;
+            for (uint32_t w = w_lo; w <= w_hi; ++w) sum += red[buf][stage][po][r][w];
+          }
           return sum;
         };
         if constexpr (kPaired) {

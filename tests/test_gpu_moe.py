@@ -101,7 +101,8 @@ def forward_rows(backend, x, ids, wts, gate, up, down, hidden, inter, experts):
     return backend.CopyD2H(d_out, dtype=np.float32).reshape(rows, hidden)
 
 
-@pytest.mark.parametrize("rows,experts,hidden,inter,top_k", [(7, 16, 512, 256, 4), (16, 12, 256, 512, 3)])
+@pytest.mark.parametrize("rows,experts,hidden,inter,top_k", [(7, 16, 512, 256, 4), (16, 12, 256, 512, 3),
+                                                             (8, 8, 2048, 512, 8)])   # the last: four weight rows a wavefront
 def test_rows_match_oracle(backend, rows, experts, hidden, inter, top_k):
     g = synth.rng(rows + experts + hidden)
     gate, up, down = expert_tensors(g, experts, hidden, inter)
@@ -271,7 +272,8 @@ def test_grouped_ffn_skewed_routing(backend):
 
 
 @pytest.mark.parametrize("experts,hidden,inter,top_k,rows", [(16, 512, 256, 4, 1), (8, 2048, 512, 8, 1),
-                                                              (5, 260, 768, 2, 3), (256, 2048, 512, 8, 2)])
+                                                              (5, 260, 768, 2, 3), (256, 2048, 512, 8, 2),
+                                                              (24, 2048, 512, 8, 8)])   # the last: four weight rows a wavefront
 def test_down_q6k_matches_oracle(backend, experts, hidden, inter, top_k, rows):
     """moe_experts_down_q6k (the reference loads it next to the Q4_K one,
     src/models/qwen3_5/moe.cpp:107-115): out[t] (+)= sum_slot wts[t][slot] * D_{ids[t][slot]} phi[t][slot],

@@ -1613,17 +1613,41 @@ hipError_t launch_gemv_r(const typename Codec::Args& args, float* c, uint32_t n,
   return hipErrorInvalidValue;
 }
 
+// The activation row of the generic kernels, staged in LDS when it is short enough: a lane's
+// slice is a few hundred contiguous bytes, so fetched straight from memory every lane of a load
+// touches its own cache line (64 lines an instruction), which for the routed-expert rows (2048 or
+// 4096 activations against two 1152-byte weight rows a wavefront) cost more than the weights.
+// The workgroup copies the row with coalesced loads; the copy is padded as StagedX expects.
+constexpr uint32_t kGenericXFloats = 8192;
+__device__ __forceinline__ float* generic_x_area() {
+  __shared__ __attribute__((aligned(16))) float xs[kGenericXFloats + kGenericXFloats / 16u];
+  return xs;
+}
+template <class Codec>
+__device__ __forceinline__ bool stage_generic_x(const typename Codec::Args& args) {
+  if constexpr (Codec::kStageX) {
+    if (args.k > kGenericXFloats) return false;   // uniform
+    float* xs = generic_x_area();
+    for (uint32_t e = threadIdx.x * 4u; e < args.k; e += blockDim.x * 4u) {
+      *reinterpret_cast<float4*>(&xs[StagedX::pad(e)]) = *reinterpret_cast<const float4*>(args.a + e);
+    }
+    __syncthreads();
+    return true;
+  } else {
+    return false;
+  }
+}
+
 // Fallback for shapes the register-resident mapping does not cover (a row longer
 // than 1024 chunks): one wavefront per weight row, lanes stride over the chunks and
-// fetch their activations from memory each time.  Correct for any K the codec
-// accepts; not tuned.
+// fetch their activations from LDS (short rows) or from memory each time.  Correct for any K the
+// codec accepts; not tuned.
 template <class Codec>
 __global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args args,
                                                            float* __restrict__ c, uint32_t n,
                                                            uint32_t cpr, uint32_t ldc) {
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (row >= n) return;  // whole wavefront leaves together
   if constexpr (requires { Codec::batch(args, 0u); }) {   // one activation row per grid.y
     Codec::batch(args, blockIdx.y);
     c += static_cast<size_t>(blockIdx.y) * ldc;
@@ -1631,15 +1655,59 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(typename Codec::Args 
   // A codec over two matrices (kTwoMatrices) takes the same row of both against one copy of the
   // activations and stores combine(first, second).
   constexpr bool kTwo = requires { Codec::kTwoMatrices; };
+  // Order of the requests: the activation row (into registers, on its way to LDS), then the
+  // fragments of the lane's first chunk; loads return in order, so the row is staged and the
+  // barrier passed while the weights are still on their way (the barrier orders LDS only).
+  constexpr int kXPer = kGenericXFloats / 4 / 256;
+  bool staged = false;
+  if constexpr (Codec::kStageX) staged = args.k <= kGenericXFloats;   // uniform
+  const bool live = row < n;
+  // rows and chunks past the end fetch the last ones (never used), so nothing here is conditional
+  const uint32_t row_in = live ? row : n - 1u, chunk_in = lane < cpr ? lane : cpr - 1u;
+  typename Codec::Frag f, f2;
+  if constexpr (Codec::kStageX) {
+    float4 x0, x1, x2, x3, x4, x5, x6, x7;
+    static_assert(kXPer == 8, "eight 16-byte pieces a thread");
+    const uint32_t last = args.k - 4u;
+    auto piece = [&](uint32_t i) {
+      const uint32_t e = (threadIdx.x + i * 256u) * 4u;
+      return *reinterpret_cast<const float4*>(args.a + (staged && e < args.k ? e : last));
+    };
+    x0 = piece(0), x1 = piece(1), x2 = piece(2), x3 = piece(3), x4 = piece(4), x5 = piece(5), x6 = piece(6), x7 = piece(7);
+    {
+      const Lane ln = Codec::make_lane(args, cpr, chunk_in, 0u);
+      Codec::load(args, ln, row_in, cpr, f);
+      if constexpr (kTwo) Codec::load(args, ln, row_in, cpr, f2, 1);
+    }
+    if (staged) {
+      float* xs = generic_x_area();
+      auto put = [&](uint32_t i, const float4& v) {
+        const uint32_t e = (threadIdx.x + i * 256u) * 4u;
+        if (e < args.k) *reinterpret_cast<float4*>(&xs[StagedX::pad(e)]) = v;
+      };
+      put(0, x0), put(1, x1), put(2, x2), put(3, x3), put(4, x4), put(5, x5), put(6, x6), put(7, x7);
+      lds_barrier();
+    }
+  } else {
+    const Lane ln = Codec::make_lane(args, cpr, chunk_in, 0u);
+    Codec::load(args, ln, row_in, cpr, f);
+    if constexpr (kTwo) Codec::load(args, ln, row_in, cpr, f2, 1);
+  }
+  if (!live) return;  // whole wavefront leaves together
   float acc = 0.0f, acc2 = 0.0f;
   for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
     typename Codec::template X<1> x;
-    typename Codec::Frag f, f2;
-    const Lane ln = Codec::make_lane(args, cpr, chunk, 0u);
-    Codec::load(args, ln, row, cpr, f);
-    if constexpr (kTwo) Codec::load(args, ln, row, cpr, f2, 1);
+    if (chunk != lane) {   // later chunks: fetched here
+      const Lane ln = Codec::make_lane(args, cpr, chunk, 0u);
+      Codec::load(args, ln, row, cpr, f);
+      if constexpr (kTwo) Codec::load(args, ln, row, cpr, f2, 1);
+    }
     if constexpr (Codec::kStageX) {
-      Codec::template load_x<1>(args, chunk, true, x, GlobalX{args.a, args.k});
+      if (staged) {
+        Codec::template load_x<1>(args, chunk, true, x, StagedX{generic_x_area(), 0u, kGenericXFloats + kGenericXFloats / 16u});
+      } else {
+        Codec::template load_x<1>(args, chunk, true, x, GlobalX{args.a, args.k});
+      }
     } else {
       Codec::template load_x<1>(args, chunk, true, x, 0);
     }
@@ -1671,11 +1739,12 @@ __global__ __launch_bounds__(256) void gemv_generic_rows_kernel(typename Codec::
                                                                 uint32_t n, uint32_t cpr, uint32_t ldc) {
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW;
-  if (row0 >= n) return;  // whole wavefront leaves together
   if constexpr (requires { Codec::batch(args, 0u); }) {   // one activation row per grid.y
     Codec::batch(args, blockIdx.y);
     c += static_cast<size_t>(blockIdx.y) * ldc;
   }
+  const bool staged = stage_generic_x<Codec>(args);
+  if (row0 >= n) return;  // whole wavefront leaves together
   constexpr bool kTwo = requires { Codec::kTwoMatrices; };
   float acc[RPW], acc2[RPW];
 #pragma unroll
@@ -1683,7 +1752,11 @@ __global__ __launch_bounds__(256) void gemv_generic_rows_kernel(typename Codec::
   for (uint32_t chunk = lane; chunk < cpr; chunk += 64u) {
     typename Codec::template X<1> x;
     if constexpr (Codec::kStageX) {
-      Codec::template load_x<1>(args, chunk, true, x, GlobalX{args.a, args.k});
+      if (staged) {
+        Codec::template load_x<1>(args, chunk, true, x, StagedX{generic_x_area(), 0u, kGenericXFloats + kGenericXFloats / 16u});
+      } else {
+        Codec::template load_x<1>(args, chunk, true, x, GlobalX{args.a, args.k});
+      }
     } else {
       Codec::template load_x<1>(args, chunk, true, x, 0);
     }

@@ -295,14 +295,19 @@ __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t* __restr
   const uint8_t* base = w + blk * kQ4KBlockBytes;
   const uint4 hd = load_u4(base);
   const uint4 q = load_u4(base + 16 + j * 16);
-  const uint8_t* p = reinterpret_cast<const uint8_t*>(&hd) + 4;
+  // byte i of the 12 scale bytes, picked out of the header's words (an indexed byte array would
+  // live in scratch memory)
+  auto p = [&](uint32_t i) {
+    const uint32_t word = i < 4u ? hd.y : i < 8u ? hd.z : hd.w;
+    return (word >> (8u * (i & 3u))) & 0xFFu;
+  };
   auto scale_min = [&](uint32_t sb, uint32_t& sc, uint32_t& mn) {
     if (sb < 4) {
-      sc = p[sb] & 63u;
-      mn = p[sb + 4] & 63u;
+      sc = p(sb) & 63u;
+      mn = p(sb + 4) & 63u;
     } else {
-      sc = (p[sb + 4] & 15u) | ((p[sb - 4] >> 6) << 4);
-      mn = (p[sb + 4] >> 4) | ((p[sb] >> 6) << 4);
+      sc = (p(sb + 4) & 15u) | ((p(sb - 4) >> 6) << 4);
+      mn = (p(sb + 4) >> 4) | ((p(sb) >> 6) << 4);
     }
   };
   uint32_t sca, mna, scb, mnb;
@@ -312,11 +317,12 @@ __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t* __restr
   const float s0 = d * static_cast<float>(sca), o0 = dmin * static_cast<float>(mna);
   const float s1 = d * static_cast<float>(scb), o1 = dmin * static_cast<float>(mnb);
   float* dst = out + blk * kQ4KBlockElems + g * 64 + h * 16;
-  const uint8_t* qb = reinterpret_cast<const uint8_t*>(&q);
+  const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    dst[i] = s0 * static_cast<float>(qb[i] & 15u) - o0;
-    dst[32 + i] = s1 * static_cast<float>(qb[i] >> 4) - o1;
+    const uint32_t byte = (qw[i >> 2] >> (8 * (i & 3))) & 0xFFu;
+    dst[i] = s0 * static_cast<float>(byte & 15u) - o0;
+    dst[32 + i] = s1 * static_cast<float>(byte >> 4) - o1;
   }
 }
 

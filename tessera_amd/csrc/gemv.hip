@@ -2028,9 +2028,17 @@ hipError_t launch_fp8_gemv_as(const float* a, const uint8_t* w, const float* s, 
       float* out = c + static_cast<size_t>(r0) * n;
       hipError_t e;
       uint32_t took;
-      if (m - r0 >= 2) {
-        e = launch_gemv_r<Fp8WideCodec, 2, 1024, 2, 1>(args, out, n, k, n, stream), took = 2;
-      } else {
+      // (with block scales two rows a pass no longer fit the registers of a 1024-thread
+      // workgroup, and a kernel that spills pays for its scratch segment at every dispatch)
+      if constexpr (!BLOCK) {
+        if (m - r0 >= 2) {
+          e = launch_gemv_r<Fp8WideCodec, 2, 1024, 2, 1>(args, out, n, k, n, stream), took = 2;
+          if (e != hipSuccess) return e;
+          r0 += took;
+          continue;
+        }
+      }
+      {
         e = launch_gemv_r<Fp8WideCodec, 1, 1024, 2, 1>(args, out, n, k, n, stream), took = 1;
       }
       if (e != hipSuccess) return e;

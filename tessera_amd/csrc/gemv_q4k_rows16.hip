@@ -36,7 +36,8 @@
 // it needs write back and invalidate the L2 of its XCD under the workgroups still streaming
 // weights.)  Stamps of the 100 MHz counter inside the kernel show what bounds it: a wavefront
 // that has a SIMD's issue slots to itself needs 0.5 us a unit and never waits for weights; ten
-// wavefronts on four SIMDs put three on two of them, and those finish last.
+// wavefronts on four SIMDs put three on two of them, and those finish last -- hence K parts of
+// twelve and eight columns where the column count allows (r16_plan_unequal).
 
 #include <type_traits>
 
@@ -52,6 +53,13 @@ constexpr int kKL = 3;                    // 16-byte pieces a lane brings per un
 constexpr uint32_t kARowBytes = 256u * 2u + 16u;   // one matrix row of a block in the conversion area
 constexpr uint32_t kConvRows = 8;         // matrix rows converted at a time (four activation rows, hi and lo)
 
+// A K part of unequal size (see r16_plan): the workgroups first_wg .. of the launch own its block
+// columns b0 .. b0 + nbp - 1, one a wavefront, tiles_per_wg tiles each.
+struct R16Part {
+  uint32_t first_wg, tiles_per_wg, b0, nbp, tiles_per_sync;
+};
+constexpr uint32_t kMaxParts = 8;
+
 struct R16Args {
   const float* a;          // m x k
   const uint8_t* w;        // n rows of k/256 blocks
@@ -61,6 +69,8 @@ struct R16Args {
   uint32_t tiles_per_wg;
   uint32_t blocks_per_part;
   uint32_t tiles_per_sync;   // tiles between two meetings of the wavefronts' partial sums
+  uint32_t n_parts;          // 0: equal parts, gridDim.y of them; else the table below, gridDim.y = 1
+  R16Part part[kMaxParts];
 };
 
 // 16 bytes from base + voff straight into LDS at lds_addr + 16 * lane (no register in between).
@@ -74,15 +84,22 @@ __device__ __forceinline__ uint32_t dpp_umax16(uint32_t v) {
   const uint32_t moved = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), kCtrl, kRowMask, 0xF, false));
   return v > moved ? v : moved;
 }
-// Largest value over the 64 lanes, DPP only; uniform result.
-__device__ __forceinline__ uint32_t wave_umax16(uint32_t v) {
-  v = dpp_umax16<0xB1, 0xF>(v);    // quad_perm [1,0,3,2]
-  v = dpp_umax16<0x4E, 0xF>(v);    // quad_perm [2,3,0,1]
-  v = dpp_umax16<0x141, 0xF>(v);   // row_half_mirror
-  v = dpp_umax16<0x140, 0xF>(v);   // row_mirror
-  v = dpp_umax16<0x142, 0xA>(v);   // row_bcast:15
-  v = dpp_umax16<0x143, 0xC>(v);   // row_bcast:31
-  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63));
+// Largest value over the 64 lanes of each of eight registers, DPP only; uniform results.
+__device__ __forceinline__ void wave_umax16_x8(uint32_t (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = dpp_umax16<0xB1, 0xF>(v[i]);    // quad_perm [1,0,3,2]
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = dpp_umax16<0x4E, 0xF>(v[i]);    // quad_perm [2,3,0,1]
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = dpp_umax16<0x141, 0xF>(v[i]);   // row_half_mirror
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = dpp_umax16<0x140, 0xF>(v[i]);   // row_mirror
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = dpp_umax16<0x142, 0xA>(v[i]);   // row_bcast:15
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = dpp_umax16<0x143, 0xC>(v[i]);   // row_bcast:31
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v[i]), 63));
 }
 template <int kCtrl>
 __device__ __forceinline__ float dpp_fadd16(float v) {
@@ -113,13 +130,25 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t waves = blockDim.x >> 6;
   const uint32_t nrow = lane & 15u, gq = lane >> 4;        // weight row of the tile, K chunk of a sub-block
-  const uint32_t nbp = p.blocks_per_part;
-  const uint32_t b0 = blockIdx.y * nbp;                    // first block of this K part
+  uint32_t nbp = p.blocks_per_part, b0 = blockIdx.y * nbp;   // block columns of this K part
+  uint32_t tiles_per_wg = p.tiles_per_wg, tiles_per_sync = p.tiles_per_sync, wg = blockIdx.x;
+  uint32_t part_index = blockIdx.y, n_parts = gridDim.y;
+  if (p.n_parts != 0u) {
+    part_index = 0;
+    for (uint32_t i = 1; i < p.n_parts; ++i) part_index = blockIdx.x >= p.part[i].first_wg ? i : part_index;
+    const R16Part& pt = p.part[part_index];
+    nbp = pt.nbp, b0 = pt.b0, tiles_per_wg = pt.tiles_per_wg, tiles_per_sync = pt.tiles_per_sync;
+    wg = blockIdx.x - pt.first_wg, n_parts = p.n_parts;
+  }
+  // wavefronts of the launch that this part has no column for leave before the first barrier
+  // (a barrier waits for the surviving wavefronts only)
+  const uint32_t live_waves = (nbp + BW - 1u) / BW;
+  if (wave >= live_waves) return;
   const uint32_t sbs = p.k / 256u, row_bytes = sbs * 144u;
   const uint32_t tiles_total = (p.n + kTile - 1u) / kTile;
-  const uint32_t tile0 = blockIdx.x * p.tiles_per_wg;
+  const uint32_t tile0 = wg * tiles_per_wg;
   if (tile0 >= tiles_total) return;                        // whole workgroup leaves together
-  const uint32_t tiles = tile0 + p.tiles_per_wg <= tiles_total ? p.tiles_per_wg : tiles_total - tile0;
+  const uint32_t tiles = tile0 + tiles_per_wg <= tiles_total ? tiles_per_wg : tiles_total - tile0;
   const uint32_t row0 = tile0 * kTile;
 
   uint8_t* ring = lds + wave * (RING * kUnitBytes);
@@ -133,8 +162,8 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
 
   // Block columns of this wavefront inside the part: wave, wave + W (BW = 2); one past the part
   // is computed with zero activations on the part's last block.
-  auto col_live = [&](uint32_t jb) { return wave + jb * waves < nbp; };
-  auto col = [&](uint32_t jb) { return b0 + (col_live(jb) ? wave + jb * waves : nbp - 1u); };
+  auto col_live = [&](uint32_t jb) { return wave + jb * live_waves < nbp; };
+  auto col = [&](uint32_t jb) { return b0 + (col_live(jb) ? wave + jb * live_waves : nbp - 1u); };
 
   // ---- the activations are requested first: a wavefront's loads return in order, so behind the
   // weight ring they would wait for it.  Requested by hand, because the compiler's own waits count
@@ -204,45 +233,58 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
   for (int jb = 0; jb < BW; ++jb) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
+      // largest magnitude of each row's block as bits (integer order = magnitude order; NaN and
+      // infinity sort above every finite value, so the same reduction finds them); the eight
+      // reductions go step by step side by side, so that no step waits for its predecessor
+      uint32_t mx[8];
+#pragma unroll
+      for (int r8 = 0; r8 < 8; ++r8) {
+        const float4_t v = xv[jb * MT + mt][r8];
+        const uint32_t m0 = bit_cast<uint32_t>(v[0]) & 0x7FFFFFFFu, m1 = bit_cast<uint32_t>(v[1]) & 0x7FFFFFFFu;
+        const uint32_t m2 = bit_cast<uint32_t>(v[2]) & 0x7FFFFFFFu, m3 = bit_cast<uint32_t>(v[3]) & 0x7FFFFFFFu;
+        mx[r8] = max(max(m0, m1), max(m2, m3));
+      }
+      wave_umax16_x8(mx);
 #pragma unroll
       for (int r8 = 0; r8 < 8; ++r8) {
         const uint32_t r = mt * 8u + r8;
-        float4_t v = xv[jb * MT + mt][r8];
-        if (r >= p.m || !col_live(jb)) v = float4_t{0.f, 0.f, 0.f, 0.f};
-        // largest magnitude of the block as bits (integer order = magnitude order; NaN and
-        // infinity sort above every finite value, so the same reduction finds them)
-        const uint32_t m0 = bit_cast<uint32_t>(v[0]) & 0x7FFFFFFFu, m1 = bit_cast<uint32_t>(v[1]) & 0x7FFFFFFFu;
-        const uint32_t m2 = bit_cast<uint32_t>(v[2]) & 0x7FFFFFFFu, m3 = bit_cast<uint32_t>(v[3]) & 0x7FFFFFFFu;
-        uint32_t mx = max(max(m0, m1), max(m2, m3));
-        mx = wave_umax16(mx);
-        const uint32_t e = mx >> 23;
-        int se = 262 - static_cast<int>(e);                       // amax * s in [2^8, 2^9)
-        se = se < 1 ? 1 : (se > 254 ? 254 : se);
-        const float s = (e == 0u || e == 0xFFu) ? 1.0f : bit_cast<float>(static_cast<uint32_t>(se) << 23);
-        // NaN or infinity anywhere in the block: the block's factor becomes NaN, as the reference's sum would
-        const float inv = e == 0xFFu ? bit_cast<float>(0x7FC00000u)
-                                     : (e == 0u ? 1.0f : bit_cast<float>(static_cast<uint32_t>(254 - se) << 23));
-        float xs[4] = {v[0] * s, v[1] * s, v[2] * s, v[3] * s};
-        _Float16 hi[4], lo[4];
-        float seen = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          if (e == 0xFFu) xs[c] = 0.0f;
-          hi[c] = static_cast<_Float16>(xs[c]);
-          lo[c] = static_cast<_Float16>(xs[c] - static_cast<float>(hi[c]));
-          seen += static_cast<float>(hi[c]) + static_cast<float>(lo[c]);
-        }
-        // the nibble masks deliver a chunk's elements in the order 0, 2, 1, 3 | 4, 6, 5, 7
-        typedef _Float16 half4v __attribute__((ext_vector_type(4)));
         const uint32_t cr = 2u * (r8 & 3);      // matrix rows 2 r8 and 2 r8 + 1, four activation rows at a time
-        *reinterpret_cast<half4v*>(conv + cr * kARowBytes + lane * 8u) = half4v{hi[0], hi[2], hi[1], hi[3]};
-        *reinterpret_cast<half4v*>(conv + (cr + 1u) * kARowBytes + lane * 8u) = half4v{lo[0], lo[2], lo[1], lo[3]};
-        // sub-block sums: eight consecutive lanes
-        seen = dpp_fadd16<0xB1>(seen);     // quad_perm [1,0,3,2]
-        seen = dpp_fadd16<0x4E>(seen);     // quad_perm [2,3,0,1]
-        seen = dpp_fadd16<0x141>(seen);    // row_half_mirror
-        if ((lane & 7u) == 0u) sx[((jb * MT + mt) * 8u + (lane >> 3)) * 8u + r8] = seen;
-        if (lane == 0u) invs[(jb * MT + mt) * 8u + r8] = inv;
+        typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        if (r >= p.m || !col_live(jb)) {
+          // a row the call does not have (the same for the whole wavefront): zero operands
+          const half4v z = {0, 0, 0, 0};
+          *reinterpret_cast<half4v*>(conv + cr * kARowBytes + lane * 8u) = z;
+          *reinterpret_cast<half4v*>(conv + (cr + 1u) * kARowBytes + lane * 8u) = z;
+          if ((lane & 7u) == 0u) sx[((jb * MT + mt) * 8u + (lane >> 3)) * 8u + r8] = 0.0f;
+          if (lane == 0u) invs[(jb * MT + mt) * 8u + r8] = 1.0f;
+        } else {
+          const float4_t v = xv[jb * MT + mt][r8];
+          const uint32_t e = mx[r8] >> 23;
+          int se = 262 - static_cast<int>(e);                       // amax * s in [2^8, 2^9)
+          se = se < 1 ? 1 : (se > 254 ? 254 : se);
+          const float s = (e == 0u || e == 0xFFu) ? 1.0f : bit_cast<float>(static_cast<uint32_t>(se) << 23);
+          // NaN or infinity anywhere in the block: the block's factor becomes NaN, as the reference's sum would
+          const float inv = e == 0xFFu ? bit_cast<float>(0x7FC00000u)
+                                       : (e == 0u ? 1.0f : bit_cast<float>(static_cast<uint32_t>(254 - se) << 23));
+          // the nibble masks deliver a chunk's elements in the order 0, 2, 1, 3 | 4, 6, 5, 7
+          float2v xa = {v[0] * s, v[2] * s}, xb = {v[1] * s, v[3] * s};
+          if (e == 0xFFu) xa = xb = float2v{0.0f, 0.0f};
+          const half2v ha = __builtin_convertvector(xa, half2v), hb = __builtin_convertvector(xb, half2v);
+          const half2v la = __builtin_convertvector(xa - __builtin_convertvector(ha, float2v), half2v);
+          const half2v lb = __builtin_convertvector(xb - __builtin_convertvector(hb, float2v), half2v);
+          *reinterpret_cast<half4v*>(conv + cr * kARowBytes + lane * 8u) = half4v{ha[0], ha[1], hb[0], hb[1]};
+          *reinterpret_cast<half4v*>(conv + (cr + 1u) * kARowBytes + lane * 8u) = half4v{la[0], la[1], lb[0], lb[1]};
+          // sub-block sums (eight consecutive lanes) of the scaled values: what the matrix core
+          // sees is these to 22 bits, and exactly these for a row of powers of two
+          float seen = (xa[0] + xa[1]) + (xb[0] + xb[1]);
+          seen = dpp_fadd16<0xB1>(seen);     // quad_perm [1,0,3,2]
+          seen = dpp_fadd16<0x4E>(seen);     // quad_perm [2,3,0,1]
+          seen = dpp_fadd16<0x141>(seen);    // row_half_mirror
+          if ((lane & 7u) == 0u) sx[((jb * MT + mt) * 8u + (lane >> 3)) * 8u + r8] = seen;
+          if (lane == 0u) invs[(jb * MT + mt) * 8u + r8] = inv;
+        }
         if ((r8 & 3) == 3) {
           // matrix row i = 2 r8 + {hi, lo} is lane % 16; K chunk gq of sub-block sb.  The lanes
           // of the eight rows just converted pick theirs up before the area is written again.
@@ -336,7 +378,7 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
 
   // ---- tiles.  Every wavefront walks the same tiles, so the barriers match.
   const size_t region = static_cast<size_t>(p.m) * p.n;
-  float* cpart = gridDim.y == 1 ? p.c : p.ws + blockIdx.y * region;
+  float* cpart = n_parts == 1u ? p.c : p.ws + part_index * region;
   // One tile: its BW units, then the wavefront's partial tile into LDS.  A unit is waited for when
   // RING - 1 later ones are all that may still be under way (stores of the sums count as well and
   // only make the wait longer); its slot is asked for again as soon as its words are in registers.
@@ -351,7 +393,7 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
       next_unit();
       read_slot = read_slot + 1u == RING ? 0u : read_slot + 1u;
     }
-    float* dst = part + ((ti * waves + wave) * (8u * MT)) * 16u;
+    float* dst = part + ((ti * live_waves + wave) * (8u * MT)) * 16u;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -359,27 +401,85 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
   };
   // The wavefronts run through a group of tiles on their own (no wavefront waits for another
   // while its ring is being refilled) and meet once a group: normally once a workgroup.
-  for (uint32_t g0 = 0; g0 < tiles; g0 += p.tiles_per_sync) {
-    const uint32_t in_group = tiles - g0 < p.tiles_per_sync ? tiles - g0 : p.tiles_per_sync;
+  for (uint32_t g0 = 0; g0 < tiles; g0 += tiles_per_sync) {
+    const uint32_t in_group = tiles - g0 < tiles_per_sync ? tiles - g0 : tiles_per_sync;
     for (uint32_t ti = 0; ti < in_group; ++ti) do_tile(ti);
     lds_barrier();
     // sum the wavefronts' partial tiles per output in wavefront order and store
-    for (uint32_t o = t; o < in_group * 8u * MT * 16u; o += blockDim.x) {
+    for (uint32_t o = t; o < in_group * 8u * MT * 16u; o += live_waves * 64u) {
       const uint32_t nn = o & 15u, r = (o >> 4) % (8u * MT), ti = o / (128u * MT);
       const uint32_t row = row0 + (g0 + ti) * kTile + nn;
       if (r >= p.m || row >= p.n) continue;
       float sum = 0.0f;
-      for (uint32_t wv = 0; wv < waves; ++wv) sum += part[((ti * waves + wv) * (8u * MT) + r) * 16u + nn];
+      for (uint32_t wv = 0; wv < live_waves; ++wv) sum += part[((ti * live_waves + wv) * (8u * MT) + r) * 16u + nn];
       cpart[static_cast<size_t>(r) * p.n + row] = sum;
     }
-    if (g0 + p.tiles_per_sync < tiles) lds_barrier();      // the table is written again
+    if (g0 + tiles_per_sync < tiles) lds_barrier();      // the table is written again
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive its workgroup
 }
 
 struct R16Plan {
   uint32_t parts, waves, bw, mt, tiles_per_wg, row_groups, ring, tiles_per_sync;
+  uint32_t n_table;              // unequal parts: entries of `table`, row_groups = all workgroups
+  R16Part table[kMaxParts];
 };
+
+constexpr uint32_t kR16Lds = 160u * 1024u - 64u;
+
+// Tiles between two meetings: as many as the LDS beside the rings holds, in equal groups.
+uint32_t r16_sync_tiles(uint32_t layout_waves, uint32_t live_waves, uint32_t mt, uint32_t bw, uint32_t ring, uint32_t per) {
+  const uint32_t tile_bytes = live_waves * 8u * mt * 16u * 4u;
+  uint32_t tps = (kR16Lds - r16_fixed_lds_bytes(layout_waves, mt, bw, ring)) / tile_bytes;
+  tps = tps > per ? per : tps;
+  const uint32_t syncs = (per + tps - 1u) / tps;
+  return (per + syncs - 1u) / syncs;
+}
+
+// Unequal K parts of twelve and eight block columns.  The launch lasts as long as the SIMD with the
+// most wavefronts works, and a wavefront's time goes to its instructions, not to waiting for
+// weights: ten columns a workgroup put three wavefronts on two SIMDs and two on the others.  Parts
+// of 12 and 8 columns fill the four SIMDs evenly (3 and 2 wavefronts each); a workgroup of an
+// 8-column part takes one and a half times the tiles, and the CUs are shared out accordingly
+// (`prologue` = the conversion of a wavefront's activations in units of one tile's work).  Measured
+// 17408 x 5120: 8 rows 20.0 -> 18.9 us, 5120 x 17408: 8 rows 23.6 -> 21.2, 16 rows 31.9 -> 27.9 us.
+bool r16_plan_unequal(uint32_t nb, uint32_t mt, uint32_t tiles_total, uint32_t cus, R16Plan& pl) {
+  if (nb % 4u != 0u || nb < 20u) return false;
+  uint32_t twelves = nb / 12u;
+  while ((nb - twelves * 12u) % 8u != 0u) --twelves;     // nb = 12 a + 8 b; a >= 1 for nb >= 20, nb % 4 == 0
+  const uint32_t eights = (nb - twelves * 12u) / 8u;
+  if (twelves == 0u || eights == 0u || twelves + eights > kMaxParts) return false;
+  const uint32_t prologue = 2;   // measured: 1..3 alike, 5 and more slower, for 8 and for 16 rows
+  uint32_t t12 = 0, t8 = 0;
+  for (uint32_t t = 1; t <= tiles_total; ++t) {
+    const uint32_t u = (3u * (prologue + t)) / 2u - prologue;
+    const uint32_t g12 = (tiles_total + t - 1u) / t, g8 = (tiles_total + u - 1u) / u;
+    if (twelves * g12 + eights * g8 <= cus) {
+      t12 = t, t8 = u;
+      break;
+    }
+  }
+  if (t12 == 0u) return false;
+  const uint32_t waves = 12, bw = 1;
+  uint32_t ring = 4;
+  while (ring > 2u && r16_lds_bytes(waves, mt, bw, ring, 1) > kR16Lds) --ring;
+  if (r16_lds_bytes(waves, mt, bw, ring, 1) > kR16Lds) return false;
+  pl = R16Plan{};
+  pl.parts = twelves + eights, pl.waves = waves, pl.bw = bw, pl.mt = mt, pl.ring = ring, pl.n_table = twelves + eights;
+  uint32_t wg = 0, b0 = 0, max_sync = 1;
+  for (uint32_t i = 0; i < pl.n_table; ++i) {
+    const uint32_t cols = i < twelves ? 12u : 8u, per = i < twelves ? t12 : t8;
+    const uint32_t tps = r16_sync_tiles(waves, cols, mt, bw, ring, per);
+    pl.table[i] = R16Part{wg, per, b0, cols, tps};
+    max_sync = tps * cols > max_sync ? tps * cols : max_sync;
+    wg += (tiles_total + per - 1u) / per;
+    b0 += cols;
+  }
+  pl.row_groups = wg;
+  pl.tiles_per_wg = t12;
+  pl.tiles_per_sync = (max_sync + waves - 1u) / waves;   // sizes the LDS table: tiles x wavefronts of the largest entry
+  return true;
+}
 
 // K parts: the fewest (a divisor of the block count) whose block columns fit the twelve wavefronts
 // of a workgroup, one column each, or two when 8 rows or fewer leave the registers for it --
@@ -390,6 +490,7 @@ bool r16_plan(uint64_t m, uint64_t n, uint64_t k, R16Plan& pl) {
   const uint32_t nb = static_cast<uint32_t>(k / 256), mt = m > 8 ? 2u : 1u, bw_max = mt == 1 ? 2u : 1u;
   const uint32_t tiles_total = static_cast<uint32_t>((n + kTile - 1) / kTile);
   const uint32_t cus = static_cast<uint32_t>(num_cus());
+  if (r16_plan_unequal(nb, mt, tiles_total, cus, pl)) return true;
   for (uint32_t parts = 1; parts <= nb; ++parts) {
     if (nb % parts != 0) continue;
     const uint32_t nbp = nb / parts;
@@ -407,16 +508,11 @@ bool r16_plan(uint64_t m, uint64_t n, uint64_t k, R16Plan& pl) {
     const uint32_t per = (tiles_total + groups - 1u) / groups;
     // the deepest ring of weight units that fits beside the conversion areas, then as many
     // tiles between two meetings as the rest holds (equal groups)
-    constexpr uint32_t kLds = 160u * 1024u - 64u;
     uint32_t ring = 4;
-    while (ring > 2u && r16_lds_bytes(waves, mt, bw, ring, 1) > kLds) --ring;
-    if (r16_lds_bytes(waves, mt, bw, ring, 1) > kLds) return false;
-    const uint32_t tile_bytes = waves * 8u * mt * 16u * 4u;
-    uint32_t tps = (kLds - r16_fixed_lds_bytes(waves, mt, bw, ring)) / tile_bytes;
-    tps = tps > per ? per : tps;
-    const uint32_t syncs = (per + tps - 1u) / tps;
-    tps = (per + syncs - 1u) / syncs;
-    pl = R16Plan{parts, waves, bw, mt, per, (tiles_total + per - 1u) / per, ring, tps};
+    while (ring > 2u && r16_lds_bytes(waves, mt, bw, ring, 1) > kR16Lds) --ring;
+    if (r16_lds_bytes(waves, mt, bw, ring, 1) > kR16Lds) return false;
+    const uint32_t tps = r16_sync_tiles(waves, waves, mt, bw, ring, per);
+    pl = R16Plan{parts, waves, bw, mt, per, (tiles_total + per - 1u) / per, ring, tps, 0, {}};
     return true;
   }
   return false;
@@ -471,8 +567,9 @@ hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* w
   R16Plan pl;
   if (!r16_plan(m, n, k, pl)) return hipErrorInvalidValue;
   R16Args args{a, w, c, static_cast<float*>(workspace), m, n, k, pl.tiles_per_wg, static_cast<uint32_t>(k / 256) / pl.parts,
-               pl.tiles_per_sync};
-  const dim3 grid(pl.row_groups, pl.parts), block(64 * pl.waves);
+               pl.tiles_per_sync, pl.n_table, {}};
+  for (uint32_t i = 0; i < pl.n_table; ++i) args.part[i] = pl.table[i];
+  const dim3 grid(pl.row_groups, pl.n_table != 0u ? 1u : pl.parts), block(64 * pl.waves);
   const uint32_t lds = r16_lds_bytes(pl.waves, pl.mt, pl.bw, pl.ring, pl.tiles_per_sync);
   r16_with_kernel(pl.mt, pl.bw, pl.ring, [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, lds, stream, args); });
   const hipError_t e = hipGetLastError();

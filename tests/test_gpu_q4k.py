@@ -231,7 +231,7 @@ def test_rows_kernels(backend, rows):
 # cover k/256 divisible by 4, by 2 only and odd (the tilings), k/256 not a multiple of 8 (ragged
 # stages), n not a multiple of 4, and every pass count.
 FEW_ROW_SHAPES = [(4096, 4096), (2060, 8192), (1030, 17408), (8200, 2048), (7400, 2304), (11000, 1536), (8194, 2048),
-                  (65540, 256), (65538, 256), (16388, 1024)]
+                  (65540, 256), (65538, 256), (16388, 1024), (3300, 5120), (1180, 14336)]
 
 
 @pytest.mark.parametrize("n,k", FEW_ROW_SHAPES)

@@ -472,23 +472,29 @@ __global__ __launch_bounds__(64 * kSkinnyWaves, 4) void mxfp4_a8_skinny_kernel(
 // Same arithmetic as the kernel above, fed differently: each direct load moves 256 contiguous
 // bytes of a weight row (four rows per instruction) into a three-stage swizzled LDS ring, so
 // HBM sees long row-contiguous runs instead of 64-byte pieces of sixteen rows, and the
-// fragment reads do the row/K transposition for free.  A workgroup of eight wavefronts owns 64
-// weight rows; per stage (512 of K) the 4 K-steps x 4 column tiles are split two to a wavefront
-// and the two wavefronts of a tile are summed through LDS at the end.
+// fragment reads do the row/K transposition for free.  A workgroup owns `rows_wg` weight rows (a
+// multiple of 4, at most 80: the rows of the matrix shared out evenly over the CUs, because the
+// bytes a CU's direct loads move set the pace -- 17408 rows as 272 groups of 64 took half as long
+// again as 16384 rows as 256) and has two wavefronts per 16-row column tile; per stage (512 of
+// K) the 4 K-steps of a tile are split two to a wavefront and the two wavefronts of a tile are
+// summed through LDS at the end.  Activation rows the call does not have are not loaded (their
+// rows of the product are never stored).
+constexpr uint32_t kStreamMaxRows = 80;
+
 template <int MT>
-__global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void mxfp4_a8_stream_kernel(
+__global__ __launch_bounds__(640) void mxfp4_a8_stream_kernel(
     const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
-    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k) {
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t rows_wg) {
   typedef float float4v __attribute__((ext_vector_type(4)));
-  constexpr uint32_t kBBytes = 64 * 256, kABytes = MT * 16 * 512, kSBytes = 64 * 16;
+  constexpr uint32_t kBBytes = kStreamMaxRows * 256, kABytes = MT * 16 * 512, kSBytes = kStreamMaxRows * 16;
   constexpr uint32_t kABase = kBBytes, kSBase = kABase + kABytes, kStage = kSBase + kSBytes;
-  constexpr int kDma = 2 + MT + 1;                      // direct loads a wavefront issues per stage
   __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kStage];
 
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t tiles = (rows_wg + 15u) / 16u;           // blockDim.x = 128 * tiles
   const uint32_t l16 = lane & 15u, kq = lane >> 4;
-  const uint32_t n0 = blockIdx.x * 64u;
+  const uint32_t n0 = blockIdx.x * rows_wg;
   const uint32_t row_bytes = k / 2, row_blocks = k / 32;
   const uint8_t* w_tile = w + static_cast<size_t>(n0) * row_bytes;
   const uint8_t* s_tile = w + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(n0) * row_blocks;
@@ -499,38 +505,70 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void mxfp4_a8_stream_kernel(
   // each: lane p fetches row 4L + p/16, chunk (p%16) ^ (row%16).  Activation block L = rows
   // 2L, 2L+1, thirty-two chunks each: row 2L + p/32, chunk (p%32) ^ (row%16).  Scale words: lane
   // p < 8 of wavefront v fetches the sixteen E8M0 bytes of row 8v + p.  Rows past the matrix
-  // edge are clamped (never stored).
-  uint32_t b_src[2], a_src[MT], s_src;
+  // edge are clamped (never stored); blocks past the workgroup's rows or the call's activation
+  // rows are not requested, so the loads a wavefront has in flight per stage differ: `my_dma`.
+  constexpr int kAMax = 4 * MT;        // activation blocks a wavefront brings at most (two wavefronts: 8 MT blocks)
+  const uint32_t waves = 2u * tiles;
+  uint32_t b_src[2], a_src[kAMax], s_src;
+  bool b_live[2], a_live[kAMax];
+  uint32_t my_dma = 0;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const uint32_t row = 4u * (wave * 2u + i) + lane / 16u;
     const uint32_t chunk = (lane % 16u) ^ (row % 16u);
     b_src[i] = (n0 + row < n ? row : n - 1u - n0) * row_bytes + chunk * 16u;
+    b_live[i] = 4u * (wave * 2u + i) < rows_wg;
+    my_dma += b_live[i] ? 1u : 0u;
   }
 #pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const uint32_t row = 2u * (wave * MT + i) + lane / 32u;
+  for (int i = 0; i < kAMax; ++i) {
+    const uint32_t blk = wave + i * waves;               // blocks go round the wavefronts
+    const uint32_t row = 2u * blk + lane / 32u;
     const uint32_t chunk = (lane % 32u) ^ (row % 16u);
     a_src[i] = (row < m ? row : m - 1u) * k + chunk * 16u;
+    a_live[i] = blk < 8u * MT && 2u * blk < m;
+    my_dma += a_live[i] ? 1u : 0u;
   }
+  const bool s_live = 8u * wave < rows_wg;
   {
     const uint32_t row = 8u * wave + (lane & 7u);
     s_src = (n0 + row < n ? row : n - 1u - n0) * row_blocks;
+    my_dma += s_live ? 1u : 0u;
   }
   auto issue_stage = [&](uint32_t stage_off, uint32_t st) {
     const uint32_t stage = lds_base + stage_off;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) direct_load16(w_tile + st * 256u, b_src[i], stage + (wave * 2u + i) * 1024u);
+    for (int i = 0; i < 2; ++i) {
+      if (b_live[i]) direct_load16(w_tile + st * 256u, b_src[i], stage + (wave * 2u + i) * 1024u);
+    }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) direct_load16(a8 + st * 512u, a_src[i], stage + kABase + (wave * MT + i) * 1024u);
-    if (lane < 8u) direct_load16(s_tile + st * 16u, s_src, stage + kSBase + wave * 128u);
+    for (int i = 0; i < kAMax; ++i) {
+      if (a_live[i]) direct_load16(a8 + st * 512u, a_src[i], stage + kABase + (wave + i * waves) * 1024u);
+    }
+    if (s_live && lane < 8u) direct_load16(s_tile + st * 16u, s_src, stage + kSBase + wave * 128u);
   };
+  // Everything but the stage requested last has landed, for every wavefront.
   auto publish = [&]() {
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kDma) : "memory");
+    switch (my_dma) {
+      case 0: asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory"); break;
+      case 7: asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory"); break;
+      case 8: asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory"); break;
+      case 9: asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory"); break;
+      case 10: asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(11) lgkmcnt(0)" ::: "memory"); break;
+    }
+    asm volatile("s_barrier" ::: "memory");
   };
+  static_assert(2 + kAMax + 1 <= 11, "publish() counts up to eleven loads a stage");
 
   // This wavefront's share of a stage: column tile `tile`, K-steps 2*half and 2*half + 1.
-  const uint32_t tile = wave & 3u, half = wave >> 2;
+  const uint32_t tile = wave % tiles, half = wave / tiles;
   const uint32_t b_row = tile * 16u + l16;
   float4v acc[MT];
 #pragma unroll
@@ -578,15 +616,27 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void mxfp4_a8_stream_kernel(
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) red[(((half * 4u + tile) * MT + i) * 4u + e) * 64u + lane] = acc[i][e];
+    for (int e = 0; e < 4; ++e) red[(((half * tiles + tile) * MT + i) * 4u + e) * 64u + lane] = acc[i][e];
   __syncthreads();
-  for (uint32_t o = t; o < m * 64u; o += 512u) {
-    const uint32_t row = o / 64u, col = o % 64u;
+  const uint32_t cols = tiles * 16u;
+  for (uint32_t o = t; o < m * cols; o += blockDim.x) {
+    const uint32_t row = o / cols, col = o % cols;
     const uint32_t i = row / 16u, r = row % 16u, ln = (r / 4u) * 16u + col % 16u, tl = col / 16u;
-    const float sum = red[(((0u * 4u + tl) * MT + i) * 4u + r % 4u) * 64u + ln] +
-                      red[(((1u * 4u + tl) * MT + i) * 4u + r % 4u) * 64u + ln];
-    if (n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row];
+    const float sum = red[(((0u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln] +
+                      red[(((1u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln];
+    if (col < rows_wg && n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row];
   }
+}
+
+// Rows a workgroup of the streamed kernel owns: the matrix shared out evenly over the CUs, as few
+// rounds of workgroups as 80 rows each allow, in multiples of the four rows a direct load moves.
+uint32_t stream_rows_per_workgroup(uint32_t n) {
+  const uint32_t cus = static_cast<uint32_t>(num_cus());
+  const uint32_t rounds = (n + kStreamMaxRows * cus - 1u) / (kStreamMaxRows * cus);
+  const uint32_t share = (n + cus * rounds - 1u) / (cus * rounds);
+  uint32_t rows = (share + 3u) / 4u * 4u;
+  rows = rows < 16u ? 16u : (rows > kStreamMaxRows ? kStreamMaxRows : rows);
+  return rows;
 }
 
 
@@ -736,11 +786,12 @@ void launch_tiles(const uint8_t* a8, const float* as, const uint8_t* w, float* c
 hipError_t launch_mxfp4_a8_gemm(const uint8_t* a8, const float* as, const uint8_t* w, float* c,
                                 uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
   if (m <= 32 && k % 512 == 0) {
-    const dim3 grid((n + 63u) / 64u), block(512);
+    const uint32_t rows = stream_rows_per_workgroup(n);
+    const dim3 grid((n + rows - 1u) / rows), block(128u * ((rows + 15u) / 16u));
     if (m <= 16) {
-      hipLaunchKernelGGL(mxfp4_a8_stream_kernel<1>, grid, block, 0, stream, a8, as, w, c, m, n, k);
+      hipLaunchKernelGGL(mxfp4_a8_stream_kernel<1>, grid, block, 0, stream, a8, as, w, c, m, n, k, rows);
     } else {
-      hipLaunchKernelGGL(mxfp4_a8_stream_kernel<2>, grid, block, 0, stream, a8, as, w, c, m, n, k);
+      hipLaunchKernelGGL(mxfp4_a8_stream_kernel<2>, grid, block, 0, stream, a8, as, w, c, m, n, k, rows);
     }
     return hipGetLastError();
   }

@@ -29,7 +29,10 @@ def w4a8(backend, x, w, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(5, 64, 256), (16, 128, 512), (33, 100, 768), (128, 128, 256),
-                                   (130, 257, 1024), (64, 192, 5120), (300, 50, 2048)])
+                                   (130, 257, 1024), (64, 192, 5120), (300, 50, 2048),
+                                   # more rows than 64 a CU: the few-row kernel shares them out evenly
+                                   # (68, 72, 80 rows a workgroup, ragged last workgroup, a second round)
+                                   (5, 16500, 512), (20, 17001, 512), (16, 19999, 1024), (3, 20500, 512), (32, 18433, 512)])
 def test_gemm_matches_oracle(backend, m, n, k):
     g = synth.rng(m * 7 + n * 3 + k)
     w = synth.mxfp4_weights(g, n, k, -8, -4)

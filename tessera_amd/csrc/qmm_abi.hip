@@ -820,6 +820,9 @@ qmm_status run_gemm_mxfp4_wmma(const LaunchCtx& c) {
   }
   // Regime: a single row stays on the VALU GEMV; from two rows on the scaled MFMA takes over
   // (a streaming kernel up to 32 rows, the tiled GEMM above that).
+  // (The streaming kernel would be faster for one row of a wide matrix as well -- 17408 x 5120:
+  // 11.1 against 12.4 us -- but its sums do not meet the single row's tolerance against the
+  // fp32 reference, so one row keeps the fp32 multiply-adds.)
   if (m > 1 && k >= 1024 && qmm::gemm_mxfp4_a8_supported(k)) {
     qmm_status st = map_hip(qmm::launch_mxfp4_a8_gemm(
         c.ptr<const uint8_t>(0), c.ptr<const float>(2), w, out,

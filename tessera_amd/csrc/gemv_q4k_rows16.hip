@@ -451,7 +451,7 @@ bool r16_plan_unequal(uint32_t nb, uint32_t mt, uint32_t tiles_total, uint32_t c
   if (twelves == 0u || eights == 0u || twelves + eights > kMaxParts) return false;
   const uint32_t prologue = 2;   // measured: 1..3 alike, 5 and more slower, for 8 and for 16 rows
   uint32_t t12 = 0, t8 = 0;
-  for (uint32_t t = 1; t <= tiles_total; ++t) {
+  for (uint32_t t = tiles_total / cus > 1u ? tiles_total / cus : 1u; t <= tiles_total; ++t) {   // a part alone needs tiles / t <= CUs
     const uint32_t u = (3u * (prologue + t)) / 2u - prologue;
     const uint32_t g12 = (tiles_total + t - 1u) / t, g8 = (tiles_total + u - 1u) / u;
     if (twelves * g12 + eights * g8 <= cus) {
@@ -466,10 +466,16 @@ bool r16_plan_unequal(uint32_t nb, uint32_t mt, uint32_t tiles_total, uint32_t c
   if (r16_lds_bytes(waves, mt, bw, ring, 1) > kR16Lds) return false;
   pl = R16Plan{};
   pl.parts = twelves + eights, pl.waves = waves, pl.bw = bw, pl.mt = mt, pl.ring = ring, pl.n_table = twelves + eights;
+  // partial tiles (one wavefront's share of a tile) the LDS table holds, a whole number of
+  // twelve-wavefront tiles: the launch sizes the table as tiles x 12 wavefronts
+  const uint32_t table_units = (kR16Lds - r16_fixed_lds_bytes(waves, mt, bw, ring)) / (8u * mt * 16u * 4u) / waves * waves;
   uint32_t wg = 0, b0 = 0, max_sync = 1;
   for (uint32_t i = 0; i < pl.n_table; ++i) {
     const uint32_t cols = i < twelves ? 12u : 8u, per = i < twelves ? t12 : t8;
-    const uint32_t tps = r16_sync_tiles(waves, cols, mt, bw, ring, per);
+    uint32_t tps = table_units / cols;
+    tps = tps > per ? per : tps;
+    const uint32_t syncs = (per + tps - 1u) / tps;
+    tps = (per + syncs - 1u) / syncs;
     pl.table[i] = R16Part{wg, per, b0, cols, tps};
     max_sync = tps * cols > max_sync ? tps * cols : max_sync;
     wg += (tiles_total + per - 1u) / per;

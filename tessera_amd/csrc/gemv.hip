@@ -1274,9 +1274,10 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
       // the weights of two stages under way meanwhile.  A barrier that waits for nothing makes
       // sure every wavefront's activation requests are out before any weights, so that no
       // wavefront's activations queue behind the others' weights: 5120 x 17408 15.5 -> 13.8 us.
-      // Short rows measured slower that way (Q6_K 17408 x 5120: 19.0 -> 21.3 us) and keep one stage.
+      // Short rows measured slower with two stages early (Q6_K 17408 x 5120: 19.0 -> 21.3 us) and
+      // keep one stage, but take the barrier too (17408 x 5120: 12.23 -> 11.88 us).
       constexpr bool kTwoStagesEarly = kXPer == 8 && D > 1;
-      if constexpr (kTwoStagesEarly) {
+      {
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_barrier");
         __builtin_amdgcn_sched_barrier(0);

@@ -177,7 +177,9 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
     return QMM_OK;
   }
   // 3..16 rows of a large matrix: one pass over the weights on the 16x16x32 MFMA.
-  if (m >= kQ4KRows16MinRows && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemv_q4k_rows16_supported(m, n, k) &&
+  // (two rows as well when the weight rows are long: 5120 x 17408 20.5 against 24.8 us on the
+  // resident kernel, 4096 x 14336 15.3 against 18.5; at 8192 and below the resident kernel leads)
+  if ((m >= kQ4KRows16MinRows || (m == 2 && k > 8192)) && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemv_q4k_rows16_supported(m, n, k) &&
       qmm::gemv_q4k_rows16_workspace_bytes(m, n, k) <= kDecodeScratchBytes) {
     void* ws = decode_scratch(ctx);
     if (ws == nullptr) {

@@ -168,7 +168,7 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
     return map_hip(qmm::launch_q4k_gemm(a, w, c, ws, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                         static_cast<uint32_t>(k), s));
   }
-  if (m > 16 && n * k >= kQ4KFewRowsMinWeights) {
+  if (m > 16 && (n * k >= kQ4KFewRowsMinWeights || qmm::gemv_q4k_rows16_supported(16, n, k))) {
     // exact, sixteen rows at a time (each chunk takes the regime of its own row count)
     for (uint64_t r = 0; r < m; r += 16) {
       const qmm_status st = q4k_matmul(ctx, a + r * k, w, c + r * n, m - r < 16 ? m - r : 16, n, k, f16_from);
@@ -179,7 +179,10 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
   // 3..16 rows of a large matrix: one pass over the weights on the 16x16x32 MFMA.
   // (two rows as well when the weight rows are long: 5120 x 17408 20.5 against 24.8 us on the
   // resident kernel, 4096 x 14336 15.3 against 18.5; at 8192 and below the resident kernel leads)
-  if ((m >= kQ4KRows16MinRows || (m == 2 && k > 8192)) && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemv_q4k_rows16_supported(m, n, k) &&
+  // From five rows on it leads at any size (1024 x 1024, 8 rows: 5.1 against 14.5 us on the
+  // multiply-add passes; four rows are level with them below 16 M weights).
+  if ((m >= kQ4KRows16MinRows || (m == 2 && k > 8192)) && m <= 16 && (n * k >= kQ4KFewRowsMinWeights || m >= 5) &&
+      qmm::gemv_q4k_rows16_supported(m, n, k) &&
       qmm::gemv_q4k_rows16_workspace_bytes(m, n, k) <= kDecodeScratchBytes) {
     void* ws = decode_scratch(ctx);
     if (ws == nullptr) {

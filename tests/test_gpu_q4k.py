@@ -248,6 +248,21 @@ def test_few_rows_match_oracle(backend, n, k, m):
     assert rms_err(got, ref) <= 1e-4, rms_err(got, ref)     # the split activations keep 22 bits
 
 
+# Five rows and more take the one-pass kernel whatever the matrix size (two K parts of unequal
+# size at k = 5120, a single wavefront's column at k = 256, ragged last tiles), 17..63 rows sixteen
+# at a time with a short last chunk.
+@pytest.mark.parametrize("n,k", [(100, 1024), (1030, 2304), (515, 5120), (64, 17408), (3001, 256)])
+@pytest.mark.parametrize("m", [5, 9, 16, 17, 21, 33])
+def test_five_rows_and_more_on_small_matrices(backend, n, k, m):
+    g = synth.rng(91 * m + n + k)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
+    got = gemm(backend, "gemm_q4k_batched", a, w, m, n, k)[0]
+    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    assert rms_err(got, ref) <= 1e-4, rms_err(got, ref)
+
+
 def test_few_rows_scaling_and_exactness(backend):
     n, k = 4096, 4096
     g = synth.rng(31337)

@@ -174,6 +174,23 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     out["q4k_few_rows_17408x5120"] = few
     del wq_list
 
+    # ---- the same ids on the down-projection shape and on a small matrix (from five rows on every
+    # size takes the one-pass MFMA kernel; the copies rotate, the small ones stay in the caches) ----
+    for (ns, ks), label in (((K_HID, N_FF), "q4k_few_rows_5120x17408"), ((4096, 2048), "q4k_few_rows_small_4096x2048")):
+        w_s = to_dev(synth.q4k_weights(g, ns, ks))
+        ws_list = [w_s] + [w_s.clone() for _ in range(copies - 1)]
+        small = {}
+        for m in (2, 8, 16, 32):
+            x = to_dev(synth.activations_f32(g, m, ks))
+            y = torch.empty(m * ns, dtype=torch.float32, device=dev)
+            launches = [(kb, KernelLaunch(grid_x=(m * ns + 7) // 8, buffers=[wrap(x), wrap(w), wrap(y)], scalars=[m, ns, ks]))
+                        for w in ws_list]
+            us = timed_us(launches, 10) / copies
+            nbytes = ns * (ks // 256) * 144 + 4 * m * ks + 4 * m * ns
+            small[f"m{m}"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}
+        out[label] = small
+        del ws_list
+
     # ---- gate and up stored as one 34816 x 5120 tensor (a loader may concatenate them): the same
     # id and kernel, one launch instead of two, so the fixed cost of a launch is paid once ----------
     w_gu = torch.cat([w_q1, w_q1.clone()])

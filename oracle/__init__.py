@@ -71,6 +71,7 @@ def _load() -> C.CDLL:
         "orc_attention_split": (C.c_int, [f32p, f32p, f32p, f32p, f32p, f32p, sz, sz, sz, sz, sz, C.c_uint64, sz, C.c_int, sz]),
         "orc_attention_combine": (C.c_int, [f32p, f32p, f32p, f32p, sz, sz, sz, sz]),
         "orc_permute_mxfp4_to_wmma": (C.c_int, [u8p, u8p, sz, sz]),
+        "orc_permute_q4k_rowgroup": (C.c_int, [u8p, u8p, sz, sz, sz, C.c_int]),
         "orc_rope": (C.c_int, [f32p, sz, sz, sz, sz, C.c_uint64, C.c_double]),
         "orc_mrope": (C.c_int, [f32p, C.POINTER(C.c_uint64), sz, sz, sz, sz, sz, sz, sz, C.c_double]),
         "orc_attention": (C.c_int, [f32p, C.c_void_p, C.c_void_p, f32p, sz, sz, sz, sz, sz, C.c_uint64, sz, C.c_int, C.c_int]),
@@ -324,6 +325,15 @@ def permute_mxfp4_to_wmma(packed, n: int, k: int) -> np.ndarray:
     out = np.empty_like(blob)
     _check(_lib.orc_permute_mxfp4_to_wmma(_p(blob, C.c_uint8), _p(out, C.c_uint8), n, k))
     return np.concatenate([out.reshape(-1), s.reshape(-1)])
+
+
+def permute_q4k_rowgroup(w, n: int, k: int, rows_per_group: int = 32, inverse: bool = False) -> np.ndarray:
+    """A Q4_K matrix between GGUF order and the row-group order of the gfx950 int8 decode kernel
+    (same byte count; `inverse` goes back)."""
+    w = _u8(w)
+    out = np.empty_like(w)
+    _check(_lib.orc_permute_q4k_rowgroup(_p(w, C.c_uint8), _p(out, C.c_uint8), n, k, rows_per_group, int(inverse)))
+    return out
 
 
 def fold_mxfp4_to_fp8(packed, n: int, k: int) -> tuple[np.ndarray, np.ndarray]:

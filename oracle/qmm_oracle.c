@@ -688,6 +688,87 @@ int orc_permute_mxfp4_to_wmma(const uint8_t* packed, uint8_t* out, size_t rows, 
   return ORC_OK;
 }
 
+/* ---- Q4_K row groups: the load-time copy that the gfx950 int8 matrix kernel reads.  No counterpart
+ *      in the reference (its own load-time hook is PermuteMxFp4ToWmma above); this is the layout's
+ *      definition, element by element, for checking the device's permutation against:
+ *      rows [g*R, g*R+rows) of group g keep, per 256-wide block b, rows*144 bytes at
+ *      (g*R*nblk + b*rows)*144: first the tiles' quants, then the rows' 16-byte headers.
+ *      Tile t (rows 16t..16t+rt-1 of the group) has two pieces c = 0,1 of rt*64 bytes at
+ *      t*2048 + c*rt*64; row nn of the tile, lane group q = 0..3, owns the 16 bytes at (q*rt + nn)*16
+ *      of a piece; byte P of them holds in its low nibble weight 16*(q%2)+P of sub-block 2c + q/2 and
+ *      in its high nibble the same weight of sub-block 2c + 4 + q/2 minus 8 (mod 16).
+ *      Header: d, dmin as in GGUF; then byte i of the next three words = sc[2i] | (mn[2i+1] & 3) << 6,
+ *      sc[2i+1] | (mn[2i+1] >> 2 & 3) << 6, mn[2i] | (mn[2i+1] >> 4) << 6 (sc, mn from GetScaleMin). ---- */
+static uint32_t orc_q4k_nibble(const uint8_t* block, int sub, int l) {
+  const uint8_t byte = block[16 + (sub / 2) * 32 + l];
+  return (sub & 1) ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 15);
+}
+int orc_permute_q4k_rowgroup(const uint8_t* in, uint8_t* out, size_t n, size_t k, size_t R, int inverse) {
+  if (n == 0 || k == 0 || k % 256 != 0 || R == 0 || R > 64) return ORC_INVALID_ARGUMENT;
+  const size_t nblk = k / 256;
+  for (size_t r = 0; r < n; ++r) {
+    const size_t row0 = r / R * R, rows = n - row0 < R ? n - row0 : R, rr = r - row0;
+    const size_t tile = rr / 16, nn = rr % 16, rt = rows - tile * 16 < 16 ? rows - tile * 16 : 16;
+    for (size_t b = 0; b < nblk; ++b) {
+      const size_t gguf = (r * nblk + b) * 144, region = (row0 * nblk + b * rows) * 144;
+      const size_t hdr = region + rows * 128 + rr * 16;
+      if (!inverse) {
+        const uint8_t* blk = in + gguf;
+        uint8_t sc[8], mn[8];
+        for (int j = 0; j < 8; ++j) orc_get_scale_min(j, blk + 4, &sc[j], &mn[j]);
+        memcpy(out + hdr, blk, 4);
+        for (int i = 0; i < 4; ++i) {
+          const uint8_t mo = mn[2 * i + 1];
+          out[hdr + 4 + i] = (uint8_t)(sc[2 * i] | ((mo & 3) << 6));
+          out[hdr + 8 + i] = (uint8_t)(sc[2 * i + 1] | (((mo >> 2) & 3) << 6));
+          out[hdr + 12 + i] = (uint8_t)(mn[2 * i] | (((mo >> 4) & 3) << 6));
+        }
+        for (int c = 0; c < 2; ++c) {
+          for (int q = 0; q < 4; ++q) {
+            uint8_t* piece = out + region + tile * 2048 + (size_t)c * rt * 64 + ((size_t)q * rt + nn) * 16;
+            for (int P = 0; P < 16; ++P) {
+              const int l = 16 * (q % 2) + P;
+              const uint32_t lo = orc_q4k_nibble(blk, 2 * c + q / 2, l);
+              const uint32_t hi = (orc_q4k_nibble(blk, 2 * c + 4 + q / 2, l) + 8u) & 15u;   /* minus 8 mod 16 */
+              piece[P] = (uint8_t)(lo | (hi << 4));
+            }
+          }
+        }
+      } else {
+        const uint8_t* h = in + hdr;
+        uint8_t* blk = out + gguf;
+        uint8_t sc[8], mn[8];
+        for (int i = 0; i < 4; ++i) {
+          sc[2 * i] = h[4 + i] & 63;
+          sc[2 * i + 1] = h[8 + i] & 63;
+          mn[2 * i] = h[12 + i] & 63;
+          mn[2 * i + 1] = (uint8_t)((h[4 + i] >> 6) | ((h[8 + i] >> 6) << 2) | ((h[12 + i] >> 6) << 4));
+        }
+        memcpy(blk, h, 4);
+        /* the reference's packing of the twelve scale bytes (quant.cpp:712-720) */
+        for (int j = 0; j < 4; ++j) {
+          blk[4 + j] = (uint8_t)(sc[j] | ((sc[j + 4] >> 4) << 6));
+          blk[8 + j] = (uint8_t)(mn[j] | ((mn[j + 4] >> 4) << 6));
+          blk[12 + j] = (uint8_t)((sc[j + 4] & 15) | ((mn[j + 4] & 15) << 4));
+        }
+        memset(blk + 16, 0, 128);
+        for (int c = 0; c < 2; ++c) {
+          for (int q = 0; q < 4; ++q) {
+            const uint8_t* piece = in + region + tile * 2048 + (size_t)c * rt * 64 + ((size_t)q * rt + nn) * 16;
+            for (int P = 0; P < 16; ++P) {
+              const int l = 16 * (q % 2) + P, shift = (q / 2) * 4;
+              const uint32_t lo = piece[P] & 15u, hi = ((uint32_t)(piece[P] >> 4) + 8u) & 15u;
+              blk[16 + c * 32 + l] |= (uint8_t)(lo << shift);          /* sub-block 2c + q/2 */
+              blk[16 + (c + 2) * 32 + l] |= (uint8_t)(hi << shift);    /* sub-block 2c + 4 + q/2 */
+            }
+          }
+        }
+      }
+    }
+  }
+  return ORC_OK;
+}
+
 /* ---- folded W4A8 GEMM: (sum fma(a8, w8)) * As[m] * 2^(wref-127)
  *      (quant.cpp:900-924) ---- */
 int orc_gemm_mxfp4_fp8_ref(const uint8_t* a8, const float* as, const uint8_t* w8,

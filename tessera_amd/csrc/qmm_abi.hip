@@ -11,6 +11,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "qmm_kernels.hpp"
 
@@ -73,11 +74,13 @@ u128 mxfp4_bytes(uint64_t n, uint64_t k) { return static_cast<u128>(n) * k / 2 +
 // same buffers and m, n, k scalars, so each id accepts every m and picks the gfx950
 // kernel that fits it.
 // Device scratch owned by the library (the fp16 copy of the activations that the Q4_K MFMA
-// GEMM reads).  Grown on demand and kept until the process ends; growing synchronises the
-// device (hipFree), so the first large prefill call must not sit inside a stream capture.
-// Launches that use it are ordered by the caller's stream, as everything else here.
+// GEMM reads).  Grown on demand; a block that has been handed to a launch is never freed before
+// the process ends (a recorded graph or another thread's launch may still point at it), so growth
+// retires the old block instead.  Growing allocates, which a stream under capture cannot do: such
+// a launch is refused.  Launches that use the block are ordered by the caller's stream.
 void* g_workspace = nullptr;
 size_t g_workspace_bytes = 0;
+std::vector<void*> g_retired_workspaces;
 // A workspace the caller owns (qmm_set_workspace): while one is set the library neither grows nor
 // frees anything in qmm_launch; a launch that needs more than it holds is refused.
 void* g_user_workspace = nullptr;
@@ -120,15 +123,25 @@ qmm_status workspace(const LaunchCtx& c, size_t bytes, void** out) {
     return QMM_OK;
   }
   if (bytes > g_workspace_bytes) {
-    if (g_workspace != nullptr) (void)hipFree(g_workspace);
-    g_workspace = nullptr;
-    g_workspace_bytes = 0;
-    const size_t want = (bytes + (size_t{1} << 24) - 1) & ~((size_t{1} << 24) - 1);
-    const hipError_t e = hipMalloc(&g_workspace, want);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(c.stream, &capturing) != hipSuccess) (void)hipGetLastError();
+    if (capturing != hipStreamCaptureStatusNone) {
+      g_last_error = "qmm_launch: this launch needs " + std::to_string(bytes) + " bytes of workspace and the library's holds " +
+                     std::to_string(g_workspace_bytes) + "; it cannot grow while the stream is being captured (hand one over "
+                     "with qmm_set_workspace, or make one eager call of this size first)";
+      return QMM_INVALID_ARGUMENT;
+    }
+    // at least double, so that the retired blocks together stay below the live one
+    size_t want = (bytes + (size_t{1} << 24) - 1) & ~((size_t{1} << 24) - 1);
+    if (want < 2 * g_workspace_bytes) want = 2 * g_workspace_bytes;
+    void* fresh = nullptr;
+    const hipError_t e = hipMalloc(&fresh, want);
     if (e != hipSuccess) {
       (void)hipGetLastError();
       return map_hip(e);
     }
+    if (g_workspace != nullptr) g_retired_workspaces.push_back(g_workspace);
+    g_workspace = fresh;
     g_workspace_bytes = want;
   }
   *out = g_workspace;
@@ -215,32 +228,62 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
   return q4k_matmul(ctx, a, w, c, m, n, k, g_q4k_tensor_rows.load(std::memory_order_relaxed));
 }
 
+// Weights handed over as the load-time row-group copy (`layout` = its rows per group; 0 = GGUF order):
+// one activation row runs on the int8 matrix kernel that the copy was made for; every other regime
+// gets the GGUF order back in the workspace first (behind what that regime itself keeps there) and
+// then runs as usual -- correct for every id, at the price of one more pass over the weights.
+bool q4k_layout_ok(uint64_t n, uint64_t k, uint64_t layout) {
+  return layout == 0 || qmm::q4k_rowgroup_supported(n, k, layout);
+}
+size_t q4k_regime_workspace(uint64_t m, uint64_t k, uint64_t f16_from) {
+  return m >= f16_from && qmm::gemm_q4k_supported(m, k) ? (qmm::gemm_q4k_workspace_bytes(m, k) + 255) & ~size_t{255} : 0;
+}
+qmm_status q4k_matmul_layout(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
+                             uint64_t k, uint64_t f16_from, uint64_t layout) {
+  if (layout == 0) return q4k_matmul(ctx, a, w, c, m, n, k, f16_from);
+  if (m == 1) {
+    return map_hip(qmm::launch_q4k_i8_gemv(a, w, c, static_cast<uint32_t>(n), static_cast<uint32_t>(k),
+                                           static_cast<uint32_t>(layout), ctx.stream));
+  }
+  const size_t front = q4k_regime_workspace(m, k, f16_from);
+  void* ws = nullptr;
+  qmm_status st = workspace(ctx, front + static_cast<size_t>(q4k_bytes(n, k)), &ws);
+  if (st != QMM_OK) return st;
+  uint8_t* gguf = static_cast<uint8_t*>(ws) + front;
+  st = map_hip(qmm::launch_q4k_rowgroup(w, gguf, static_cast<uint32_t>(n), static_cast<uint32_t>(k),
+                                        static_cast<uint32_t>(layout), true, ctx.stream));
+  if (st != QMM_OK) return st;
+  return q4k_matmul(ctx, a, gguf, c, m, n, k, f16_from);
+}
+
 // "gemm_q4k", "gemm_q4k_row", "gemm_q4k_batched", "gemm_q4k_wmma": buffers A, W, C;
 // scalars m, n, k (include/tessera/backend.hpp:153-161,207-209,397-415;
-// src/core/decode_internal.hpp:1484-1504).
+// src/core/decode_internal.hpp:1484-1504), optionally followed by `layout` (see q4k_matmul_layout).
 qmm_status run_gemm_q4k_id(const LaunchCtx& c, bool wmma) {
-  if (!counts(c, 3, 3)) return bad("gemm_q4k: expects 3 buffers and 3 scalars");
-  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2];
+  if (!counts(c, 3, 3) && !counts(c, 3, 4)) return bad("gemm_q4k: expects 3 buffers and 3 scalars (a fourth: layout)");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], layout = c.nsc > 3 ? c.sc[3] : 0;
   if (!dims_ok(m, n, k) || k % 256 != 0) return bad("gemm_q4k: m, n, k must be non-zero and k a multiple of 256");
+  if (!q4k_layout_ok(n, k, layout)) return bad("gemm_q4k: layout is 0 (GGUF order) or the rows per group of a row-group copy (1..64)");
   if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, q4k_bytes(n, k)) ||
       !c.fits(2, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_q4k: a buffer is smaller than m, n, k require");
   }
-  return q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k,
-                    wmma ? kQ4KGemmMinRows : g_q4k_tensor_rows.load(std::memory_order_relaxed));
+  return q4k_matmul_layout(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2), m, n, k,
+                           wmma ? kQ4KGemmMinRows : g_q4k_tensor_rows.load(std::memory_order_relaxed), layout);
 }
 qmm_status run_gemm_q4k(const LaunchCtx& c) { return run_gemm_q4k_id(c, false); }
 qmm_status run_gemm_q4k_wmma(const LaunchCtx& c) { return run_gemm_q4k_id(c, true); }
 
 // "gemm_q4k_vec" and "gemm_q4k_rows{R}": buffers A, W, C; scalars m, n, k, split
-// (src/backends/rocm/rocm_kernels_gemv.cpp:17-24,103-156).  C has `split` regions of
+// (src/backends/rocm/rocm_kernels_gemv.cpp:17-24,103-156), optionally followed by `layout`.  C has `split` regions of
 // m*n floats whose sum is the result: either every region receives the partial sums of its K
 // slice (one row, slices of 4096 weights or more), or region 0 receives the whole dot product and
 // regions 1..split-1 are zeroed; "gemm_vec_reduce" over them yields the result either way.
 qmm_status run_gemm_q4k_split(const LaunchCtx& c, uint64_t rows_required) {
-  if (!counts(c, 3, 4)) return bad("gemm_q4k_vec/rows: expects 3 buffers and 4 scalars");
-  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], split = c.sc[3];
+  if (!counts(c, 3, 4) && !counts(c, 3, 5)) return bad("gemm_q4k_vec/rows: expects 3 buffers and 4 scalars (a fifth: layout)");
+  const uint64_t m = c.sc[0], n = c.sc[1], k = c.sc[2], split = c.sc[3], layout = c.nsc > 4 ? c.sc[4] : 0;
   if (!dims_ok(m, n, k) || k % 256 != 0) return bad("gemm_q4k_vec/rows: bad m, n, k");
+  if (!q4k_layout_ok(n, k, layout)) return bad("gemm_q4k_vec/rows: layout is 0 (GGUF order) or the rows per group of a row-group copy (1..64)");
   if (rows_required != 0 && m != rows_required) return bad("gemm_q4k_rowsR: m must equal R");
   if (split == 0 || split > 64 || (k / 256) % split != 0) return bad("gemm_q4k_vec/rows: split must divide k/256");
   const u128 region = static_cast<u128>(m) * n * 4;
@@ -250,11 +293,12 @@ qmm_status run_gemm_q4k_split(const LaunchCtx& c, uint64_t rows_required) {
   float* out = c.ptr<float>(2);
   // One row of a large matrix with long enough slices: real partial sums, one region per slice,
   // each workgroup staging only its slice of the activations.
-  if (m == 1 && n <= 0xFFFFFFFFull && k <= 0xFFFFFFFFull && qmm::q4k_gemv_split_supported(n, k, split)) {
+  if (layout == 0 && m == 1 && n <= 0xFFFFFFFFull && k <= 0xFFFFFFFFull && qmm::q4k_gemv_split_supported(n, k, split)) {
     return map_hip(qmm::launch_q4k_gemv_split(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, static_cast<uint32_t>(n),
                                               static_cast<uint32_t>(k), static_cast<uint32_t>(split), c.stream));
   }
-  qmm_status st = q4k_matmul(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, m, n, k);
+  qmm_status st = q4k_matmul_layout(c, c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, m, n, k,
+                                    g_q4k_tensor_rows.load(std::memory_order_relaxed), layout);
   if (st == QMM_OK && split > 1) {
     st = map_hip(qmm::launch_fill_f32(out + m * n, 0.0f, (split - 1) * m * n, c.stream));
   }
@@ -859,6 +903,22 @@ qmm_status run_permute_mxfp4_wmma(const LaunchCtx& c) {
   return map_hip(qmm::launch_permute_mxfp4_wmma(c.ptr<const uint8_t>(0), c.ptr<uint8_t>(1), n, k, inverse == 1, c.stream));
 }
 
+// "permute_q4k_rowgroup" (not a reference id; the Q4_K counterpart of the hook above, for this part's
+// int8 matrix instruction): buffers In, Out (n x k/256 Q4_K blocks each); scalars n, k, rows per group
+// (1..64; 0 = the default, 32), inverse (0: GGUF order -> row groups, 1: back).
+qmm_status run_permute_q4k_rowgroup(const LaunchCtx& c) {
+  if (!counts(c, 2, 4)) return bad("permute_q4k_rowgroup: expects 2 buffers and 4 scalars");
+  const uint64_t n = c.sc[0], k = c.sc[1], inverse = c.sc[3];
+  const uint64_t rows = c.sc[2] == 0 ? qmm::q4k_rowgroup_default_rows(n) : c.sc[2];
+  if (!dims_ok(1, n, k) || k % 256 != 0 || inverse > 1 || !qmm::q4k_rowgroup_supported(n, k, rows)) {
+    return bad("permute_q4k_rowgroup: k a multiple of 256, 1..64 rows per group, inverse 0 or 1");
+  }
+  if (!c.fits(0, q4k_bytes(n, k)) || !c.fits(1, q4k_bytes(n, k))) return bad("permute_q4k_rowgroup: buffer too small");
+  if (c.buf[0] == c.buf[1]) return bad("permute_q4k_rowgroup: not in place");
+  return map_hip(qmm::launch_q4k_rowgroup(c.ptr<const uint8_t>(0), c.ptr<uint8_t>(1), static_cast<uint32_t>(n),
+                                          static_cast<uint32_t>(k), static_cast<uint32_t>(rows), inverse == 1, c.stream));
+}
+
 // "dequant_mxfp4" (not a reference id): buffers W (packed), Out (n x k fp32); scalars n, k.
 qmm_status run_dequant_mxfp4(const LaunchCtx& c) {
   if (!counts(c, 2, 2)) return bad("dequant_mxfp4: expects 2 buffers and 2 scalars");
@@ -1205,6 +1265,7 @@ const Entry kTable[] = {
     {"dequant_q6k", run_dequant_q6k},
     {"dequant_mxfp4", run_dequant_mxfp4},
     {"permute_mxfp4_wmma", run_permute_mxfp4_wmma},
+    {"permute_q4k_rowgroup", run_permute_q4k_rowgroup},
     {"quantize_fp8_pack_a16", run_quantize_fp8_pack_a16},
 };
 constexpr size_t kTableSize = sizeof(kTable) / sizeof(kTable[0]);
@@ -1388,9 +1449,12 @@ qmm_status qmm_workspace_bytes(qmm_kernel kernel, const uint64_t* scalars, size_
   auto sc = [&](size_t i) { return i < nscalars ? scalars[i] : uint64_t{0}; };
   auto starts = [&](const char* prefix) { return id.rfind(prefix, 0) == 0; };
   if (starts("gemm_q4k")) {
-    const uint64_t m = sc(0), k = sc(2);
+    const uint64_t m = sc(0), n = sc(1), k = sc(2);
+    const bool split_id = id == "gemm_q4k_vec" || starts("gemm_q4k_rows");
+    const uint64_t layout = sc(split_id ? 4 : 3);
     const uint64_t from = id == "gemm_q4k_wmma" ? kQ4KGemmMinRows : g_q4k_tensor_rows.load(std::memory_order_relaxed);
     if (m >= from && qmm::gemm_q4k_supported(m, k)) *out_bytes = qmm::gemm_q4k_workspace_bytes(m, k);
+    if (layout != 0 && m > 1 && k % 256 == 0) *out_bytes = q4k_regime_workspace(m, k, from) + static_cast<size_t>(q4k_bytes(n, k));
   } else if (id == "ffn_gate_up_silu_q4k") {
     const uint64_t m = sc(0), n = sc(1), k = sc(2);
     if (m >= 2 && n != 0 && k != 0) *out_bytes = ffn_scratch(m, n, k).workspace_bytes;

@@ -43,6 +43,19 @@ size_t gemv_q4k_mfma_workspace_bytes(uint64_t m, uint64_t k);
 hipError_t launch_q4k_gemv_mfma(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                                 uint32_t n, uint32_t k, hipStream_t stream);
 
+// Q4_K in row-group order (gemv_q4k_i8.hip): a load-time copy of a GGUF Q4_K matrix, same byte count, in which
+// `rows_per_group` consecutive rows (at most kQ4KRowGroupMaxRows; the last group may be shorter) are stored
+// together block by block in the operand order of the int8 matrix instruction.
+constexpr uint32_t kQ4KRowGroupMaxRows = 64;
+uint32_t q4k_rowgroup_default_rows(uint64_t n);
+bool q4k_rowgroup_supported(uint64_t n, uint64_t k, uint64_t rows_per_group);
+// GGUF -> row groups (inverse: back); not in place.
+hipError_t launch_q4k_rowgroup(const uint8_t* in, uint8_t* out, uint32_t n, uint32_t k, uint32_t rows_per_group,
+                               bool inverse, hipStream_t stream);
+// c (n fp32) = deq(W) . a for one activation row, W in row-group order.
+hipError_t launch_q4k_i8_gemv(const float* a, const uint8_t* w, float* c, uint32_t n, uint32_t k,
+                              uint32_t rows_per_group, hipStream_t stream);
+
 // ---- routed experts, Q4_K (gemv.hip) ----------------------------------------------
 // phi[t][slot*inter + j] = silu(G_e x_t)[j] * (U_e x_t)[j], e = ids[t][slot]; `rows` tokens.
 hipError_t launch_moe_gate_up_q4k(const float* x, const uint8_t* gate, const uint8_t* up,

@@ -139,3 +139,54 @@ def test_gemm_q4k_rejects_bad_shapes():
         with pytest.raises(oracle.OracleError) as e:
             oracle.gemm_q4k(np.zeros(max(m * k, 1), np.float32), np.zeros(144, np.uint8), m, n, k)
         assert e.value.code == 1
+
+
+def decode_rowgroups(buf: np.ndarray, n: int, k: int, R: int) -> np.ndarray:
+    """deq(W) read straight from a row-group copy, following the layout's text only (no call into the
+    oracle): group g keeps, per block, the tiles' quants and then the rows' headers; a weight of
+    sub-block s < 4 is a low nibble of pair set s // 2, one of s >= 4 a high nibble (stored minus 8) of
+    pair set (s - 4) // 2; value = RN32(d * sc * q - dmin * mn) from exact products."""
+    buf = np.asarray(buf, np.uint8).reshape(-1)
+    nblk = k // 256
+    out = np.empty((n, k), np.float32)
+    for r in range(n):
+        row0 = r // R * R
+        rows = min(R, n - row0)
+        rr = r - row0
+        tile, nn = divmod(rr, 16)
+        rt = min(16, rows - tile * 16)
+        for b in range(nblk):
+            region = (row0 * nblk + b * rows) * 144
+            h = buf[region + rows * 128 + rr * 16:][:16]
+            d, dmin = (float(v) for v in h[:4].view(np.float16))
+            for s in range(8):
+                i, odd = divmod(s, 2)
+                if odd:
+                    sc = int(h[8 + i]) & 63
+                    mn = (int(h[4 + i]) >> 6) | ((int(h[8 + i]) >> 6) << 2) | ((int(h[12 + i]) >> 6) << 4)
+                else:
+                    sc = int(h[4 + i]) & 63
+                    mn = int(h[12 + i]) & 63
+                c = (s % 4) // 2
+                for l in range(32):
+                    q4 = 2 * (s % 2) + l // 16
+                    byte = int(buf[region + tile * 2048 + c * rt * 64 + (q4 * rt + nn) * 16 + l % 16])
+                    q = (byte & 15) if s < 4 else (((byte >> 4) + 8) & 15)
+                    out[r, b * 256 + s * 32 + l] = np.float32(d * sc * q - dmin * mn)   # float64, rounded once
+    return out
+
+
+@pytest.mark.parametrize("n,k,R", [(40, 512, 32), (21, 256, 16), (70, 256, 64), (9, 512, 7), (33, 256, 20)])
+def test_rowgroup_copy_is_a_permutation_that_decodes_to_the_same_weights(n, k, R):
+    g = synth.rng(77 + n)
+    w = synth.q4k_weights(g, n, k)
+    # every scale / min value somewhere, so that a wrong bit position in the re-packed header shows
+    blocks = np.asarray(w).reshape(-1, 144)
+    blocks[:, 4:16] = g.integers(0, 256, (blocks.shape[0], 12), dtype=np.uint8)
+    w = blocks.reshape(-1)
+    p = oracle.permute_q4k_rowgroup(w, n, k, R)
+    assert p.shape == w.shape
+    assert np.array_equal(oracle.permute_q4k_rowgroup(p, n, k, R, inverse=True), w)
+    want = oracle.dequantize_q4k(w).reshape(n, k)
+    got = decode_rowgroups(p, n, k, R)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

@@ -17,6 +17,16 @@ def rel_err(got: np.ndarray, ref: np.ndarray) -> float:
     return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps)))
 
 
+def strict_rel_err(got: np.ndarray, ref: np.ndarray) -> float:
+    """The same figure with the floor the measurement plan names, eps = 1e-3 * rms(ref): reported next
+    to rel_err by the full-size tests.  Near that floor it measures the reference's own summation
+    noise as much as the device's (see rel_err), so it is printed, and asserted only loosely."""
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    eps = 1e-3 * np.sqrt(np.mean(ref * ref)) + 1e-30
+    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps)))
+
+
 def rms_err(got: np.ndarray, ref: np.ndarray) -> float:
     """max |got - ref| / rms(ref): the absolute error in units of a typical output."""
     got = np.asarray(got, dtype=np.float64).reshape(-1)

@@ -159,12 +159,13 @@ qmm_status qmm_set_workspace(void* device_ptr, size_t bytes);
 /* The row count from which the Q4_K ids other than "gemm_q4k_wmma" ("gemm_q4k", "gemm_q4k_batched",
  * "ffn_gate_up_silu_q4k") use the fp16 tensor-core tile, whose operands are rounded to fp16.
  * Default 64: the reference's regime table switches to its own fp16 tile there (kGemmWmmaMinRows,
- * src/core/decode_internal.hpp:1349-1361) and keeps fp32 activations below
- * (src/models/qwen3_5/project.cpp:307-322), so by default a result carries the fp16 operand
+ * src/core/decode_internal.hpp:1428, used at src/models/qwen3_5/project.cpp:307) and keeps fp32
+ * activations below (src/models/qwen3_5/project.cpp:307-322), so by default a result carries the fp16 operand
  * rounding exactly where the reference's does; 17..63 rows then run sixteen at a time through the
  * exact kernels (about 28 us per 16 rows of a 17408 x 5120 matrix, against 35..46 us for the
  * tile).  A caller that prefers the tile's speed there sets a lower count, at least 17 (up to 16
- * rows, the speculative-verify batch, always stay exact); 0 restores the default.
+ * rows, the speculative-verify batch, always stay exact); a higher count keeps more rows on the
+ * exact kernels, sixteen at a time; 0 restores the default.
  * "gemm_q4k_wmma" itself uses the tile from 17 rows whatever this says.  Process-wide; not a
  * reference interface (its table is compiled in). */
 qmm_status qmm_set_q4k_tensor_rows(uint32_t rows);

@@ -160,7 +160,7 @@ void* decode_scratch(const LaunchCtx& c) {
 // once).  The tiled fp16 MFMA GEMM, whose operands are rounded to fp16 as in the reference's
 // tensor-core tile: "gemm_q4k_wmma" from kQ4KGemmMinRows rows, the other ids from
 // g_q4k_tensor_rows rows -- 64 by default, where the reference's own regime table switches to its
-// fp16 tile (src/core/decode_internal.hpp:1349-1361), so that below it results keep the fp32
+// fp16 tile (kGemmWmmaMinRows, src/core/decode_internal.hpp:1428; src/models/qwen3_5/project.cpp:307), so that below it results keep the fp32
 // contract of the reference's tiled kernel; more rows than 16 below that run sixteen at a time
 // through the exact kernels.  qmm_set_q4k_tensor_rows lowers it (at least kQ4KGemmMinRows).
 constexpr uint64_t kQ4KGemmMinRows = 17;
@@ -619,7 +619,10 @@ FfnScratch ffn_scratch(uint64_t m, uint64_t n, uint64_t k) {
     room = room > parts_tail ? room : parts_tail;
     const size_t up_off = (room + 255) & ~size_t{255};
     if (up_off + up_bytes <= kDecodeScratchBytes) return FfnScratch{true, up_off, 0};
-    return FfnScratch{false, 0, up_bytes};
+    // In the workspace, but still behind the few-row kernels' room: qmm_launch_static serves the
+    // workspace and the decode scratch from the same array, where offset 0 would be under their
+    // partial sums.
+    return FfnScratch{false, up_off, up_off + up_bytes};
   }
   const size_t up_off = (qmm::gemm_q4k_workspace_bytes(m, k) + 255) & ~size_t{255};
   return FfnScratch{false, up_off, up_off + up_bytes};

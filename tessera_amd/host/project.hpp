@@ -16,7 +16,7 @@ namespace tessera_amd {
 constexpr std::size_t kGemmVecOutputsPerBlock = 8;
 constexpr std::size_t kGemmVecSplitTargetBlocks = 2048;
 constexpr std::size_t kGemmVecMaxSplit = 8;
-// src/core/decode_internal.hpp:1349-1361,1425-1441.
+// src/core/decode_internal.hpp:1349-1361 (tile sizes), 1425-1441 (kGemmWmmaMinRows at 1428).
 constexpr std::size_t kGemmWmmaMinRows = 64;
 constexpr std::size_t kGemmWmmaMinCols = 32;
 constexpr std::size_t kTiledMinRows = 16;
@@ -163,7 +163,10 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
     auto gemm = CachedKernel(backend, h, m == 1 ? "gemm_mxfp4" : (m <= 16 ? "gemm_mxfp4_rows" : "gemm_mxfp4_batched"));
     if (!gemm) return unexpected(gemm.error());
     KernelLaunch l;
-    l.grid_x = static_cast<std::uint32_t>(m == 1 ? (n + 7) / 8 : (n + 7) / 8);
+    // the reference's shapes: a warp per column for one row and for up to 16 rows
+    // (src/backends/rocm/rocm_kernels_basic.cpp:1097-1214), 32 x 32 tiles for the batched kernel; the
+    // library picks its own geometry from m, n, k either way
+    l.grid_x = static_cast<std::uint32_t>(m <= 16 ? (n + 7) / 8 : ((m + 31) / 32) * ((n + 31) / 32));
     l.buffers = {&a, &w, &out};
     l.scalars = {m, n, k};
     return backend.LaunchKernel(**gemm, l);

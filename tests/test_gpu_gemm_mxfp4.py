@@ -45,6 +45,16 @@ def test_gemm_matches_oracle(backend, m, n, k):
     assert rel_err(got, ref) <= 1e-2, rel_err(got, ref)
 
 
+def w4a8_oracle(x, w, m, n, k):
+    """QuantizeFp8Ref then GemmMxFp4Ref on all host cores: the threaded fp32-activation oracle fed with
+    the quantize-dequantized rows e4m3(code) * scale, which is what the single-threaded W4A8 oracle
+    multiplies (checked bit for bit on two rows where this is used)."""
+    codes, scale = oracle.quantize_fp8_pack(x, m, k)
+    lut = np.array([oracle.fp8_e4m3_to_float(c) for c in range(256)], np.float32)
+    qdq = (lut[codes] * scale.reshape(m, 1)).astype(np.float32)
+    return oracle.gemm_mxfp4(qdq, w, m, n, k, threads=True)
+
+
 def test_gemm_block_scales_and_codes_exact(backend):
     """Every E2M1 code under a wide spread of E8M0 exponents, one-hot E4M3 activations: each
     output is a single exact product, so the MFMA operand layout (which lane supplies which
@@ -70,10 +80,18 @@ def test_full_size_prefill_rows(backend):
     w = synth.mxfp4_weights(g, n, k, -8, -4)
     x = synth.activations_bf16(g, m, k)
     got = w4a8(backend, x, w, m, n, k)
-    rows = [0, 1, 777, 2047]
-    codes, scale = oracle.quantize_fp8_pack(x[rows], len(rows), k)
-    ref = oracle.gemm_mxfp4_w4a8(codes, scale, w, len(rows), n, k)
+    # 72 rows: every position inside a 32-row MFMA tile, spread over all eight 256-row tiles, all
+    # columns (the 256 x 256 tiles and the 128 x 64 ones that take the leftover columns)
+    rows = sorted({(37 * i) % 2048 for i in range(64)} | {0, 31, 32, 255, 256, 1023, 2016, 2047})
+    assert {r % 32 for r in rows} == set(range(32)) and {r // 256 for r in rows} == set(range(8))
+    ref = w4a8_oracle(x[rows], w, len(rows), n, k)
+    few = [0, 3]
+    codes, scale = oracle.quantize_fp8_pack(x[rows][few], len(few), k)
+    assert np.array_equal(ref[few], oracle.gemm_mxfp4_w4a8(codes, scale, w, len(few), n, k))
+    print(f"configs[3] W4A8 2048x17408x5120, {len(rows)} rows: max|d|/rms {rms_err(got[rows], ref):.2e}, "
+          f"2-norm {norm_err(got[rows], ref):.2e}, rel (floor 0.05 rms) {rel_err(got[rows], ref):.2e}")
     assert rms_err(got[rows], ref) <= 5e-4, rms_err(got[rows], ref)
+    assert norm_err(got[rows], ref) <= 5e-5, norm_err(got[rows], ref)
     shard = synth.mxfp4_column_shard(w, n, k, 0, n // 2)
     got_shard = w4a8(backend, x, shard, m, n // 2, k)
     assert np.array_equal(got_shard, got[:, : n // 2])
@@ -86,9 +104,9 @@ def test_down_projection_shape_prefill_rows(backend):
     w = synth.mxfp4_weights(g, n, k, -8, -4)
     x = synth.activations_bf16(g, m, k)
     got = w4a8(backend, x, w, m, n, k)
-    rows = [0, 255, 256, 499]
-    codes, scale = oracle.quantize_fp8_pack(x[rows], len(rows), k)
-    ref = oracle.gemm_mxfp4_w4a8(codes, scale, w, len(rows), n, k)
+    rows = sorted({(37 * i) % 500 for i in range(40)} | {0, 31, 32, 255, 256, 499})
+    assert {r % 32 for r in rows} == set(range(32))
+    ref = w4a8_oracle(x[rows], w, len(rows), n, k)
     assert rms_err(got[rows], ref) <= 5e-4, rms_err(got[rows], ref)
 
 

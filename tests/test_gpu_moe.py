@@ -161,7 +161,18 @@ def test_config4_shapes(backend):
     x = synth.activations_bf16(g, rows, hidden)
     ids, vals = synth.moe_routing(g, rows, experts, top_k)
     wts = np.stack([oracle.moe_gate(v) for v in vals])
-    sample = [0, 1, 100, 255, 256, 511]
+    # tokens picked greedily until every one of the 256 experts has been routed to (at least 64 of them)
+    sample, seen = [0, 1, 100, 255, 256, 511], set()
+    for r in sample:
+        seen.update(int(e) for e in ids[r])
+    order = [int(r) for r in g.permutation(rows)]
+    while len(seen) < experts or len(sample) < 64:
+        r = max(order[:64], key=lambda t: len(set(int(e) for e in ids[t]) - seen)) if len(seen) < experts else order[0]
+        order.remove(r)
+        if r not in sample:
+            sample.append(r)
+            seen.update(int(e) for e in ids[r])
+    assert len(seen) == experts and len(sample) >= 64
     ref = oracle.moe_batch_forward_q4k(x[sample], ids[sample], wts[sample], gate, up, down, hidden, inter)
     # Up to 16 tokens the two row-batched ids take one exact fp32 pass per token.
     few = forward_rows(backend, x[:16], ids[:16], wts[:16], gate, up, down, hidden, inter, experts)

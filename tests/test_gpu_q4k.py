@@ -9,7 +9,7 @@ import pytest
 
 import oracle
 from tessera_amd import StatusCode, StatusError, synth
-from util import ref_grid_vec, rel_err, rms_err, run, same_bits, same_bits_zero_sign_free
+from util import ref_grid_vec, rel_err, rms_err, run, same_bits, same_bits_zero_sign_free, strict_rel_err
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -302,14 +302,18 @@ def test_few_rows_scaling_and_exactness(backend):
 
 
 def test_few_rows_full_size(backend):
-    """configs[1] shapes with 4 and 8 rows (speculative verify), against the oracle."""
-    for seed, (n, k, m) in enumerate([(17408, 5120, 4), (5120, 17408, 8)]):
+    """configs[1] shapes with 4, 8 and 16 rows (speculative verify; the split of K into parts depends
+    on both N and the row count), every row and column against the threaded oracle."""
+    for seed, (n, k, m) in enumerate([(17408, 5120, 4), (5120, 17408, 8), (17408, 5120, 16), (5120, 17408, 16),
+                                      (17408, 5120, 9), (5120, 17408, 2)]):
         g = synth.rng(909 + seed)
         w = synth.q4k_weights(g, n, k)
         a = synth.activations_f32(g, m, k)
         ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
         got = gemm(backend, f"gemm_q4k_rows{m}" if m <= 5 else "gemm_q4k_batched", a, w, m, n, k,
                    extra=(1,) if m <= 5 else ())[0]
+        print(f"Q4_K {m} rows {n}x{k}: rel_err {rel_err(got, ref):.2e} (floor 0.05 rms), "
+              f"{strict_rel_err(got, ref):.2e} (floor 1e-3 rms), max|d|/rms {rms_err(got, ref):.2e}")
         assert rel_err(got, ref) <= TOL, (n, k, m, rel_err(got, ref))
         # each row equals the single-row kernel's answer to fp32 summation-order noise
         one = gemm(backend, "gemm_q4k_vec", a[:1], w, 1, n, k, extra=(1,))[0]
@@ -334,6 +338,8 @@ def test_full_size_configs(backend):
         a = synth.activations_f32(g, 1, k)
         ref = oracle.gemm_q4k(a, w, 1, n, k, threads=True)
         got = gemm(backend, "gemm_q4k_vec", a, w, 1, n, k, extra=(1,))[0]
+        print(f"Q4_K gemv {n}x{k}: rel_err {rel_err(got, ref):.2e} (floor 0.05 rms), "
+              f"{strict_rel_err(got, ref):.2e} (floor 1e-3 rms), max|d|/rms {rms_err(got, ref):.2e}")
         assert rel_err(got, ref) <= TOL, (n, k, rel_err(got, ref))
         # linearity, a size-independent property: W(2a) == 2 W a exactly (power-of-two scaling)
         got2 = gemm(backend, "gemm_q4k_vec", 2 * a, w, 1, n, k, extra=(1,))[0]

@@ -47,6 +47,25 @@ def test_static_scratch_matches_allocating_entry_point(backend):
             assert np.array_equal(_bits(got), _bits(ref)), ("ffn_gate_up_silu_q4k", m)
 
 
+def test_static_scratch_up_product_that_does_not_fit_the_decode_room(backend):
+    """ffn_gate_up_silu_q4k with 40 rows of a wide matrix: the up product (21 MB) does not fit beside the
+    few-row kernels' partial sums in the first 16 MB, so it goes behind them in the same static array and
+    must not be overwritten by the second 16-row chunk's partials; then a smaller call."""
+    g = synth.rng(4245)
+    n, k = 131072, 2048
+    base = synth.q4k_weights(g, 4096, k)
+    w = np.tile(np.asarray(base).reshape(-1), n // 4096)
+    up = np.roll(w, 144 * 77)
+    dw, dup = backend.Upload(w), backend.Upload(up)
+    for m in (40, 18):
+        a = synth.activations_f32(g, m, k)
+        da = backend.Upload(a)
+        out = backend.AllocateBuffer(4 * m * n)
+        ref, got = _both(backend, "ffn_gate_up_silu_q4k", [da, dw, dup, out], out, [m, n, k], (m * n + 7) // 8)
+        assert np.isfinite(ref).all()
+        assert np.array_equal(_bits(got), _bits(ref)), m
+
+
 def test_static_scratch_grouped_experts_then_smaller_chunk(backend):
     g = synth.rng(4243)
     experts, hidden, inter, top_k = 16, 512, 256, 4

@@ -138,3 +138,76 @@ def test_prefill_call_recorded_with_a_caller_owned_workspace(backend):
         backend.SetWorkspace(None)
     backend.LaunchKernel(kern, KernelLaunch(grid_x=1, buffers=[wrap(xb), wrap(w), wrap(yb)], scalars=[2 * m, n, k]))
     torch.cuda.synchronize()
+
+
+def test_recorded_prefill_survives_growth_of_the_library_workspace(backend):
+    """A prefill-sized call recorded against the library-owned workspace, then a larger eager call
+    that makes the library get a bigger block: the block the graph points at is retired, not freed,
+    so the replays still equal eager launches.  And while a stream is being captured the library's
+    block cannot grow: such a launch is refused, and works once an eager call of that size has run."""
+    from tessera_amd import StatusCode, StatusError
+    dev = torch.device("cuda:0")
+    g = synth.rng(902)
+    n, k = 1030, 4096
+    to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    wrap = lambda t: backend.WrapBuffer(t.data_ptr(), t.numel() * t.element_size())
+    w = to_dev(synth.q4k_weights(g, n, k))
+    kern = backend.LoadKernel("gemm_q4k_wmma")
+    cur = torch.cuda.current_stream()
+    backend.SetStream(cur.cuda_stream)
+    backend.SetWorkspace(None)
+    # far larger than anything another test asks for (the largest is a 178 MB decode of a K-quant tensor),
+    # so that this call and the next both make the block grow; inputs are made on the device
+    m_small, m_big = 40000, 90000
+    assert backend.WorkspaceBytes(kern, [m_big, n, k]) > 2 * backend.WorkspaceBytes(kern, [m_small, n, k]) > (512 << 20)
+    gen = torch.Generator(device=dev)
+
+    def fill(t, seed):
+        gen.manual_seed(seed)
+        t.normal_(generator=gen)
+    x = torch.empty(m_small * k, device=dev)
+    y = torch.empty(m_small * n, device=dev)
+    launch = KernelLaunch(grid_x=n // 64 + 1, buffers=[wrap(x), wrap(w), wrap(y)], scalars=[m_small, n, k])
+    fill(x, 21)
+    # capture before any eager call of this size: the library would have to allocate, refused
+    graph = torch.cuda.CUDAGraph()
+    refused = False
+    with torch.cuda.graph(graph):
+        backend.SetStream(torch.cuda.current_stream().cuda_stream)
+        try:
+            backend.LaunchKernel(kern, launch)
+        except StatusError as e:
+            refused = e.code == StatusCode.InvalidArgument and "captured" in str(e)
+    backend.SetStream(cur.cuda_stream)
+    assert refused
+    backend.LaunchKernel(kern, launch)          # eager: the block grows to this size
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        backend.SetStream(torch.cuda.current_stream().cuda_stream)
+        backend.LaunchKernel(kern, launch)
+    backend.SetStream(cur.cuda_stream)
+    xb = torch.empty(m_big * k, device=dev)
+    fill(xb, 22)
+    yb = torch.empty(m_big * n, device=dev)
+    for seed in (21, 23):
+        fill(x, seed)
+        y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.cpu().numpy().copy()
+        # a larger eager call: the library's block is replaced (on the first pass)
+        backend.LaunchKernel(kern, KernelLaunch(grid_x=1, buffers=[wrap(xb), wrap(w), wrap(yb)], scalars=[m_big, n, k]))
+        torch.cuda.synchronize()
+        y.fill_(float("nan"))
+        backend.LaunchKernel(kern, launch)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.view(np.uint32), y.cpu().numpy().view(np.uint32)), seed
+    # and once more through the graph, now that its block is a retired one
+    y.fill_(float("nan"))
+    graph.replay()
+    torch.cuda.synchronize()
+    backend.LaunchKernel(kern, launch)
+    got = y.cpu().numpy().copy()
+    torch.cuda.synchronize()
+    assert np.array_equal(got.view(np.uint32), y.cpu().numpy().view(np.uint32))

@@ -279,6 +279,24 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
             del wf_list, wf
         out[f"{fmt}_gemv"] = res
 
+    # ---- the matrix-core ceiling as measured here: a register-only loop of each GEMM's instruction
+    # ("mfma_probe"), constant operands and hashed ones (the part's power limit prices the toggling bits)
+    kmp = backend.LoadKernel("mfma_probe")
+    probe_wgs, probe_iters = 1024, 4000
+    pout = torch.empty(probe_wgs * 256, dtype=torch.float32, device=dev)
+    ceiling = {}
+    for kind, label, flop, per_clk in ((0, "f16_32x32x16", 2 * 32 * 32 * 16, 1024), (1, "f8f4_scaled_32x32x64", 2 * 32 * 32 * 64, 2048),
+                                       (2, "i8_16x16x64", 2 * 16 * 16 * 64, 2048)):
+        for rnd in (0, 1):
+            us = timed_us([(kmp, KernelLaunch(grid_x=probe_wgs, buffers=[wrap(pout)], scalars=[kind, rnd, probe_iters, probe_wgs]))],
+                          3, graph=False)
+            tflops = probe_wgs * 16 * probe_iters * flop / us / 1e6
+            ceiling[f"{label}_{'random' if rnd else 'constant'}"] = {
+                "TFLOPs": round(tflops, 1),
+                # what core clock that rate means if the instruction issues back to back at its nominal rate
+                "implied_GHz": round(tflops * 1e12 / (256 * 4 * per_clk) / 1e9, 3)}
+    out["mfma_ceiling"] = ceiling
+
     # ---- configs[3]: prefill GEMM M=2048 ---------------------------------------------------
     m = 2048
     prefill = {}
@@ -333,6 +351,10 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
         prefill[f"{fmt}_n17408"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * n * k / us / 1e6, 1),
                                     "frac_fp16_peak": round(2 * m * n * k / us / 1e6 / 2500.0, 4)}
         del wf
+    for key, val in prefill.items():
+        ref_key = "f8f4_scaled_32x32x64_random" if key.startswith("mxfp4") else "f16_32x32x16_random"
+        mult = val.get("e4m3_terms", 1)          # the fp32-row form does `terms` times the fp8 work per product flop
+        val["frac_of_measured_ceiling"] = round(val["TFLOPs"] * mult / ceiling[ref_key]["TFLOPs"], 4)
     out["prefill_gemm_m2048_k5120"] = prefill
 
     # ---- the same prefill at the down-projection shape (N=5120, K=17408) ---------------------------

@@ -499,6 +499,97 @@ hipError_t launch_read_probe(const void* src, uint32_t* out, uint64_t bytes, hip
   return hipGetLastError();
 }
 
+// Ceiling of the matrix cores as the GEMMs meet it (the "mfma_probe" id): a register-only loop of one
+// matrix instruction, four independent accumulators per wavefront, four wavefronts per SIMD, operands
+// either constant (few bits toggle between instructions) or hashed (random bits, which is what real
+// weights and activations look like and what the part's power limit prices).  kind 0:
+// v_mfma_f32_32x32x16_f16, 1: v_mfma_scale_f32_32x32x64_f8f6f4 with an E4M3 and an E2M1 operand (the
+// W4A8 prefill's instruction), 2: v_mfma_i32_16x16x64_i8 (the row-group decode GEMV's).
+template <int KIND, bool RANDOM>
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float* out, uint32_t iters) {
+  auto hash = [](uint32_t v) {
+    v *= 2654435761u, v ^= v >> 15, v *= 2246822519u, v ^= v >> 13, v *= 3266489917u, v ^= v >> 16;
+    return v;
+  };
+  const uint32_t seed = threadIdx.x * 8u + blockIdx.x * 977u;
+  float result = 0.0f;
+  if constexpr (KIND == 0) {
+    half8_t a, b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      // random: values in [1, 2) with random mantissas and signs; constant: small integers
+      const uint32_t ha = hash(seed + e), hb = hash(seed + 64u + e);
+      a[e] = RANDOM ? bit_cast<_Float16>(static_cast<uint16_t>(0x3C00u | (ha & 0x83FFu))) : static_cast<_Float16>(1.0f);
+      b[e] = RANDOM ? bit_cast<_Float16>(static_cast<uint16_t>(0x3C00u | (hb & 0x83FFu))) : static_cast<_Float16>(0.5f);
+    }
+    float16_t acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+    for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) result += acc[i][e];
+  } else if constexpr (KIND == 1) {
+    int8v_t a, b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      a[e] = RANDOM ? static_cast<int>(hash(seed + e) & 0x77777777u) : 0x38383838;   // E4M3, exponent capped
+      b[e] = RANDOM ? static_cast<int>(hash(seed + 64u + e)) : 0x22222222;           // E2M1 in the low half
+    }
+    float16_t acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+    for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i], 0, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) result += acc[i][e];
+  } else {
+    int4v_t a, b;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[e] = RANDOM ? static_cast<int>(hash(seed + e)) : 0x01010101;
+      b[e] = RANDOM ? static_cast<int>(hash(seed + 64u + e) & 0x0F0F0F0Fu) : 0x03030303;
+    }
+    int4v_t acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = int4v_t{0, 0, 0, 0};
+    for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) result += static_cast<float>(acc[i][0] ^ acc[i][1] ^ acc[i][2] ^ acc[i][3]);
+  }
+  out[static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x] = result;
+}
+
+hipError_t launch_mfma_probe(float* out, uint32_t kind, bool random, uint32_t iters, uint32_t workgroups,
+                             hipStream_t stream) {
+#define QMM_PROBE(K)                                                                                          \
+  if (kind == K) {                                                                                            \
+    if (random) hipLaunchKernelGGL((mfma_probe_kernel<K, true>), dim3(workgroups), dim3(256), 0, stream, out, iters); \
+    else hipLaunchKernelGGL((mfma_probe_kernel<K, false>), dim3(workgroups), dim3(256), 0, stream, out, iters);       \
+    return hipGetLastError();                                                                                 \
+  }
+  QMM_PROBE(0) QMM_PROBE(1) QMM_PROBE(2)
+#undef QMM_PROBE
+  return hipErrorInvalidValue;
+}
+
 hipError_t launch_fill_i32(int32_t* out, int32_t value, uint64_t n, hipStream_t stream) {
   hipLaunchKernelGGL(fill_i32_kernel, grid_for(n, 256), dim3(256), 0, stream, out, value, n);
   return hipGetLastError();

@@ -351,6 +351,20 @@ qmm_status run_read_probe(const LaunchCtx& c) {
   return map_hip(qmm::launch_read_probe(c.ptr<const void>(0), c.ptr<uint32_t>(1), bytes, c.stream));
 }
 
+// "mfma_probe" (not a reference id; the matrix-core ceiling the prefill GEMMs are compared with, as
+// "read_probe" is the memory one): buffer out (workgroups * 256 fp32); scalars kind (0: fp16 32x32x16,
+// 1: scaled E4M3 x E2M1 32x32x64, 2: int8 16x16x64), random (0: constant operands, 1: hashed), iters,
+// workgroups.  Executes workgroups * 4 * 4 * iters matrix instructions and nothing else.
+qmm_status run_mfma_probe(const LaunchCtx& c) {
+  if (!counts(c, 1, 4)) return bad("mfma_probe: expects 1 buffer and 4 scalars");
+  const uint64_t kind = c.sc[0], random = c.sc[1], iters = c.sc[2], wgs = c.sc[3];
+  if (kind > 2 || random > 1 || iters == 0 || iters > (1u << 24) || wgs == 0 || wgs > 65536 || !c.fits(0, wgs * 1024)) {
+    return bad("mfma_probe: kind 0..2, random 0 or 1, 1..2^24 iterations, 1..65536 workgroups, out of workgroups * 256 floats");
+  }
+  return map_hip(qmm::launch_mfma_probe(c.ptr<float>(0), static_cast<uint32_t>(kind), random == 1, static_cast<uint32_t>(iters),
+                                        static_cast<uint32_t>(wgs), c.stream));
+}
+
 // "fill": buffer 0 is an int32 array; scalars value, count (include/tessera/backend.hpp:151-152,393-396).
 qmm_status run_fill(const LaunchCtx& c) {
   if (!counts(c, 1, 2)) return bad("fill: expects 1 buffer and 2 scalars");
@@ -1204,6 +1218,7 @@ const Entry kTable[] = {
     {"add", run_add},
     {"fill", run_fill},
     {"read_probe", run_read_probe},
+    {"mfma_probe", run_mfma_probe},
     {"rmsnorm", run_rmsnorm},
     {"rope", run_rope},
     {"mrope", run_mrope},

@@ -137,6 +137,10 @@ hipError_t launch_vec_reduce(const float* part, float* c, uint64_t total, uint64
 hipError_t launch_fill_f32(float* dst, float value, uint64_t count, hipStream_t stream);
 hipError_t launch_add(const float* a, const float* b, float* o, uint64_t n, hipStream_t stream);
 hipError_t launch_fill_i32(int32_t* out, int32_t value, uint64_t n, hipStream_t stream);
+// Register-only loop of one matrix instruction (kind 0: fp16 32x32x16, 1: scaled fp8 x fp4 32x32x64, 2: int8
+// 16x16x64), `workgroups` x 4 wavefronts x 4 accumulators x `iters`; out holds workgroups * 256 floats.
+hipError_t launch_mfma_probe(float* out, uint32_t kind, bool random, uint32_t iters, uint32_t workgroups,
+                             hipStream_t stream);
 hipError_t launch_read_probe(const void* src, uint32_t* out, uint64_t bytes, hipStream_t stream);
 hipError_t launch_rmsnorm(const float* x, const float* w, float* y, uint64_t rows, uint64_t cols, float eps,
                           hipStream_t stream);

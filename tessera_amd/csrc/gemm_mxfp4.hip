@@ -481,10 +481,13 @@ __global__ __launch_bounds__(64 * kSkinnyWaves, 4) void mxfp4_a8_skinny_kernel(
 // rows of the product are never stored).
 constexpr uint32_t kStreamMaxRows = 80;
 
-template <int MT>
+// TERMS: the activation rows are fp32 rows split into kMaxTerms E4M3 planes (split_rows_kernel): matrix row
+// t * rows + r is term t of row r, `a8` points at row 0 of plane 0, the planes lie `plane` bytes apart, `m` counts
+// the matrix rows (kMaxTerms * rows), and the store adds a row's terms with their weights 16^-t.
+template <int MT, bool TERMS = false>
 __global__ __launch_bounds__(640) void mxfp4_a8_stream_kernel(
     const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
-    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t rows_wg) {
+    float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t rows_wg, uint64_t plane = 0) {
   typedef float float4v __attribute__((ext_vector_type(4)));
   constexpr uint32_t kBBytes = kStreamMaxRows * 256, kABytes = MT * 16 * 512, kSBytes = kStreamMaxRows * 16;
   constexpr uint32_t kABase = kBBytes, kSBase = kABase + kABytes, kStage = kSBase + kSBytes;
@@ -525,7 +528,13 @@ __global__ __launch_bounds__(640) void mxfp4_a8_stream_kernel(
     const uint32_t blk = wave + i * waves;               // blocks go round the wavefronts
     const uint32_t row = 2u * blk + lane / 32u;
     const uint32_t chunk = (lane % 32u) ^ (row % 16u);
-    a_src[i] = (row < m ? row : m - 1u) * k + chunk * 16u;
+    const uint32_t src_row = row < m ? row : m - 1u;
+    if constexpr (TERMS) {
+      const uint32_t real = m / kMaxTerms, term = src_row / real;
+      a_src[i] = static_cast<uint32_t>(term * plane) + (src_row - term * real) * k + chunk * 16u;
+    } else {
+      a_src[i] = src_row * k + chunk * 16u;
+    }
     a_live[i] = blk < 8u * MT && 2u * blk < m;
     my_dma += a_live[i] ? 1u : 0u;
   }
@@ -619,12 +628,25 @@ __global__ __launch_bounds__(640) void mxfp4_a8_stream_kernel(
     for (int e = 0; e < 4; ++e) red[(((half * tiles + tile) * MT + i) * 4u + e) * 64u + lane] = acc[i][e];
   __syncthreads();
   const uint32_t cols = tiles * 16u;
-  for (uint32_t o = t; o < m * cols; o += blockDim.x) {
-    const uint32_t row = o / cols, col = o % cols;
+  auto tile_sum = [&](uint32_t row, uint32_t col) {
     const uint32_t i = row / 16u, r = row % 16u, ln = (r / 4u) * 16u + col % 16u, tl = col / 16u;
-    const float sum = red[(((0u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln] +
-                      red[(((1u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln];
-    if (col < rows_wg && n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row];
+    return red[(((0u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln] +
+           red[(((1u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln];
+  };
+  if constexpr (TERMS) {
+    const uint32_t real = m / kMaxTerms;
+    for (uint32_t o = t; o < real * cols; o += blockDim.x) {
+      const uint32_t row = o / cols, col = o % cols;
+      float sum = tile_sum((kMaxTerms - 1) * real + row, col);
+#pragma unroll
+      for (int term = kMaxTerms - 2; term >= 0; --term) sum = fmaf(sum, 0.0625f, tile_sum(term * real + row, col));
+      if (col < rows_wg && n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row];
+    }
+  } else {
+    for (uint32_t o = t; o < m * cols; o += blockDim.x) {
+      const uint32_t row = o / cols, col = o % cols;
+      if (col < rows_wg && n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = tile_sum(row, col) * as[row];
+    }
   }
 }
 
@@ -819,6 +841,37 @@ hipError_t launch_mxfp4_a8_gemm_wperm(const uint8_t* a8, const float* as, const 
 }
 
 bool gemm_mxfp4_f32_supported(uint64_t m, uint64_t k) { return m >= 17 && k >= 1024 && gemm_mxfp4_a8_supported(k); }
+
+// 2..16 fp32 rows: the same E4M3 terms through the streamed kernel, eight rows (32 matrix rows) a pass.
+bool gemm_mxfp4_f32_rows_supported(uint64_t m, uint64_t n, uint64_t k) {
+  return m >= 2 && m <= 16 && k % 512 == 0 && k <= (1u << 20) && n >= 16 &&
+         static_cast<uint64_t>(kMaxTerms) * m * k <= 0xFFFFFFFFull;
+}
+size_t gemm_mxfp4_f32_rows_workspace_bytes(uint64_t m, uint64_t k) { return gemm_mxfp4_f32_workspace_bytes(m, k); }
+
+hipError_t launch_mxfp4_f32_rows(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,
+                                 uint32_t k, hipStream_t stream) {
+  uint8_t* planes = static_cast<uint8_t*>(workspace);
+  float* as = reinterpret_cast<float*>(planes + static_cast<size_t>(kMaxTerms) * m * k);
+  uint8_t* need = reinterpret_cast<uint8_t*>(as) + ((static_cast<size_t>(m) * 4 + 255) / 256) * 256;
+  hipLaunchKernelGGL(split_rows_kernel, dim3(m), dim3(256), 0, stream, a, planes, as, need, m, k);
+  const uint32_t rows = stream_rows_per_workgroup(n);
+  const dim3 grid((n + rows - 1u) / rows), block(128u * ((rows + 15u) / 16u));
+  const uint64_t plane = static_cast<uint64_t>(m) * k;
+  for (uint32_t r0 = 0; r0 < m; r0 += 8u) {
+    const uint32_t real = m - r0 < 8u ? m - r0 : 8u;
+    const uint8_t* a8 = planes + static_cast<size_t>(r0) * k;
+    float* out = c + static_cast<size_t>(r0) * n;
+    if (real <= 4u) {
+      hipLaunchKernelGGL((mxfp4_a8_stream_kernel<1, true>), grid, block, 0, stream, a8, as + r0, w, out, kMaxTerms * real, n,
+                         k, rows, plane);
+    } else {
+      hipLaunchKernelGGL((mxfp4_a8_stream_kernel<2, true>), grid, block, 0, stream, a8, as + r0, w, out, kMaxTerms * real, n,
+                         k, rows, plane);
+    }
+  }
+  return hipGetLastError();
+}
 
 size_t gemm_mxfp4_f32_workspace_bytes(uint64_t m, uint64_t k) {
   return static_cast<size_t>(kMaxTerms) * m * k + ((m * 4 + 255) / 256) * 256 + ((m + 255) / 256) * 256;

@@ -824,6 +824,14 @@ qmm_status run_gemm_mxfp4(const LaunchCtx& c) {
                                               static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                               static_cast<uint32_t>(k), c.stream));
   }
+  // 2..16 rows of a matrix large enough to be worth a second launch: the same terms through the streamed
+  // few-row kernel (weights read once per eight rows) instead of four rows a pass on the vector unit.
+  if (m >= 2 && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemm_mxfp4_f32_rows_supported(m, n, k) &&
+      qmm::gemm_mxfp4_f32_rows_workspace_bytes(m, k) <= kDecodeScratchBytes && decode_scratch(c) != nullptr) {
+    return map_hip(qmm::launch_mxfp4_f32_rows(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2),
+                                              decode_scratch(c), static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                              static_cast<uint32_t>(k), c.stream));
+  }
   return map_hip(qmm::launch_mxfp4_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<float>(2),
                                         static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                         static_cast<uint32_t>(k), c.stream));

@@ -92,6 +92,12 @@ hipError_t launch_permute_mxfp4_wmma(const uint8_t* in, uint8_t* out, uint64_t n
 // MXFP4 weights, fp32 activation rows (17 or more): the rows are split into E4M3 terms in the
 // workspace and multiplied on the same scaled MFMA, one pass over K per term.
 bool gemm_mxfp4_f32_supported(uint64_t m, uint64_t k);
+// 2..16 fp32 rows (k a multiple of 512): the same terms through the streamed few-row kernel, the weights read
+// once per eight rows.
+bool gemm_mxfp4_f32_rows_supported(uint64_t m, uint64_t n, uint64_t k);
+size_t gemm_mxfp4_f32_rows_workspace_bytes(uint64_t m, uint64_t k);
+hipError_t launch_mxfp4_f32_rows(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,
+                                 uint32_t k, hipStream_t stream);
 size_t gemm_mxfp4_f32_workspace_bytes(uint64_t m, uint64_t k);
 hipError_t launch_mxfp4_f32_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                                  uint32_t n, uint32_t k, hipStream_t stream);

@@ -183,3 +183,45 @@ def test_full_size_prefill_rows(backend):
     shard = synth.mxfp4_column_shard(w, n, k, 0, n // 2)
     got_shard = mx_gemm(backend, "gemm_mxfp4_batched", a, shard, m, n // 2, k)
     assert np.array_equal(got_shard, got[:, : n // 2])
+
+
+# ---- 2..16 fp32 rows of a large matrix: the same terms through the streamed few-row kernel ----
+@pytest.mark.parametrize("m,n,k", [(2, 4100, 4096), (4, 3300, 5120), (5, 4100, 4096), (8, 3300, 5120), (9, 4100, 4096),
+                                   (13, 1030, 17408), (16, 3300, 5120)])
+@pytest.mark.parametrize("kind", ["bf16", "bf16_outliers", "f32"])
+def test_few_rows_on_the_matrix_cores_match_oracle(backend, m, n, k, kind):
+    """gemm_mxfp4 / gemm_mxfp4_rows with 2..16 rows against 16 M weights or more (the reference's one
+    warp per column with 16 accumulators, src/backends/rocm/rocm_kernels_basic.cpp:1153-1214): always
+    four terms, eight rows a weight pass; same bounds as from 17 rows."""
+    g = synth.rng(2300 * m + n + k)
+    w = synth.mxfp4_weights(g, n, k)
+    a = {"bf16": synth.activations_bf16, "bf16_outliers": synth.activations_bf16_outliers,
+         "f32": synth.activations_f32}[kind](g, m, k)
+    ref = oracle.gemm_mxfp4(a, w, m, n, k, threads=True)
+    for name in ("gemm_mxfp4_rows", "gemm_mxfp4"):
+        got = mx_gemm(backend, name, a, w, m, n, k)
+        check(got, a, w, m, n, k, 4, ref, f"{name} {m}x{n}x{k} {kind}", kind == "bf16_outliers")
+
+
+def test_few_rows_one_hot_and_zero_rows(backend):
+    """One-hot rows of 8- and 12-bit values return single exact products (which lane supplies which
+    block, the term order, the 16^-t weights); a zero row gives zeros; a non-finite element spoils its
+    row only."""
+    g = synth.rng(2400)
+    m, n, k = 6, 4100, 4096
+    w = synth.mxfp4_weights(g, n, k, -20, 20)
+    deq = oracle.dequantize_mxfp4(w, n, k)
+    pos = [0, 31, 32, 777, 4095]
+    vals = np.array([1.0, 1.5, 0.8125, 3.99609375, 2.0 ** -20], np.float32)      # up to 12 significant bits
+    a = np.zeros((m, k), np.float32)
+    for r, (t, v) in enumerate(zip(pos, vals)):
+        a[r, t] = v
+    got = mx_gemm(backend, "gemm_mxfp4_rows", a, w, m, n, k)
+    for r, (t, v) in enumerate(zip(pos, vals)):
+        assert same_bits_zero_sign_free(got[r], deq[:, t] * v), (r, t)
+    assert np.all(got[5] == 0.0)
+    a = synth.activations_f32(g, m, k)
+    a[2, 100] = np.inf
+    a[4, 7] = np.nan
+    got = mx_gemm(backend, "gemm_mxfp4_rows", a, w, m, n, k)
+    assert not np.isfinite(got[[2, 4]]).any() and np.isfinite(got[[0, 1, 3, 5]]).all()

@@ -159,6 +159,17 @@ hipError_t launch_round_bf16(float* x, uint64_t n, hipStream_t stream);
 // weight side (gemv_q4k_rows16.hip).  `workspace` holds the K parts' output regions.
 hipError_t gemv_q4k_rows16_prepare();   // once per device, from qmm_init
 hipError_t moe_q4k_prepare();           // once per device, from qmm_init (moe_q4k.hip)
+
+// Q4_K / Q5_K / Q6_K x a few fp32 rows in one pass over the weights on the int8 matrix cores
+// (gemv_kquant_rows.hip); any m, taken some rows a pass (eight, eight, four).
+hipError_t gemv_kquant_rows_prepare();   // once per device, from qmm_init
+bool gemv_kquant_rows_supported(uint64_t m, uint64_t n, uint64_t k);
+hipError_t launch_q4k_rows_i8(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n, uint32_t k,
+                              hipStream_t stream);
+hipError_t launch_q5k_rows_i8(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n, uint32_t k,
+                              hipStream_t stream);
+hipError_t launch_q6k_rows_i8(const float* a, const uint8_t* w, float* c, uint32_t m, uint32_t n, uint32_t k,
+                              hipStream_t stream);
 bool gemv_q4k_rows16_supported(uint64_t m, uint64_t n, uint64_t k);
 size_t gemv_q4k_rows16_workspace_bytes(uint64_t m, uint64_t n, uint64_t k);
 hipError_t launch_q4k_rows16(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,

@@ -20,8 +20,11 @@
  *     scratch of the decode-sized kernels once; prefill-sized launches (Q4_K/Q5_K/Q6_K from 17
  *     rows, the grouped routed-expert ids) need a workspace, which is the caller's when one was
  *     set with qmm_set_workspace and otherwise a library-owned block that qmm_launch grows on
- *     demand (hipFree + hipMalloc, which synchronises the device and must not happen under stream
- *     capture).  qmm_launch_static never allocates.
+ *     demand with hipMalloc.  A block that a launch has used is never freed (growth allocates a
+ *     new one of at least twice the size and keeps the old until the process ends, so a launch
+ *     recorded into a HIP graph keeps a valid pointer); growth while `stream` is being captured
+ *     returns InvalidArgument with a message: grow before capturing, or set a workspace.
+ *     qmm_launch_static never allocates.
  */
 #ifndef TESSERA_QMM_H_
 #define TESSERA_QMM_H_
@@ -121,6 +124,22 @@ const char* qmm_kernel_name(size_t index);
  * per-slice partial sums for one row of a large Q4_K matrix, else everything in region 0 and
  * zeros in the others), so the reference's reduce pass ("gemm_vec_reduce",
  * "gemm_mxfp4_wmma_reduce") still works.
+ *
+ * Ids and scalars beyond the reference's table (each optional; a caller that never uses them sees
+ * the reference's contracts unchanged):
+ *   - "permute_q4k_rowgroup": buffers In, Out; scalars n, k, rows_per_group (0 = the default, 32;
+ *     at most 64), inverse (0 = GGUF order -> row groups, 1 = back).  The gfx950 counterpart of the
+ *     reference's load-time re-ordering hook (PermuteMxFp4ToWmma, src/core/numerics/quant.cpp:926-954):
+ *     a copy of a Q4_K tensor, same byte count, laid out for the int8 matrix cores.
+ *   - the Q4_K GEMM ids ("gemm_q4k", "_row", "_vec", "_rows{2..5}", "_batched", "_wmma") take one
+ *     more trailing scalar, `layout`: absent or 0 = W is in GGUF order; R = W is the copy made by
+ *     "permute_q4k_rowgroup" with rows_per_group R (as `wperm` selects the re-ordered MXFP4 tensor,
+ *     src/models/qwen3_5/project.cpp:212).  One row runs on the copy directly; more rows have it put
+ *     back into GGUF order in the workspace first (qmm_workspace_bytes counts that).
+ *   - "mfma_probe": buffer Out (workgroups * 256 floats); scalars kind (0 fp16 32x32x16, 1 scaled
+ *     fp8 x fp4 32x32x64, 2 int8 16x16x64), random (0 constant operands, 1 hashed), iterations,
+ *     workgroups.  "read_probe": a plain read of a buffer.  Measurement ids: the matrix-core and the
+ *     read ceiling of the part the library runs on, for the benchmark's roofline.
  */
 qmm_status qmm_launch(qmm_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
                       void* const* buffers, const size_t* buf_bytes, size_t nbuffers,

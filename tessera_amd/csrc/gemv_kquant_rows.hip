@@ -11,17 +11,19 @@
 // what a floating-point kernel spends per weight (scale, min, convert) is spent here per sixteen or
 // thirty-two weights on the integer sums that come back:
 //
-//  * B, 16 weight rows x 64 K: lane (n, g) holds sixteen quants of row n.  Q4_K / Q5_K: the 64 K of
-//    "chunk" c are sub-blocks 2c (low nibbles; lanes g = 0, 1) and 2c + 1 (high nibbles; g = 2, 3),
-//    sixteen consecutive weights per lane.  Q6_K: chunk (half h, p) is quarters p (low nibbles) and
-//    p + 2 (high) of the half's 128 weights; with the two high bits the byte becomes 4 (q - 32), so
-//    the format's offset costs nothing.
+//  * B, 16 weight rows x 64 K: lane (n, g) loads eight bytes of row n and holds sixteen quants: the
+//    low nibbles in its K slots 0..7, the high nibbles in slots 8..15, no byte loaded twice.  Q4_K /
+//    Q5_K: the 64 K of "chunk" c are sub-blocks 2c (low nibbles) and 2c + 1 (high nibbles), bytes
+//    [8g, 8g + 8) of the chunk's 32 per lane.  Q6_K: chunk (half h, p) is quarters p (low nibbles)
+//    and p + 2 (high) of the half's 128 weights; with the two high bits the byte becomes 4 (q - 32),
+//    so the format's offset costs nothing.
 //  * A, 16 matrix rows x 64 K: Q4_K / Q5_K: rows 8 r + 4 par + l = limb l of activation row r
-//    (two rows per instruction) with everything but sub-block parity par zeroed, so that the lane
-//    group that receives matrix rows 4 g'..4 g' + 3 has, for its own weight row, the four limb sums of
-//    ONE sub-block and folds them with that sub-block's 6-bit scale by 24-bit integer multiply-adds.
-//    Q6_K has four scales per 64 K, so all sixteen matrix rows go to one activation row: 4 v + l = limb
-//    l against the sixteen weights of lane group v.
+//    (two rows per instruction) with the K slots of the other sub-block parity zeroed, so that the
+//    lane group that receives matrix rows 4 g'..4 g' + 3 has, for its own weight row, the four limb
+//    sums of ONE sub-block and folds them with that sub-block's 6-bit scale by 24-bit integer
+//    multiply-adds.  Q6_K has four scales per 64 K (per slot half and per pair of lane groups), so
+//    all sixteen matrix rows go to one activation row: 4 v + l = limb l against the sixteen weights
+//    under scale v of the chunk.
 //  * per block and activation row the integer sums meet d, dmin and the block's power of two in fp32:
 //    y += d * T * 2^-sh - dmin * sum_s mn_s S_s (S_s = the activations' sub-block sums), so a one-hot
 //    activation returns the reference's dequantized weight RN(d * sc * q - dmin * mn) bit for bit.
@@ -52,14 +54,9 @@ struct KqArgs {
 };
 
 typedef uint4 uint4_u2 __attribute__((aligned(2)));
+typedef uint2 uint2_u2 __attribute__((aligned(2)));
 __device__ __forceinline__ uint4 load_u4_unaligned(const void* p) { return *reinterpret_cast<const uint4_u2*>(p); }
-
-__device__ __forceinline__ int4v_t mask4(const uint4 v, uint32_t shift, uint32_t mask) {
-  int4v_t r;
-  r[0] = static_cast<int>((v.x >> shift) & mask), r[1] = static_cast<int>((v.y >> shift) & mask);
-  r[2] = static_cast<int>((v.z >> shift) & mask), r[3] = static_cast<int>((v.w >> shift) & mask);
-  return r;
-}
+__device__ __forceinline__ uint2 load_u2_unaligned(const void* p) { return *reinterpret_cast<const uint2_u2*>(p); }
 
 // The four limb sums of one lane times 256^l, as a float (each step exact while the total fits 24
 // bits, which a one-hot row does).
@@ -89,8 +86,8 @@ struct Sub32Format {
   static constexpr uint32_t kMaxWaves[4] = {16u, 12u, 8u, 8u};
   struct Unit {
     uint4 h;
-    uint4 qh;      // Q5_K: the fifth bits of the lane's sixteen weights, one bit per sub-block
-    uint4 q[4];
+    uint2 qh;      // Q5_K: the fifth bits of the lane's eight byte positions, one bit per sub-block
+    uint2 q[4];
   };
   struct Ctx {
     float4 S;      // sums of the four sub-blocks of the lane's parity, of the lane's activation row
@@ -100,9 +97,9 @@ struct Sub32Format {
   // The lane's registers of a unit out of its row's block.
   static __device__ __forceinline__ void read(Unit& u, const uint8_t* blk, uint32_t g) {
     u.h = *reinterpret_cast<const uint4*>(blk);
-    if (kFiveBits) u.qh = *reinterpret_cast<const uint4*>(blk + 16u + 16u * (g & 1u));
+    if (kFiveBits) u.qh = *reinterpret_cast<const uint2*>(blk + 16u + 8u * g);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) u.q[c] = *reinterpret_cast<const uint4*>(blk + kQs + 32u * c + 16u * (g & 1u));
+    for (int c = 0; c < 4; ++c) u.q[c] = *reinterpret_cast<const uint2*>(blk + kQs + 32u * c + 8u * g);
   }
 
   // Activation row r has just been converted into `slot`: the lanes whose matrix rows carry it
@@ -113,11 +110,15 @@ struct Sub32Format {
     const uint32_t ln = lane & 15u, g = lane >> 4;
     const uint32_t apar = (ln >> 2) & 1u;
     if ((ln >> 3) == (r & 1u)) {
-      const bool live = (g >> 1) == apar && r < m;
-      const uint8_t* a = slot + apar * 128u + (g & 1u) * 64u + (ln & 3u) * 16u;
-      const int4v_t zero = {0, 0, 0, 0};
+      // eight weights' limbs in the K slots of the lane's parity, zeros in the other eight
+      const uint8_t* a = slot + apar * 128u + (g >> 1) * 64u + (ln & 3u) * 16u + (g & 1u) * 8u;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) A[c] = live ? *reinterpret_cast<const int4v_t*>(a + c * 256) : zero;
+      for (int c = 0; c < 4; ++c) {
+        uint2 v = *reinterpret_cast<const uint2*>(a + c * 256);
+        if (r >= m) v = make_uint2(0u, 0u);
+        const int x = static_cast<int>(v.x), y = static_cast<int>(v.y);
+        A[c] = apar ? int4v_t{0, 0, x, y} : int4v_t{x, y, 0, 0};
+      }
     }
     if ((g >> 1) == (r & 1u)) {
       if (r < m) {
@@ -133,7 +134,7 @@ struct Sub32Format {
   template <int NA>
   static __device__ __forceinline__ void dot(const Unit& u, const int4v_t (&A)[NA][4], const Ctx (&ctx)[NA],
                                              float (&val)[NA], uint32_t lane) {
-    const uint32_t g = lane >> 4, upper = g >> 1;
+    const uint32_t g = lane >> 4;
     int sc[4];
     float mn[4];
     scales_of_parity(u.h, g & 1u, sc, mn);
@@ -141,13 +142,14 @@ struct Sub32Format {
     int4v_t B[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      B[c] = mask4(u.q[c], 4u * upper, 0x0F0F0F0Fu);
+      constexpr uint32_t kN = 0x0F0F0F0Fu, kOne = 0x01010101u;
+      uint32_t b0 = u.q[c].x & kN, b1 = u.q[c].y & kN, b2 = (u.q[c].x >> 4) & kN, b3 = (u.q[c].y >> 4) & kN;
       if (kFiveBits) {
-        // bit 2c + upper of the fifth-bit bytes -> bit 4
-        const int4v_t hb = mask4(u.qh, 2u * c + upper, 0x01010101u);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) B[c][i] |= hb[i] << 4;
+        // bits 2c (low nibbles' sub-block) and 2c + 1 of the fifth-bit bytes -> bit 4
+        b0 |= ((u.qh.x >> (2 * c)) & kOne) << 4, b1 |= ((u.qh.y >> (2 * c)) & kOne) << 4;
+        b2 |= ((u.qh.x >> (2 * c + 1)) & kOne) << 4, b3 |= ((u.qh.y >> (2 * c + 1)) & kOne) << 4;
       }
+      B[c] = int4v_t{static_cast<int>(b0), static_cast<int>(b1), static_cast<int>(b2), static_cast<int>(b3)};
     }
     const int4v_t zero = {0, 0, 0, 0};
 #pragma unroll
@@ -180,10 +182,10 @@ struct Sub32Format {
 struct Q6KFormat {
   static constexpr uint32_t kBlock = 210u;
   static constexpr int kRowsPerSet = 1;
-  static constexpr uint32_t kMaxWaves[4] = {16u, 12u, 8u, 8u};
+  static constexpr uint32_t kMaxWaves[4] = {16u, 16u, 12u, 8u};
   struct Unit {
-    uint4 ql[4];   // chunk 2h + p: bytes 64h + 32p + 16 (g % 2) ..
-    uint4 qh[2];   // half h: bytes 128 + 32h + 16 (g % 2) ..
+    uint2 ql[4];   // chunk 2h + p: bytes 64h + 32p + 8g ..
+    uint2 qh[2];   // half h: bytes 128 + 32h + 8g ..
     uint4 sc;
     uint32_t d;
   };
@@ -194,9 +196,9 @@ struct Q6KFormat {
   // (blocks of 210 bytes start on even addresses only)
   static __device__ __forceinline__ void read(Unit& u, const uint8_t* blk, uint32_t g) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) u.ql[c] = load_u4_unaligned(blk + 32u * c + 16u * (g & 1u));
+    for (int c = 0; c < 4; ++c) u.ql[c] = load_u2_unaligned(blk + 32u * c + 8u * g);
 #pragma unroll
-    for (int h = 0; h < 2; ++h) u.qh[h] = load_u4_unaligned(blk + 128u + 32u * h + 16u * (g & 1u));
+    for (int h = 0; h < 2; ++h) u.qh[h] = load_u2_unaligned(blk + 128u + 32u * h + 8u * g);
     u.sc = load_u4_unaligned(blk + 192u);
     u.d = *reinterpret_cast<const uint16_t*>(blk + 208u);
   }
@@ -204,12 +206,19 @@ struct Q6KFormat {
   static __device__ __forceinline__ void fetch(int4v_t (&A)[4], Ctx& ctx, const uint8_t* slot, uint32_t r, uint32_t m,
                                                uint32_t lane) {
     const uint32_t ln = lane & 15u, g = lane >> 4;
-    const bool live = (ln >> 2) == g && r < m;
-    // chunk 2h + p, lane group g: quarter p + 2 (g / 2) of half h = sub-block 4h + p + 2 (g / 2)
-    const uint8_t* a = slot + (g >> 1) * 256u + (g & 1u) * 64u + (ln & 3u) * 16u;
-    const int4v_t zero = {0, 0, 0, 0};
+    // Matrix row 4v + l: v = 2 (which half of a lane's K slots: quarter p or p + 2) + (which 16 of the
+    // quarter's 32 weights: lanes g / 2).  Chunk 2h + p: sub-block 4h + p + 2 (v / 2), the lane's eight
+    // weights [8g, 8g + 8) of it.
+    const uint32_t v = ln >> 2;
+    const bool live = (g >> 1) == (v & 1u) && r < m;
+    const uint8_t* a = slot + (v >> 1) * 256u + (g >> 1) * 64u + (ln & 3u) * 16u + (g & 1u) * 8u;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) A[c] = live ? *reinterpret_cast<const int4v_t*>(a + (c >> 1) * 512 + (c & 1) * 128) : zero;
+    for (int c = 0; c < 4; ++c) {
+      uint2 w = *reinterpret_cast<const uint2*>(a + (c >> 1) * 512 + (c & 1) * 128);
+      if (!live) w = make_uint2(0u, 0u);
+      const int x = static_cast<int>(w.x), y = static_cast<int>(w.y);
+      A[c] = (v >> 1) ? int4v_t{0, 0, x, y} : int4v_t{x, y, 0, 0};
+    }
     ctx.f = 0.0f;
     if (r < m) {
       // An infinity shows in the block's shift, a NaN (which the largest-magnitude search skips) in
@@ -237,17 +246,20 @@ struct Q6KFormat {
     int4v_t B[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const uint4 ql = u.ql[c], qh = u.qh[c >> 1];
-      const uint32_t l4[4] = {ql.x, ql.y, ql.z, ql.w}, h4[4] = {qh.x, qh.y, qh.z, qh.w};
+      const uint32_t l2[2] = {u.ql[c].x, u.ql[c].y}, h2[2] = {u.qh[c >> 1].x, u.qh[c >> 1].y};
       // nibble -> bits 2..5 (a rotation: what crosses a byte border is masked away), the two high bits
-      // of quarter p + 2 upper -> bits 6..7, and the sign flipped: the byte is 4 (q - 32)
-      const uint32_t rot_n = upper ? 2u : 30u;
-      const uint32_t rot_h = (26u + 2u * ((c & 1) + 2u * upper)) & 31u;   // bit 2 quarter -> bit 6
+      // of the quarter (p for the low nibbles, p + 2 for the high ones) -> bits 6..7, and the sign
+      // flipped: the byte is 4 (q - 32)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t nib = __builtin_amdgcn_alignbit(l4[i], l4[i], rot_n) & 0x3C3C3C3Cu;
-        const uint32_t hi = __builtin_amdgcn_alignbit(h4[i], h4[i], rot_h) & 0xC0C0C0C0u;
-        B[c][i] = static_cast<int>((nib | hi) ^ 0x80808080u);
+      for (int half = 0; half < 2; ++half) {
+        const uint32_t rot_n = half ? 2u : 30u;
+        const uint32_t rot_h = (26u + 2u * ((c & 1) + 2u * half)) & 31u;   // bit 2 quarter -> bit 6
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const uint32_t nib = __builtin_amdgcn_alignbit(l2[i], l2[i], rot_n) & 0x3C3C3C3Cu;
+          const uint32_t hi = __builtin_amdgcn_alignbit(h2[i], h2[i], rot_h) & 0xC0C0C0C0u;
+          B[c][2 * half + i] = static_cast<int>((nib | hi) ^ 0x80808080u);
+        }
       }
     }
     const int4v_t zero = {0, 0, 0, 0};
@@ -378,13 +390,19 @@ constexpr uint32_t kq_max_waves() {
 template <class F, int NA>
 bool kq_plan(uint32_t n, uint32_t nblk, uint32_t cus, KqPlan& pl) {
   const uint32_t wmax = kq_max_waves<F, NA>();
-  // wavefronts: the count from eight up that leaves the fewest idle block turns, the larger on a tie
-  uint32_t best = wmax, best_waste = ~0u;
-  for (uint32_t w = wmax; w >= 8u; --w) {
-    const uint32_t turns = (nblk + w - 1u) / w, waste = turns * w - nblk;
-    if (waste < best_waste) best = w, best_waste = waste;
+  // Wavefronts: a CU runs them on four SIMDs (wavefront w on SIMD w % 4) and the launch lasts as
+  // long as the SIMD with the most blocks to work through, so the count that makes that number
+  // smallest, the larger count on a tie (more wavefronts hide more of each other's waits).
+  uint32_t best = wmax, best_cost = ~0u;
+  for (uint32_t w = wmax; w >= 4u; --w) {
+    uint32_t cost = 0;
+    for (uint32_t simd = 0; simd < 4u; ++simd) {
+      uint32_t blocks = 0;
+      for (uint32_t wv = simd; wv < w; wv += 4u) blocks += wv < nblk ? (nblk - wv + w - 1u) / w : 0u;
+      cost = blocks > cost ? blocks : cost;
+    }
+    if (cost < best_cost) best = w, best_cost = cost;
   }
-  if (nblk < 8u) best = nblk < 4u ? 4u : nblk;
   // equal shares of the rows, one workgroup a CU; more rounds of workgroups when a share's tables
   // would not fit the LDS
   for (uint32_t rounds = 1; rounds <= 64u; ++rounds) {

@@ -170,6 +170,7 @@ constexpr uint64_t kMxfp4GemmMinRows = 17;   // below: the VALU GEMV passes, exa
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KRows16MinRows = 3;      // from here the 16x16x32 kernel, below the 4x4x4 one
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
+constexpr uint64_t kQ4KRowsI8MaxK = 5120;      // up to here the int8 one-pass kernel leads for 2..4 rows
 
 qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
                       uint64_t k, uint64_t f16_from) {
@@ -188,6 +189,16 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
       if (st != QMM_OK) return st;
     }
     return QMM_OK;
+  }
+  // 2..4 rows against weight rows of up to 5120: one pass on the int8 matrix cores with the activations
+  // as 8-bit limbs, whole K per workgroup, nothing left for a second launch to add up.  Measured
+  // against the kernels below, 2 / 3 / 4 rows: 17408 x 5120 14.6 / 17.3 / 17.8 against 17.7 / 17.7 / 18.4 us,
+  // 4096 x 4096 6.6 / 7.8 / 8.2 against 8.1 / 9.3, 32768 x 1024 two rows 7.8 against 11.7; longer rows
+  // go the other way (8192 x 8192 two rows 15.6 against 14.2, 5120 x 17408 three rows 26 against 19.4).
+  if (m >= 2 && m <= 4 && k <= kQ4KRowsI8MaxK && n * k >= kQ4KFewRowsMinWeights &&
+      qmm::gemv_kquant_rows_supported(m, n, k)) {
+    return map_hip(qmm::launch_q4k_rows_i8(a, w, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                                           static_cast<uint32_t>(k), s));
   }
   // 3..16 rows of a large matrix: one pass over the weights on the 16x16x32 MFMA.
   // (two rows as well when the weight rows are long: 5120 x 17408 20.5 against 24.8 us on the

@@ -1,6 +1,8 @@
 """GPU parity of the one-pass several-row kernels for Q5_K and Q6_K (int8 matrix cores, weights read
 once for up to eight resp. four activation rows) against the oracle: decode exactness through one-hot
-rows, every row count of a pass and across passes, ragged and tiny shapes, the 27B FFN shapes."""
+rows, every row count of a pass and across passes, ragged and tiny shapes, the 27B FFN shapes.  The
+same kernel takes Q4_K with 2..4 rows on matrices of 16 M weights or more whose rows are at most 5120
+long: covered at the end."""
 import numpy as np
 import pytest
 
@@ -145,3 +147,51 @@ def test_rows_ids_and_split_regions(backend, fmt):
         got = backend.CopyD2H(dc, dtype=np.float32).reshape(split, rows, n)
         assert rel_err(got.sum(axis=0), ref_fn(a, w, rows, n, k)) <= TOL
         assert np.all(got[1:] == 0.0)
+
+
+Q4K_SHAPES = [(3300, 5120), (8200, 2048), (16390, 1024), (4099, 4096), (17408, 5120)]
+
+
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("n,k", Q4K_SHAPES[:4])
+def test_q4k_one_hot_rows_bit_exact(backend, m, n, k):
+    g = synth.rng(7800 + m + n)
+    w = synth.q4k_weights(g, n, k)
+    deq = oracle.dequantize_q4k(w).reshape(n, k).astype(np.float64)
+    for scale in (1.0, 2.0 ** -100, 2.0 ** 90, -(2.0 ** -3)):
+        pos = [int(t) for t in g.integers(0, k, m)]
+        a = synth.one_hot_rows(k, pos) * np.float32(scale)
+        got = gemm(backend, "gemm_q4k_batched", a, w, m, n, k)
+        for r, t in enumerate(pos):
+            assert same_bits_zero_sign_free(got[r], (deq[:, t] * scale).astype(np.float32)), (m, n, k, scale, r, t)
+
+
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("n,k", Q4K_SHAPES)
+def test_q4k_rows_match_oracle(backend, m, n, k):
+    g = synth.rng(7900 + m + n)
+    w = synth.q4k_weights(g, n, k)
+    a = synth.activations_f32(g, m, k)
+    ref = oracle.gemm_q4k(a, w, m, n, k, threads=True)
+    for name in ("gemm_q4k", "gemm_q4k_batched"):
+        got = gemm(backend, name, a, w, m, n, k)
+        assert rel_err(got, ref) <= TOL and rms_err(got, ref) < 5e-5, (name, m, n, k, rel_err(got, ref), rms_err(got, ref))
+
+
+def test_q4k_non_finite_values_stay_in_their_row(backend):
+    g = synth.rng(7950)
+    m, n, k = 3, 3300, 5120
+    w = synth.q4k_weights(g, n, k).reshape(n, -1)
+    bad_rows = [5, 1700, 3299]
+    for r in bad_rows:
+        w[r, 144 * (r % 20):144 * (r % 20) + 2] = np.array([0x00, 0x7C], np.uint8)   # d = +inf
+    w = w.reshape(-1)
+    a = synth.activations_f32(g, m, k)
+    a[1, 4000] = np.nan
+    got = gemm(backend, "gemm_q4k_batched", a, w, m, n, k)
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = oracle.gemm_q4k(a[[0, 2]], w, 2, n, k, threads=True)
+    good = [r for r in range(n) if r not in bad_rows]
+    assert not np.isfinite(got[1]).any()
+    assert not np.isfinite(got[:, bad_rows]).any()
+    assert rel_err(got[[0, 2]][:, good], ref[:, good]) <= TOL

@@ -170,7 +170,7 @@ constexpr uint64_t kMxfp4GemmMinRows = 17;   // below: the VALU GEMV passes, exa
 constexpr uint64_t kQ4KFewRowsMinWeights = uint64_t{16} << 20;
 constexpr uint64_t kQ4KRows16MinRows = 3;      // from here the 16x16x32 kernel, below the 4x4x4 one
 constexpr uint64_t kQ4KFewRowsMaxK = 262144;   // its activation operand must fit the decode scratch
-constexpr uint64_t kQ4KRowsI8MaxK = 5120;      // up to here the int8 one-pass kernel leads for 2..4 rows
+constexpr uint64_t kQ4KRowsI8MaxK = 5120;      // up to here the int8 one-pass kernel leads for two rows
 
 qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, float* c, uint64_t m, uint64_t n,
                       uint64_t k, uint64_t f16_from) {
@@ -190,12 +190,13 @@ qmm_status q4k_matmul(const LaunchCtx& ctx, const float* a, const uint8_t* w, fl
     }
     return QMM_OK;
   }
-  // 2..4 rows against weight rows of up to 5120: one pass on the int8 matrix cores with the activations
+  // Two rows against weight rows of up to 5120: one pass on the int8 matrix cores with the activations
   // as 8-bit limbs, whole K per workgroup, nothing left for a second launch to add up.  Measured
-  // against the kernels below, 2 / 3 / 4 rows: 17408 x 5120 14.6 / 17.3 / 17.8 against 17.7 / 17.7 / 18.4 us,
-  // 4096 x 4096 6.6 / 7.8 / 8.2 against 8.1 / 9.3, 32768 x 1024 two rows 7.8 against 11.7; longer rows
-  // go the other way (8192 x 8192 two rows 15.6 against 14.2, 5120 x 17408 three rows 26 against 19.4).
-  if (m >= 2 && m <= 4 && k <= kQ4KRowsI8MaxK && n * k >= kQ4KFewRowsMinWeights &&
+  // against the kernels below: 17408 x 5120 14.6..16.6 against 17.7..18.2 us, 4096 x 4096 6.6 against
+  // 8.1, 32768 x 1024 7.8 against 11.7; longer rows go the other way (8192 x 8192 15.6 against 14.2),
+  // and three and four rows are level with the 16x16x32 kernel (17.3 / 17.8 against 17.7 / 18.4 us in
+  // one harness, 19.5 against 18.9 in another), so they stay there.
+  if (m == 2 && k <= kQ4KRowsI8MaxK && n * k >= kQ4KFewRowsMinWeights &&
       qmm::gemv_kquant_rows_supported(m, n, k)) {
     return map_hip(qmm::launch_q4k_rows_i8(a, w, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                            static_cast<uint32_t>(k), s));

@@ -1,8 +1,8 @@
 """GPU parity of the one-pass several-row kernels for Q5_K and Q6_K (int8 matrix cores, weights read
 once for up to eight resp. four activation rows) against the oracle: decode exactness through one-hot
 rows, every row count of a pass and across passes, ragged and tiny shapes, the 27B FFN shapes.  The
-same kernel takes Q4_K with 2..4 rows on matrices of 16 M weights or more whose rows are at most 5120
-long: covered at the end."""
+same kernel takes Q4_K with two rows on matrices of 16 M weights or more whose rows are at most 5120
+long: covered at the end (three and four rows of those shapes run beside it for comparison)."""
 import numpy as np
 import pytest
 

@@ -732,7 +732,7 @@ qmm_status q5k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, ui
     return kquant_prefill(c, 176, m, n, k, split);
   }
   // Several rows: one pass over the weights for up to eight of them on the int8 matrix cores
-  // (17408 x 5120: 2 rows 20.5 us against 30.3 on a multiply-add pass per row, 8 rows 32 against 121).
+  // (17408 x 5120: 2 rows 17.6 us against 30.3 on a multiply-add pass per row, 8 rows 31 against 121).
   const bool one_pass = m >= 2 && qmm::gemv_kquant_rows_supported(m, n, k);
   const auto launch = one_pass ? qmm::launch_q5k_rows_i8 : qmm::launch_q5k_gemv;
   qmm_status st = map_hip(launch(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, static_cast<uint32_t>(m),
@@ -785,8 +785,8 @@ qmm_status q6k_matmul(const LaunchCtx& c, uint64_t m, uint64_t n, uint64_t k, ui
     return kquant_prefill(c, 210, m, n, k, split);
   }
   // From three rows: one pass over the weights for up to four of them on the int8 matrix cores
-  // (17408 x 5120: 4 rows 40 us against 52 on multiply-add passes of two rows, 8 rows 78 against 103;
-  // two rows stay on the multiply-add pass, 26 against 38 us).
+  // (17408 x 5120: 4 rows 32 us against 52 on multiply-add passes of two rows, 8 rows 61 against 103;
+  // two rows stay on the multiply-add pass, 26 against 29 us).
   const bool one_pass = m >= 3 && qmm::gemv_kquant_rows_supported(m, n, k);
   const auto launch = one_pass ? qmm::launch_q6k_rows_i8 : qmm::launch_q6k_gemv;
   qmm_status st = map_hip(launch(c.ptr<const float>(0), c.ptr<const uint8_t>(1), out, static_cast<uint32_t>(m),

@@ -136,6 +136,11 @@ const char* qmm_kernel_name(size_t index);
  *     "permute_q4k_rowgroup" with rows_per_group R (as `wperm` selects the re-ordered MXFP4 tensor,
  *     src/models/qwen3_5/project.cpp:212).  One row runs on the copy directly; more rows have it put
  *     back into GGUF order in the workspace first (qmm_workspace_bytes counts that).
+ *   - "gemm_mxfp4", "gemm_mxfp4_rows", "gemm_mxfp4_batched" keep the reference's contract (fp32
+ *     activations, no activation quantization).  Where they run on the matrix cores (2..16 rows of a
+ *     matrix of 16 M weights or more with k a multiple of 512; from 17 rows with k a multiple of 128)
+ *     each activation is carried to 16 significant bits under its row's largest magnitude (exactly,
+ *     when it has no more); one row and the small shapes carry the full fp32 value.
  *   - "mfma_probe": buffer Out (workgroups * 256 floats); scalars kind (0 fp16 32x32x16, 1 scaled
  *     fp8 x fp4 32x32x64, 2 int8 16x16x64), random (0 constant operands, 1 hashed), iterations,
  *     workgroups.  "read_probe": a plain read of a buffer.  Measurement ids: the matrix-core and the

@@ -167,7 +167,10 @@ __global__ __launch_bounds__(768) void q4k_rows16_kernel(R16Args p) {
 
   // ---- the activations are requested first: a wavefront's loads return in order, so behind the
   // weight ring they would wait for it.  Requested by hand, because the compiler's own waits count
-  // only the loads it knows of and would wait for the ring as well.
+  // only the loads it knows of and would wait for the ring as well.  Between the request and the
+  // wait below nothing names xv, and the kernel must not spill (a copy of a register that its load
+  // has not filled yet would go unnoticed): tests/test_kernel_resources.py compiles this file and
+  // fails on any scratch use.
   float4_t xv[BW * MT][8];
 #pragma unroll
   for (int jb = 0; jb < BW; ++jb)

@@ -611,6 +611,11 @@ def main():
         per = len(plans_[0]) if only is None else len(only)
         return median(replay_times_ms(graph, reps * per)) * 1e3 / reps
 
+    # ... and that fused launch followed by the down projection over its row-group copy
+    fused_rg_plans = [[plan[0], (kern, KernelLaunch(grid_x=K_HID // 8, buffers=[wrap(x_ff), wrap(dn), wrap(y_down)],
+                                                    scalars=[1, K_HID, N_FF, 1, RG]))]
+                      for plan, dn in zip(fused_plans, rg_down)]
+    us_fused_rg_step = timed_plans_us(fused_rg_plans, args.steps)
     us_fused_step = timed_plans_us(fused_plans, args.steps)
     us_fused_gate_up = timed_plans_us(fused_plans, args.steps, only=(0,))
     us_down_split = timed_plans_us(split_plans, args.steps)
@@ -660,6 +665,10 @@ def main():
             "pct_hbm_peak": round(100 * fused_step_bytes / us_fused_step / 1e3 / HBM_PEAK_GBS, 1),
             "gate_up_us": round(us_fused_gate_up, 3), "gate_up_GBps": round(fused_bytes / us_fused_gate_up / 1e3, 1),
             "gate_up_frac_hbm": round(fused_bytes / us_fused_gate_up / 1e3 / HBM_PEAK_GBS, 4)},
+        "decode_step_fused_gate_up_down_as_rowgroup_copy": {
+            "what": "ffn_gate_up_silu_q4k + gemm_q4k_vec over the down projection's row-group copy",
+            "us_per_step": round(us_fused_rg_step, 3), "GBps": round(fused_step_bytes / us_fused_rg_step / 1e3, 1),
+            "pct_hbm_peak": round(100 * fused_step_bytes / us_fused_rg_step / 1e3 / HBM_PEAK_GBS, 1)},
         "down_split4_plus_reduce_us": round(us_down_split, 3),
     }
     if not args.no_also:

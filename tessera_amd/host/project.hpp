@@ -42,6 +42,10 @@ struct ProjectState {
   std::unique_ptr<Buffer> gemv_part;                     // split-K partials
   std::unique_ptr<Buffer> wmma_a, wmma_as;               // E4M3 codes and row scales of A
   std::map<const Buffer*, std::unique_ptr<Buffer>> mxfp4_wref;
+  // Q4_K tensors kept as this backend's load-time row-group copy (RowGroupCopyQ4K below): the rows
+  // per group that the Q4_K GEMM ids then receive as their trailing `layout` scalar -- what the
+  // reference does for MXFP4 with PermuteMxFp4ToWmma and `wperm` (src/models/qwen3_5/project.cpp:212).
+  std::map<const Buffer*, std::uint64_t> q4k_layout;
   // The reference splits K to fill a 96-CU card; this backend takes any split (it writes the
   // whole result to region 0) but gains nothing from it, so the default passes split = 1.
   bool honour_reference_split = false;
@@ -82,7 +86,8 @@ inline Expected<void> Grow(Backend& backend, std::unique_ptr<Buffer>& slot, std:
 // "_vec" / "_rows{R}" launch with the split-K partials and the reduce pass
 // (ProjectGemvDevice / ProjectGemvRowsDevice, src/models/qwen3_5/internal.hpp:104-199).
 inline Expected<void> ProjectGemvDevice(Backend& backend, ProjectState& h, const Kernel& gemm, const Buffer& a,
-                                        const Buffer& w, Buffer& out, std::size_t m, std::size_t n, std::size_t k) {
+                                        const Buffer& w, Buffer& out, std::size_t m, std::size_t n, std::size_t k,
+                                        std::uint64_t layout = 0) {
   const std::size_t split = h.honour_reference_split ? GemmVecSplit(m * n, k) : 1;
   const Buffer* dst = &out;
   if (split > 1) {
@@ -94,6 +99,7 @@ inline Expected<void> ProjectGemvDevice(Backend& backend, ProjectState& h, const
   l.grid_y = static_cast<std::uint32_t>(split);
   l.buffers = {&a, &w, dst};
   l.scalars = {m, n, k, split};
+  if (layout != 0) l.scalars.push_back(layout);
   if (auto ok = backend.LaunchKernel(gemm, l); !ok) return ok;
   if (split > 1) {
     auto reduce = CachedKernel(backend, h, "gemm_vec_reduce");
@@ -105,6 +111,25 @@ inline Expected<void> ProjectGemvDevice(Backend& backend, ProjectState& h, const
     return backend.LaunchKernel(**reduce, r);
   }
   return {};
+}
+
+// Load-time hook, not a reference function: replaces a Q4_K tensor of n rows x k by this backend's
+// row-group copy (same byte count) and remembers its layout, so that every later ProjectBatch on
+// the returned buffer passes the `layout` scalar.  A loader would call it for the tensors it wants
+// kept that way (one row against long weight rows gains: 5120 x 17408 13.3 against 14.0 us) right
+// after upload and drop the GGUF-order buffer.  Returns UnsupportedFeature where the backend has no such id.
+inline Expected<std::unique_ptr<Buffer>> RowGroupCopyQ4K(Backend& backend, ProjectState& h, const Buffer& w,
+                                                         std::size_t n, std::size_t k, std::uint64_t rows_per_group = 32) {
+  auto perm = CachedKernel(backend, h, "permute_q4k_rowgroup");
+  if (!perm) return unexpected(perm.error());
+  auto copy = backend.AllocateBuffer(w.Size());
+  if (!copy) return unexpected(copy.error());
+  KernelLaunch l;
+  l.buffers = {&w, copy->get()};
+  l.scalars = {n, k, rows_per_group, 0};
+  if (auto ok = backend.LaunchKernel(**perm, l); !ok) return unexpected(ok.error());
+  h.q4k_layout[copy->get()] = rows_per_group;
+  return std::move(*copy);
 }
 
 // MXFP4 weights with per-token E4M3 activations (ProjectWmma,
@@ -177,10 +202,14 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
     // columns, the batched id from kTiledMinRows, the vec id otherwise.
     if (k % 256 != 0) return unexpected(StatusCode::InvalidArgument);
     const std::string fmt = dtype == DType::Q4K ? "q4k" : dtype == DType::Q5K ? "q5k" : "q6k";
+    std::uint64_t layout = 0;
+    if (dtype == DType::Q4K) {
+      if (auto it = h.q4k_layout.find(&w); it != h.q4k_layout.end()) layout = it->second;
+    }
     if (m >= 2 && m <= 4) {
       auto rows = CachedKernel(backend, h, "gemm_" + fmt + "_rows" + std::to_string(m));
       if (!rows) return unexpected(rows.error());
-      return ProjectGemvDevice(backend, h, **rows, a, w, out, m, n, k);
+      return ProjectGemvDevice(backend, h, **rows, a, w, out, m, n, k, layout);
     }
     if (m >= kGemmWmmaMinRows && n >= kGemmWmmaMinCols) {
       auto wmma = CachedKernel(backend, h, "gemm_" + fmt + "_wmma");
@@ -190,6 +219,7 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
       l.grid_y = static_cast<std::uint32_t>((m + 127) / 128);
       l.buffers = {&a, &w, &out};
       l.scalars = {m, n, k};
+      if (layout != 0) l.scalars.push_back(layout);
       return backend.LaunchKernel(**wmma, l);
     }
     if (m >= kTiledMinRows) {
@@ -199,11 +229,12 @@ inline Expected<void> ProjectBatch(Backend& backend, ProjectState& h, DType dtyp
       l.grid_x = static_cast<std::uint32_t>(((m + 31) / 32) * ((n + 31) / 32));
       l.buffers = {&a, &w, &out};
       l.scalars = {m, n, k};
+      if (layout != 0) l.scalars.push_back(layout);
       return backend.LaunchKernel(**tiled, l);
     }
     auto vec = CachedKernel(backend, h, "gemm_" + fmt + "_vec");
     if (!vec) return unexpected(vec.error());
-    return ProjectGemvDevice(backend, h, **vec, a, w, out, m, n, k);
+    return ProjectGemvDevice(backend, h, **vec, a, w, out, m, n, k, layout);
   }
   return unexpected(StatusCode::UnsupportedFeature);
 }

@@ -94,6 +94,7 @@ struct Case {
   bool reference_split;
   double rel_tol, rms_tol;     // see tests/test_gpu_q4k.py, test_gpu_gemm_q4k.py, test_gpu_gemm_mxfp4.py, test_gpu_gemm_mxfp4_f32.py
   bool fp8_prefill = false;    // ProjectState::mxfp4_fp8_prefill: E4M3 activations beyond 16 rows (reference: QDQ + GemmMxFp4Ref)
+  bool row_groups = false;     // the Q4_K tensor is replaced by RowGroupCopyQ4K's copy before the projection
 };
 const Case kCases[] = {
     {"q4k decode m=1 (gemm_q4k_vec)", DType::Q4K, 1, 640, 5120, false, 1e-3, 1e-3},
@@ -102,6 +103,9 @@ const Case kCases[] = {
     {"q4k m=7 (gemm_q4k_vec, m rows)", DType::Q4K, 7, 129, 1280, false, 1e-3, 1e-3},
     {"q4k m=16 (gemm_q4k_batched)", DType::Q4K, 16, 256, 1024, false, 1e-3, 1e-3},
     {"q4k prefill m=192 (gemm_q4k_wmma, fp16 MFMA)", DType::Q4K, 192, 320, 1024, false, 1.0, 4e-3},
+    {"q4k decode m=1 over the load-time row-group copy (layout scalar)", DType::Q4K, 1, 650, 5120, false, 1e-3, 1e-3, false, true},
+    {"q4k verify m=3 over the row-group copy, reference split-K", DType::Q4K, 3, 333, 2048, true, 1e-3, 1e-3, false, true},
+    {"q4k prefill m=192 over the row-group copy (gemm_q4k_wmma)", DType::Q4K, 192, 320, 1024, false, 1.0, 4e-3, false, true},
     {"q6k decode m=1, reference split-K (gemm_q6k_vec)", DType::Q6K, 1, 640, 5120, true, 1e-3, 1e-3},
     {"q6k verify m=3 (gemm_q6k_rows3)", DType::Q6K, 3, 333, 2048, true, 1e-3, 1e-3},
     {"q6k prefill m=192 (gemm_q6k_wmma, fp16 MFMA)", DType::Q6K, 192, 320, 1024, false, 1.0, 4e-3},
@@ -211,6 +215,15 @@ int main(int argc, char** argv) {
     }
     auto da = Upload(*backend, a);
     auto dw = Upload(*backend, w);
+    if (c.row_groups) {
+      auto copy = RowGroupCopyQ4K(*backend, h, *dw, c.n, c.k);
+      if (!copy) {
+        std::printf("FAIL %s: RowGroupCopyQ4K status %d (%s)\n", c.name, static_cast<int>(copy.error()), backend->LastError());
+        ++failed;
+        continue;
+      }
+      dw = std::move(*copy);     // the loader drops the GGUF-order buffer
+    }
     auto out = backend->AllocateBuffer(c.m * c.n * 4);
     auto st = ProjectBatch(*backend, h, c.dtype, *da, *dw, **out, c.m, c.n, c.k);
     backend->Synchronize();

@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per gate/up launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # same counter reads for a device copy of known size (profiles/q4k_gemv_m1_ffn27b_hbm_traffic.md);
 # a counter figure, not measured by this script.
-GATE_UP_HBM_TRAFFIC_BYTES = 50_510_000
+GATE_UP_HBM_TRAFFIC_BYTES = 50_530_000
 N_FF, K_HID = 17408, 5120
 
 

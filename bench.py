@@ -51,6 +51,26 @@ def vulkan_on_cpu_probe():
     return found, all(found.values())
 
 
+def gpu_clocks():
+    """Core and memory clocks as rocm-smi reports them right after the timed region (best effort: None
+    where the tool is missing or refuses an ordinary user)."""
+    import re
+    import shutil
+    import subprocess
+
+    smi = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    try:
+        out = subprocess.run([smi, "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    clocks = {}
+    for name in ("sclk", "mclk", "fclk"):
+        m = re.search(name + r" clock level: \S+: \((\d+)Mhz\)", out)
+        if m:
+            clocks[name + "_MHz"] = int(m.group(1))
+    return clocks or None
+
+
 def cpu_baseline(seconds_budget=12.0):
     """Reference host GEMM (GemmQ4KRef restated in oracle/qmm_oracle.c) on configs[0]:
     Q4_K GEMV M=1, N=K=5120, on this host's cores.  The Vulkan-on-lavapipe baseline the
@@ -542,6 +562,7 @@ def main():
     ms = median(ts)
     value = step_bytes * args.steps / (ms * 1e-3) / 1e9
     us_down = us_down_rg if rg_headline else us_down_gguf
+    clocks = gpu_clocks()
 
     # Roofline of the dominant kernel: the gate/up GEMV alone, back to back over the layers.
     ts_gu = timed_ms(only=(0, 1))
@@ -635,7 +656,7 @@ def main():
                                "copy (permute_q4k_rowgroup, q4k_i8_gemv_kernel)") if rg_headline else
                               "all three tensors in GGUF order (gemv_kernel<Q4KPairCodec>)",
                    "layers_rotated": args.layers, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
-                   "untimed_graph_launches_before_timing": 1,
+                   "untimed_graph_launches_before_timing": 1, "clocks_after_timing": clocks,
                    "timing": "median of single replays of one HIP graph of `steps` steps; ms_per_step_min is the fastest replay"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),

@@ -31,9 +31,10 @@
 // Work split.  A workgroup owns a range of weight rows over all of K (so nothing is left to add up
 // in a second launch) and its wavefronts share the blocks of K: wavefront w takes blocks w, w + W, ...
 // and, for each, walks the workgroup's 16-row tiles with the block's A operands in registers and two
-// units of weights in flight.  It converts the activations of its own blocks itself, one block ahead
-// of use, into a private LDS area; the sums of a tile live in a private LDS table; the wavefronts meet
-// once, at the end, and their tables are added in wavefront order.  The row ranges are equal shares
+// units of weights in flight.  It asks for the activations of its next block one block ahead and turns
+// them into limbs when it gets there, row by row through one private 1 KB LDS slot; the sums of a
+// tile live in a private LDS table; the wavefronts meet once, at the end, and their tables are added
+// in wavefront order.  The row ranges are equal shares
 // of the matrix whether or not that is a multiple of 16 rows: the CUs then stream equal byte counts,
 // which is what sets the duration of a launch that is bound by memory.
 

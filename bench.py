@@ -268,7 +268,7 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
             (torch.randint(0, 2, (nn * kk,), dtype=torch.uint8, device=dev) << 7)
         scales = torch.rand(nn, dtype=torch.float32, device=dev) * 1e-4 + 1e-5
         wl = [codes] + [codes.clone() for _ in range(3)]
-        for m in (1, 4):
+        for m in (1, 4, 16):
             x = to_dev(synth.activations_f32(g, m, kk))
             y = torch.empty(m * nn, dtype=torch.float32, device=dev)
             launches = [(kf8, KernelLaunch(grid_x=(m * nn + 255) // 256, buffers=[wrap(x), wrap(w), wrap(scales), wrap(y)],

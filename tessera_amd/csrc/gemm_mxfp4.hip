@@ -689,6 +689,172 @@ __global__ __launch_bounds__(640) void mxfp4_a8_stream_kernel(
   }
 }
 
+// ---- FP8 E4M3 weights x a few fp32 rows ("gemm_fp8", 2..16 rows), streamed the same way -----------
+// The weights are E4M3 already, so they are the B operand of the same matrix instruction as they are
+// stored (format E4M3 instead of E2M1, unit block scale); the fp32 rows go in as E4M3 terms as above
+// (matrix row t * rows + r = term t of row r), the weight row's fp32 scale and the activation row's
+// power of two are applied at the store.  A weight row is 512 bytes a stage instead of 256, so a
+// direct load moves two rows and the workgroup's share of rows is sized to the LDS it leaves: the
+// stage ring is dynamic shared memory of 3 x (rows x 512 + MT x 8192) bytes.
+template <int MT>
+__global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
+    const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
+    const float* __restrict__ wscale, float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t rows_wg,
+    uint64_t plane) {
+  typedef float float4v __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const uint32_t kABase = rows_wg * 512u, kStage = kABase + MT * 16u * 512u;
+
+  const uint32_t t = threadIdx.x, lane = t & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const uint32_t tiles = (rows_wg + 15u) / 16u;           // blockDim.x = 128 * tiles
+  const uint32_t l16 = lane & 15u, kq = lane >> 4;
+  const uint32_t n0 = blockIdx.x * rows_wg;
+  const uint8_t* w_tile = w + static_cast<size_t>(n0) * k;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) uint8_t*)lds));
+
+  // Direct loads of one stage.  Weight block L (1 KB) = rows 2L, 2L+1, thirty-two 16-byte chunks
+  // each: lane p fetches row 2L + p/32, chunk (p%32) ^ (row%16); wavefront v brings blocks 4v..4v+3
+  // (rows 8v..8v+7).  Activation blocks as in the kernel above.
+  constexpr int kAMax = 4 * MT;
+  const uint32_t waves = 2u * tiles;
+  uint32_t b_src[4], a_src[kAMax];
+  bool b_live[4], a_live[kAMax];
+  uint32_t my_dma = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t blk = wave * 4u + i;
+    const uint32_t row = 2u * blk + lane / 32u;
+    const uint32_t chunk = (lane % 32u) ^ (row % 16u);
+    b_src[i] = (n0 + row < n ? row : n - 1u - n0) * k + chunk * 16u;
+    b_live[i] = 2u * blk < rows_wg;
+    my_dma += b_live[i] ? 1u : 0u;
+  }
+#pragma unroll
+  for (int i = 0; i < kAMax; ++i) {
+    const uint32_t blk = wave + i * waves;
+    const uint32_t row = 2u * blk + lane / 32u;
+    const uint32_t chunk = (lane % 32u) ^ (row % 16u);
+    const uint32_t src_row = row < m ? row : m - 1u;
+    const uint32_t real = m / kMaxTerms, term = src_row / real;
+    a_src[i] = static_cast<uint32_t>(term * plane) + (src_row - term * real) * k + chunk * 16u;
+    a_live[i] = blk < 8u * MT && 2u * blk < m;
+    my_dma += a_live[i] ? 1u : 0u;
+  }
+  auto issue_stage = [&](uint32_t stage_off, uint32_t st) {
+    const uint32_t stage = lds_base + stage_off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (b_live[i]) direct_load16(w_tile + st * 512u, b_src[i], stage + (wave * 4u + i) * 1024u);
+    }
+#pragma unroll
+    for (int i = 0; i < kAMax; ++i) {
+      if (a_live[i]) direct_load16(a8 + st * 512u, a_src[i], stage + kABase + (wave + i * waves) * 1024u);
+    }
+  };
+  // Everything but the stage requested last has landed, for every wavefront.
+  auto publish = [&]() {
+    switch (my_dma) {
+      case 0: asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory"); break;
+      case 7: asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory"); break;
+      case 8: asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory"); break;
+      case 9: asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory"); break;
+      case 10: asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory"); break;
+      case 11: asm volatile("s_waitcnt vmcnt(11) lgkmcnt(0)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory"); break;
+    }
+    asm volatile("s_barrier" ::: "memory");
+  };
+  static_assert(4 + kAMax <= 12, "publish() counts up to twelve loads a stage");
+
+  // This wavefront's share of a stage: column tile `tile`, K-steps 2*half and 2*half + 1.
+  const uint32_t tile = wave % tiles, half = wave / tiles;
+  const uint32_t b_row = tile * 16u + l16;
+  float4v acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const uint32_t stages = k / 512u;
+  issue_stage(0, 0);
+  issue_stage(kStage, stages > 1 ? 1 : 0);
+  publish();
+  uint32_t rd = 0, nx = kStage, fill = 2 * kStage;
+  for (uint32_t st = 0; st < stages; ++st) {
+    issue_stage(fill, st + 2 < stages ? st + 2 : stages - 1u);
+    const uint8_t* stage = lds + rd;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t step = half * 2u + u;
+      // a row of the last, partly filled tile past the workgroup's rows reads what follows the weight
+      // area (activation bytes, still inside the stage): its column is never stored
+      const uint8_t* brow = stage + b_row * 512u;
+      const uint4 blo = *reinterpret_cast<const uint4*>(brow + (((step * 8u + kq) ^ l16) * 16u));
+      const uint4 bhi = *reinterpret_cast<const uint4*>(brow + (((step * 8u + 4u + kq) ^ l16) * 16u));
+      const int8v_t bf = int8v_t{static_cast<int>(blo.x), static_cast<int>(blo.y), static_cast<int>(blo.z),
+                                 static_cast<int>(blo.w), static_cast<int>(bhi.x), static_cast<int>(bhi.y),
+                                 static_cast<int>(bhi.z), static_cast<int>(bhi.w)};
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const uint8_t* arow = stage + kABase + (i * 16u + l16) * 512u;
+        const uint4 lo = *reinterpret_cast<const uint4*>(arow + (((step * 8u + kq) ^ l16) * 16u));
+        const uint4 hi = *reinterpret_cast<const uint4*>(arow + (((step * 8u + 4u + kq) ^ l16) * 16u));
+        const int8v_t af = int8v_t{static_cast<int>(lo.x), static_cast<int>(lo.y), static_cast<int>(lo.z),
+                                   static_cast<int>(lo.w), static_cast<int>(hi.x), static_cast<int>(hi.y),
+                                   static_cast<int>(hi.z), static_cast<int>(hi.w)};
+        // both operands E4M3 (cbsz 0, blgp 0) with unit E8M0 scales
+        acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf, acc[i], 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+      }
+    }
+    publish();
+    const uint32_t done = rd;
+    rd = nx;
+    nx = fill;
+    fill = done;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive its workgroup
+  __syncthreads();
+
+  // Sum the two wavefronts of each tile (stage memory is free now), add a row's terms, scale.
+  float* red = reinterpret_cast<float*>(lds);          // [half][tile][MT][4][64]
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[(((half * tiles + tile) * MT + i) * 4u + e) * 64u + lane] = acc[i][e];
+  __syncthreads();
+  const uint32_t cols = tiles * 16u;
+  auto tile_sum = [&](uint32_t row, uint32_t col) {
+    const uint32_t i = row / 16u, r = row % 16u, ln = (r / 4u) * 16u + col % 16u, tl = col / 16u;
+    return red[(((0u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln] +
+           red[(((1u * tiles + tl) * MT + i) * 4u + r % 4u) * 64u + ln];
+  };
+  const uint32_t real = m / kMaxTerms;
+  for (uint32_t o = t; o < real * cols; o += blockDim.x) {
+    const uint32_t row = o / cols, col = o % cols;
+    float sum = tile_sum((kMaxTerms - 1) * real + row, col);
+#pragma unroll
+    for (int term = kMaxTerms - 2; term >= 0; --term) sum = fmaf(sum, 0.0625f, tile_sum(term * real + row, col));
+    if (col < rows_wg && n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row] * wscale[n0 + col];
+  }
+}
+
+// Rows a workgroup of the FP8 kernel owns: the matrix shared out evenly over the CUs, in multiples
+// of four rows, as many as the stage ring leaves room for (80 with one activation tile, 72 with two).
+uint32_t fp8_rows_per_workgroup(uint32_t n, uint32_t max_rows) {
+  const uint32_t cus = static_cast<uint32_t>(num_cus());
+  const uint32_t rounds = (n + max_rows * cus - 1u) / (max_rows * cus);
+  const uint32_t share = (n + cus * rounds - 1u) / (cus * rounds);
+  uint32_t rows = (share + 3u) / 4u * 4u;
+  rows = rows < 16u ? 16u : (rows > max_rows ? max_rows : rows);
+  return rows;
+}
+
 // Rows a workgroup of the streamed kernel owns: the matrix shared out evenly over the CUs, as few
 // rounds of workgroups as 80 rows each allow, in multiples of the four rows a direct load moves.
 uint32_t stream_rows_per_workgroup(uint32_t n) {
@@ -961,6 +1127,48 @@ hipError_t launch_mxfp4_f32_gemm(const float* a, const uint8_t* w, float* c, voi
   uint8_t* need = reinterpret_cast<uint8_t*>(as) + ((static_cast<size_t>(m) * 4 + 255) / 256) * 256;
   launch_split_rows(a, planes, as, need, m, k, stream);
   launch_tiles(planes, as, w, c, m, n, k, need, false, stream);
+  return hipGetLastError();
+}
+
+// ---- "gemm_fp8" with 2..16 fp32 rows on the scaled matrix instruction ---------------------------------
+bool gemm_fp8_f32_rows_supported(uint64_t m, uint64_t n, uint64_t k) {
+  return m >= 2 && m <= 16 && k % 512 == 0 && k <= (1u << 20) && n >= 16 && n <= 0x7FFFFFFFull &&
+         static_cast<uint64_t>(kMaxTerms) * m * k <= 0xFFFFFFFFull;
+}
+
+hipError_t gemm_fp8_f32_rows_prepare() {
+  const int lim = 160 * 1024 - 1024;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_terms_stream_kernel<1>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_terms_stream_kernel<2>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+}
+
+// Workspace as for the MXFP4 rows: the term planes, the rows' powers of two, the term counts.
+hipError_t launch_fp8_f32_rows(const float* a, const uint8_t* w, const float* wscale, float* c, void* workspace,
+                               uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
+  uint8_t* planes = static_cast<uint8_t*>(workspace);
+  float* as = reinterpret_cast<float*>(planes + static_cast<size_t>(kMaxTerms) * m * k);
+  uint8_t* need = reinterpret_cast<uint8_t*>(as) + ((static_cast<size_t>(m) * 4 + 255) / 256) * 256;
+  launch_split_rows(a, planes, as, need, m, k, stream);
+  const uint64_t plane = static_cast<uint64_t>(m) * k;
+  for (uint32_t r0 = 0; r0 < m; r0 += 8u) {
+    const uint32_t real = m - r0 < 8u ? m - r0 : 8u;
+    const uint32_t mt = real <= 4u ? 1u : 2u;
+    const uint32_t rows = fp8_rows_per_workgroup(n, mt == 1u ? 80u : 72u);
+    const dim3 grid((n + rows - 1u) / rows), block(128u * ((rows + 15u) / 16u));
+    const uint32_t lds = 3u * (rows * 512u + mt * 16u * 512u);
+    const uint8_t* a8 = planes + static_cast<size_t>(r0) * k;
+    float* out = c + static_cast<size_t>(r0) * n;
+    if (mt == 1u) {
+      hipLaunchKernelGGL((fp8_terms_stream_kernel<1>), grid, block, lds, stream, a8, as + r0, w, wscale, out,
+                         kMaxTerms * real, n, k, rows, plane);
+    } else {
+      hipLaunchKernelGGL((fp8_terms_stream_kernel<2>), grid, block, lds, stream, a8, as + r0, w, wscale, out,
+                         kMaxTerms * real, n, k, rows, plane);
+    }
+  }
   return hipGetLastError();
 }
 

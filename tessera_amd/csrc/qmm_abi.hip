@@ -1017,6 +1017,14 @@ qmm_status run_gemm_fp8(const LaunchCtx& c) {
       !c.fits(2, static_cast<u128>(n) * 4) || !c.fits(3, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_fp8: a buffer is smaller than m, n, k require");
   }
+  // 2..16 rows of a large matrix: the weights through the matrix cores as they are (E4M3 operand), the
+  // fp32 rows as E4M3 terms, weights read once per eight rows (gemm_mxfp4.hip).
+  if (m >= 2 && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemm_fp8_f32_rows_supported(m, n, k) &&
+      qmm::gemm_mxfp4_f32_rows_workspace_bytes(m, k) <= kDecodeScratchBytes && decode_scratch(c) != nullptr) {
+    return map_hip(qmm::launch_fp8_f32_rows(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
+                                            c.ptr<float>(3), decode_scratch(c), static_cast<uint32_t>(m),
+                                            static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
+  }
   return map_hip(qmm::launch_fp8_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
                                       c.ptr<float>(3), static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                                       static_cast<uint32_t>(k), c.stream));
@@ -1346,7 +1354,7 @@ qmm_status qmm_init(int device) {
     g_static_scratch[device] = p;
   }
   if ((e = qmm::gemv_q4k_rows16_prepare()) != hipSuccess || (e = qmm::moe_q4k_prepare()) != hipSuccess ||
-      (e = qmm::gemv_kquant_rows_prepare()) != hipSuccess) {
+      (e = qmm::gemv_kquant_rows_prepare()) != hipSuccess || (e = qmm::gemm_fp8_f32_rows_prepare()) != hipSuccess) {
     g_device = -1;
     return map_hip(e);
   }

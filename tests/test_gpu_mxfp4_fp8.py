@@ -9,7 +9,7 @@ import pytest
 
 import oracle
 from tessera_amd import StatusCode, StatusError, synth
-from util import rel_err, rms_err, run, same_bits, same_bits_zero_sign_free, strict_rel_err
+from util import norm_err, rel_err, rms_err, run, same_bits, same_bits_zero_sign_free, strict_rel_err
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -107,7 +107,12 @@ def test_fp8_many_output_columns(backend, n, k, m):
     run(backend, "gemm_fp8", [da, dw, ds, dc], [m, n, k], grid=((m * n + 255) // 256, 1, 1))
     backend.Synchronize()
     got = backend.CopyD2H(dc, dtype=np.float32).reshape(m, n)
-    assert rel_err(got, ref) <= TOL, rel_err(got, ref)
+    if m >= 2 and n * k >= 1 << 24 and k % 512 == 0:
+        # several rows of 16 M weights or more go through the matrix cores: that path's bound
+        # (tests/test_gpu_fp8_rows.py)
+        assert rms_err(got, ref) <= 2e-4 and norm_err(got, ref) <= 2e-5, (rms_err(got, ref), norm_err(got, ref))
+    else:
+        assert rel_err(got, ref) <= TOL, rel_err(got, ref)
 
 
 def quant_inputs(g, rows, cols):

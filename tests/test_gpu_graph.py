@@ -1,7 +1,8 @@
 """A decode step recorded into a HIP graph: every replay must give what the eager launches give,
 also after the inputs changed and after eager work (including a prefill-sized call, which grows
 the library's workspace) ran between the replays.  The ids recorded here are the ones that use
-library-owned scratch: the few-row Q4_K path and the fused feed-forward id (decode scratch)."""
+library-owned scratch: the few-row Q4_K path, the fused feed-forward id, and MXFP4 / FP8 weights with four
+fp32 rows (their E4M3 terms), all in the decode scratch."""
 import numpy as np
 import pytest
 import torch
@@ -26,6 +27,11 @@ def test_recorded_decode_step_replays_like_eager(backend):
     y4 = torch.empty(4 * n, device=dev)
     f1 = torch.empty(n, device=dev)
     f4 = torch.empty(4 * n, device=dev)
+    mx = to_dev(synth.mxfp4_weights(g, n, k, -8, -4))
+    codes_h, scales_h = synth.fp8_weights(g, n, k)
+    codes, scales = to_dev(codes_h), to_dev(scales_h)
+    m4, e4 = torch.empty(4 * n, device=dev), torch.empty(4 * n, device=dev)
+    km, k8 = backend.LoadKernel("gemm_mxfp4_rows"), backend.LoadKernel("gemm_fp8")
     kq, kb, kf = backend.LoadKernel("gemm_q4k_vec"), backend.LoadKernel("gemm_q4k_batched"), backend.LoadKernel("ffn_gate_up_silu_q4k")
 
     def step():
@@ -33,6 +39,9 @@ def test_recorded_decode_step_replays_like_eager(backend):
         backend.LaunchKernel(kb, KernelLaunch(grid_x=(4 * n + 7) // 8, buffers=[wrap(x4), wrap(gate), wrap(y4)], scalars=[4, n, k]))
         backend.LaunchKernel(kf, KernelLaunch(grid_x=(n + 7) // 8, buffers=[wrap(x1), wrap(gate), wrap(up), wrap(f1)], scalars=[1, n, k]))
         backend.LaunchKernel(kf, KernelLaunch(grid_x=(4 * n + 7) // 8, buffers=[wrap(x4), wrap(gate), wrap(up), wrap(f4)], scalars=[4, n, k]))
+        backend.LaunchKernel(km, KernelLaunch(grid_x=(4 * n + 7) // 8, buffers=[wrap(x4), wrap(mx), wrap(m4)], scalars=[4, n, k]))
+        backend.LaunchKernel(k8, KernelLaunch(grid_x=(4 * n + 255) // 256, buffers=[wrap(x4), wrap(codes), wrap(scales), wrap(e4)],
+                                              scalars=[4, n, k]))
 
     def set_inputs(seed):
         a = synth.activations_f32(synth.rng(seed), 5, k)
@@ -57,22 +66,23 @@ def test_recorded_decode_step_replays_like_eager(backend):
     kw = backend.LoadKernel("gemm_q4k_wmma")
     for replay, seed in enumerate((1, 2, 3, 2)):
         a = set_inputs(seed)
-        for t in (y1, y4, f1, f4):
+        for t in (y1, y4, f1, f4, m4, e4):
             t.fill_(float("nan"))
         graph.replay()
         torch.cuda.synchronize()
-        got = [t.cpu().numpy().copy() for t in (y1, y4, f1, f4)]
-        for t in (y1, y4, f1, f4):
+        got = [t.cpu().numpy().copy() for t in (y1, y4, f1, f4, m4, e4)]
+        for t in (y1, y4, f1, f4, m4, e4):
             t.fill_(float("nan"))
         step()                            # the same work eagerly
         torch.cuda.synchronize()
-        eager = [t.cpu().numpy().copy() for t in (y1, y4, f1, f4)]
+        eager = [t.cpu().numpy().copy() for t in (y1, y4, f1, f4, m4, e4)]
         for gv, ev in zip(got, eager):
             assert np.array_equal(gv.view(np.uint32), ev.view(np.uint32)), (replay, seed)
         if replay == 0:                   # and the eager result is right
             assert rel_err(eager[0], oracle.gemm_q4k(a[0], gate_h, 1, n, k)) < 1e-3
             assert rel_err(eager[1], oracle.gemm_q4k(a[1:], gate_h, 4, n, k)) < 1e-3
             assert rel_err(eager[3], oracle.ffn_gate_up_silu_q4k(a[1:], gate_h, up_h, 4, n, k)) < 1e-3
+            assert rel_err(eager[5], oracle.gemm_fp8(a[1:], codes_h, scales_h, 4, n, k)) < 2e-3
         backend.LaunchKernel(kw, KernelLaunch(grid_x=n // 64 + 1, grid_y=1, buffers=[wrap(xb), wrap(gate), wrap(yb)],
                                               scalars=[big_m, n, k]))
         torch.cuda.synchronize()

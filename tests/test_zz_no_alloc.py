@@ -66,6 +66,24 @@ def test_static_scratch_up_product_that_does_not_fit_the_decode_room(backend):
         assert np.array_equal(_bits(got), _bits(ref)), m
 
 
+def test_static_scratch_fp32_rows_on_the_scaled_matrix_instruction(backend):
+    """MXFP4 and FP8 weights with 2..16 fp32 rows keep the rows' E4M3 terms in scratch; 12 rows then 3."""
+    g = synth.rng(4246)
+    n, k = 4100, 4096
+    mx = backend.Upload(synth.mxfp4_weights(g, n, k, -8, -4))
+    codes, scales = synth.fp8_weights(g, n, k)
+    dcodes, dscales = backend.Upload(codes), backend.Upload(scales)
+    for m in (12, 3):
+        da = backend.Upload(synth.activations_f32(g, m, k))
+        out = backend.AllocateBuffer(4 * m * n)
+        ref, got = _both(backend, "gemm_mxfp4_rows", [da, mx, out], out, [m, n, k], (m * n + 7) // 8)
+        assert np.isfinite(ref).all()
+        assert np.array_equal(_bits(got), _bits(ref)), ("gemm_mxfp4_rows", m)
+        ref, got = _both(backend, "gemm_fp8", [da, dcodes, dscales, out], out, [m, n, k], (m * n + 255) // 256)
+        assert np.isfinite(ref).all()
+        assert np.array_equal(_bits(got), _bits(ref)), ("gemm_fp8", m)
+
+
 def test_static_scratch_grouped_experts_then_smaller_chunk(backend):
     g = synth.rng(4243)
     experts, hidden, inter, top_k = 16, 512, 256, 4

@@ -310,7 +310,7 @@ struct Q4KPairCodec {
   template <int R>
   struct X {
     float lo[R][32];
-    float hi[R][32];  // activation / 16
+    float hi[R][32];
     float slo[R];
     float shi[R];
     uint32_t sh;
@@ -354,7 +354,6 @@ struct Q4KPairCodec {
       for (int i = 0; i < 32; ++i) {
         sl += x.lo[r][i];
         sh += x.hi[r][i];
-        x.hi[r][i] *= 0.0625f;
       }
       x.slo[r] = sl;
       x.shi[r] = sh;
@@ -406,7 +405,8 @@ struct Q4KPairCodec {
         al = fmaf(x.lo[r][4 * wi + 3], static_cast<float>(l13[1]), al);
         ah = fmaf(x.hi[r][4 * wi + 3], static_cast<float>(h13[1]), ah);
       }
-      const float t1 = fmaf(scb, ah, sca * al);
+      // the high nibbles were masked in place (16 q): their 1/16 goes to the sub-block's scale, exactly
+      const float t1 = fmaf(scb * 0.0625f, ah, sca * al);
       const float t2 = fmaf(mnb, x.shi[r], mna * x.slo[r]);
       out[r] = fmaf(d24, t1, -(dmin * t2));
     }
@@ -1181,6 +1181,7 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   // barrier.  Otherwise each wavefront reduces its (at most two) rows itself, which is faster
   // when rows are long.
   constexpr int kMaxWaves = MAXT / kWave;
+  static_assert(MAXT <= 1024, "the row of a thread is found by a float division that is exact up to 1024");
   __shared__ float red[2][D][P][R][LR ? 1 : kMaxWaves];
   // Rows whose chunk count is a multiple of 16: an aligned run of 16 lanes never straddles two
   // rows, so one four-step sum per run replaces the two masked six-step sums over the wavefront,
@@ -1196,7 +1197,9 @@ __global__ __launch_bounds__(MAXT) void gemv_kernel(typename Codec::Args args, f
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const uint32_t slots = P * cpr;
   const bool valid = t < slots;
-  const uint32_t prow = valid ? t / cpr : 0u;
+  // t / cpr for t < 1024: (t + 1/2) / cpr is at least 1 / (2 cpr) away from an integer, far more than
+  // the reciprocal's rounding moves it
+  const uint32_t prow = valid ? static_cast<uint32_t>((static_cast<float>(t) + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(cpr))) : 0u;
   const uint32_t chunk = valid ? t - prow * cpr : 0u;
 
   // Which of the P rows this wavefront's lanes belong to: at most two when a row has at least

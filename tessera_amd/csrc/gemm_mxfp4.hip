@@ -696,14 +696,19 @@ __global__ __launch_bounds__(640) void mxfp4_a8_stream_kernel(
 // power of two are applied at the store.  A weight row is 512 bytes a stage instead of 256, so a
 // direct load moves two rows and the workgroup's share of rows is sized to the LDS it leaves: the
 // stage ring is dynamic shared memory of 3 x (rows x 512 + MT x 8192) bytes.
-template <int MT>
+// BLOCK ("gemm_fp8_block"): `wscale` is one fp32 per 128 x 128 block of W, (n/128) x (k/128) row-major.
+// An instruction covers 128 of K, i.e. exactly one block column, so its sum is taken by itself and
+// multiplied by the block's scale before it joins the accumulator; the four scales a weight row
+// needs per stage come with the stage (one more 16-byte direct load per row, rows x 16 more bytes).
+template <int MT, bool BLOCK = false>
 __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
     const uint8_t* __restrict__ a8, const float* __restrict__ as, const uint8_t* __restrict__ w,
     const float* __restrict__ wscale, float* __restrict__ c, uint32_t m, uint32_t n, uint32_t k, uint32_t rows_wg,
     uint64_t plane) {
   typedef float float4v __attribute__((ext_vector_type(4)));
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  const uint32_t kABase = rows_wg * 512u, kStage = kABase + MT * 16u * 512u;
+  const uint32_t kABase = rows_wg * 512u, kSBase = kABase + MT * 16u * 512u;
+  const uint32_t kStage = kSBase + (BLOCK ? rows_wg * 16u : 0u);
 
   const uint32_t t = threadIdx.x, lane = t & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -711,6 +716,7 @@ __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
   const uint32_t l16 = lane & 15u, kq = lane >> 4;
   const uint32_t n0 = blockIdx.x * rows_wg;
   const uint8_t* w_tile = w + static_cast<size_t>(n0) * k;
+  const uint8_t* s_base = reinterpret_cast<const uint8_t*>(wscale);
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (__attribute__((address_space(3))) uint8_t*)lds));
 
@@ -742,6 +748,14 @@ __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
     a_live[i] = blk < 8u * MT && 2u * blk < m;
     my_dma += a_live[i] ? 1u : 0u;
   }
+  // BLOCK: lane p < 8 of wavefront v fetches the stage's four scales (16 bytes) of row 8v + p
+  const bool s_live = BLOCK && 8u * wave < rows_wg;
+  uint32_t s_src = 0;
+  if (BLOCK) {
+    const uint32_t row = 8u * wave + (lane & 7u);
+    s_src = ((n0 + row < n ? n0 + row : n - 1u) / 128u) * (k / 128u) * 4u;
+    my_dma += s_live ? 1u : 0u;
+  }
   auto issue_stage = [&](uint32_t stage_off, uint32_t st) {
     const uint32_t stage = lds_base + stage_off;
 #pragma unroll
@@ -752,6 +766,9 @@ __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
     for (int i = 0; i < kAMax; ++i) {
       if (a_live[i]) direct_load16(a8 + st * 512u, a_src[i], stage + kABase + (wave + i * waves) * 1024u);
     }
+    // (rows_wg is a multiple of four, not of eight: the lanes past it stay out, their bytes would land in
+    // the next stage)
+    if (s_live && lane < 8u && 8u * wave + lane < rows_wg) direct_load16(s_base + st * 16u, s_src, stage + kSBase + wave * 128u);
   };
   // Everything but the stage requested last has landed, for every wavefront.
   auto publish = [&]() {
@@ -768,11 +785,12 @@ __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
       case 9: asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory"); break;
       case 10: asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory"); break;
       case 11: asm volatile("s_waitcnt vmcnt(11) lgkmcnt(0)" ::: "memory"); break;
-      default: asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory"); break;
+      case 12: asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(13) lgkmcnt(0)" ::: "memory"); break;
     }
     asm volatile("s_barrier" ::: "memory");
   };
-  static_assert(4 + kAMax <= 12, "publish() counts up to twelve loads a stage");
+  static_assert(4 + kAMax + 1 <= 13, "publish() counts up to thirteen loads a stage");
 
   // This wavefront's share of a stage: column tile `tile`, K-steps 2*half and 2*half + 1.
   const uint32_t tile = wave % tiles, half = wave / tiles;
@@ -809,7 +827,16 @@ __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
                                    static_cast<int>(lo.w), static_cast<int>(hi.x), static_cast<int>(hi.y),
                                    static_cast<int>(hi.z), static_cast<int>(hi.w)};
         // both operands E4M3 (cbsz 0, blgp 0) with unit E8M0 scales
-        acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf, acc[i], 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+        if constexpr (BLOCK) {
+          const float4v d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf, float4v{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0,
+                                                                              0x7F7F7F7F, 0, 0x7F7F7F7F);
+          const uint32_t s_row = b_row < rows_wg ? b_row : rows_wg - 1u;      // (a column past the rows is never stored)
+          const float bs = *reinterpret_cast<const float*>(stage + kSBase + s_row * 16u + step * 4u);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][e] = fmaf(bs, d[e], acc[i][e]);
+        } else {
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf, acc[i], 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+        }
       }
     }
     publish();
@@ -840,7 +867,9 @@ __global__ __launch_bounds__(640) void fp8_terms_stream_kernel(
     float sum = tile_sum((kMaxTerms - 1) * real + row, col);
 #pragma unroll
     for (int term = kMaxTerms - 2; term >= 0; --term) sum = fmaf(sum, 0.0625f, tile_sum(term * real + row, col));
-    if (col < rows_wg && n0 + col < n) c[static_cast<size_t>(row) * n + n0 + col] = sum * as[row] * wscale[n0 + col];
+    if (col < rows_wg && n0 + col < n) {
+      c[static_cast<size_t>(row) * n + n0 + col] = BLOCK ? sum * as[row] : sum * as[row] * wscale[n0 + col];
+    }
   }
 }
 
@@ -1138,16 +1167,20 @@ bool gemm_fp8_f32_rows_supported(uint64_t m, uint64_t n, uint64_t k) {
 
 hipError_t gemm_fp8_f32_rows_prepare() {
   const int lim = 160 * 1024 - 1024;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_terms_stream_kernel<1>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, lim);
-  if (e != hipSuccess) return e;
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_terms_stream_kernel<2>),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+  const void* kernels[4] = {reinterpret_cast<const void*>(fp8_terms_stream_kernel<1>),
+                            reinterpret_cast<const void*>(fp8_terms_stream_kernel<2>),
+                            reinterpret_cast<const void*>(fp8_terms_stream_kernel<1, true>),
+                            reinterpret_cast<const void*>(fp8_terms_stream_kernel<2, true>)};
+  for (const void* kern : kernels) {
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 // Workspace as for the MXFP4 rows: the term planes, the rows' powers of two, the term counts.
 hipError_t launch_fp8_f32_rows(const float* a, const uint8_t* w, const float* wscale, float* c, void* workspace,
-                               uint32_t m, uint32_t n, uint32_t k, hipStream_t stream) {
+                               uint32_t m, uint32_t n, uint32_t k, bool block_scales, hipStream_t stream) {
   uint8_t* planes = static_cast<uint8_t*>(workspace);
   float* as = reinterpret_cast<float*>(planes + static_cast<size_t>(kMaxTerms) * m * k);
   uint8_t* need = reinterpret_cast<uint8_t*>(as) + ((static_cast<size_t>(m) * 4 + 255) / 256) * 256;
@@ -1156,17 +1189,22 @@ hipError_t launch_fp8_f32_rows(const float* a, const uint8_t* w, const float* ws
   for (uint32_t r0 = 0; r0 < m; r0 += 8u) {
     const uint32_t real = m - r0 < 8u ? m - r0 : 8u;
     const uint32_t mt = real <= 4u ? 1u : 2u;
-    const uint32_t rows = fp8_rows_per_workgroup(n, mt == 1u ? 80u : 72u);
+    // rows of a workgroup: what the stage ring leaves room for (a row takes 512 bytes of weights a stage,
+    // 16 more with block scales)
+    const uint32_t rows = fp8_rows_per_workgroup(n, mt == 1u ? 80u : (block_scales ? 68u : 72u));
     const dim3 grid((n + rows - 1u) / rows), block(128u * ((rows + 15u) / 16u));
-    const uint32_t lds = 3u * (rows * 512u + mt * 16u * 512u);
+    const uint32_t lds = 3u * (rows * (block_scales ? 528u : 512u) + mt * 16u * 512u);
     const uint8_t* a8 = planes + static_cast<size_t>(r0) * k;
     float* out = c + static_cast<size_t>(r0) * n;
-    if (mt == 1u) {
-      hipLaunchKernelGGL((fp8_terms_stream_kernel<1>), grid, block, lds, stream, a8, as + r0, w, wscale, out,
-                         kMaxTerms * real, n, k, rows, plane);
+    const uint32_t mrows = kMaxTerms * real;
+    if (mt == 1u && !block_scales) {
+      hipLaunchKernelGGL((fp8_terms_stream_kernel<1>), grid, block, lds, stream, a8, as + r0, w, wscale, out, mrows, n, k, rows, plane);
+    } else if (!block_scales) {
+      hipLaunchKernelGGL((fp8_terms_stream_kernel<2>), grid, block, lds, stream, a8, as + r0, w, wscale, out, mrows, n, k, rows, plane);
+    } else if (mt == 1u) {
+      hipLaunchKernelGGL((fp8_terms_stream_kernel<1, true>), grid, block, lds, stream, a8, as + r0, w, wscale, out, mrows, n, k, rows, plane);
     } else {
-      hipLaunchKernelGGL((fp8_terms_stream_kernel<2>), grid, block, lds, stream, a8, as + r0, w, wscale, out,
-                         kMaxTerms * real, n, k, rows, plane);
+      hipLaunchKernelGGL((fp8_terms_stream_kernel<2, true>), grid, block, lds, stream, a8, as + r0, w, wscale, out, mrows, n, k, rows, plane);
     }
   }
   return hipGetLastError();

@@ -1023,7 +1023,7 @@ qmm_status run_gemm_fp8(const LaunchCtx& c) {
       qmm::gemm_mxfp4_f32_rows_workspace_bytes(m, k) <= kDecodeScratchBytes && decode_scratch(c) != nullptr) {
     return map_hip(qmm::launch_fp8_f32_rows(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
                                             c.ptr<float>(3), decode_scratch(c), static_cast<uint32_t>(m),
-                                            static_cast<uint32_t>(n), static_cast<uint32_t>(k), c.stream));
+                                            static_cast<uint32_t>(n), static_cast<uint32_t>(k), false, c.stream));
   }
   return map_hip(qmm::launch_fp8_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
                                       c.ptr<float>(3), static_cast<uint32_t>(m), static_cast<uint32_t>(n),
@@ -1040,6 +1040,14 @@ qmm_status run_gemm_fp8_block(const LaunchCtx& c) {
   if (!c.fits(0, static_cast<u128>(m) * k * 4) || !c.fits(1, static_cast<u128>(n) * k) ||
       !c.fits(2, static_cast<u128>(n / 128) * (k / 128) * 4) || !c.fits(3, static_cast<u128>(m) * n * 4)) {
     return bad("gemm_fp8_block: a buffer is smaller than m, n, k require");
+  }
+  // 2..16 rows of a large matrix: the matrix cores as for gemm_fp8, an instruction's sum (128 of K: one
+  // block column) times the block's scale
+  if (m >= 2 && m <= 16 && n * k >= kQ4KFewRowsMinWeights && qmm::gemm_fp8_f32_rows_supported(m, n, k) &&
+      qmm::gemm_mxfp4_f32_rows_workspace_bytes(m, k) <= kDecodeScratchBytes && decode_scratch(c) != nullptr) {
+    return map_hip(qmm::launch_fp8_f32_rows(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
+                                            c.ptr<float>(3), decode_scratch(c), static_cast<uint32_t>(m),
+                                            static_cast<uint32_t>(n), static_cast<uint32_t>(k), true, c.stream));
   }
   return map_hip(qmm::launch_fp8_block_gemv(c.ptr<const float>(0), c.ptr<const uint8_t>(1), c.ptr<const float>(2),
                                             c.ptr<float>(3), static_cast<uint32_t>(m), static_cast<uint32_t>(n),

@@ -98,12 +98,14 @@ bool gemm_mxfp4_f32_rows_supported(uint64_t m, uint64_t n, uint64_t k);
 size_t gemm_mxfp4_f32_rows_workspace_bytes(uint64_t m, uint64_t k);
 hipError_t launch_mxfp4_f32_rows(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m, uint32_t n,
                                  uint32_t k, hipStream_t stream);
-// "gemm_fp8" with 2..16 fp32 rows: E4M3 weights as the matrix instruction's other operand, the rows as
-// E4M3 terms; same workspace as gemm_mxfp4_f32_rows_workspace_bytes.  prepare() once per device.
+// "gemm_fp8" / "gemm_fp8_block" with 2..16 fp32 rows: E4M3 weights as the matrix instruction's other
+// operand, the rows as E4M3 terms; same workspace as gemm_mxfp4_f32_rows_workspace_bytes.  `wscale`:
+// one fp32 per weight row, or (block_scales) one per 128 x 128 block, (n/128) x (k/128).  prepare()
+// once per device.
 bool gemm_fp8_f32_rows_supported(uint64_t m, uint64_t n, uint64_t k);
 hipError_t gemm_fp8_f32_rows_prepare();
 hipError_t launch_fp8_f32_rows(const float* a, const uint8_t* w, const float* wscale, float* c, void* workspace,
-                               uint32_t m, uint32_t n, uint32_t k, hipStream_t stream);
+                               uint32_t m, uint32_t n, uint32_t k, bool block_scales, hipStream_t stream);
 size_t gemm_mxfp4_f32_workspace_bytes(uint64_t m, uint64_t k);
 hipError_t launch_mxfp4_f32_gemm(const float* a, const uint8_t* w, float* c, void* workspace, uint32_t m,
                                  uint32_t n, uint32_t k, hipStream_t stream);

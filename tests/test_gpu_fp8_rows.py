@@ -31,7 +31,8 @@ def fp8_gemm(backend, a, codes, scales, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(2, 4100, 4096), (3, 8200, 2048), (4, 3300, 5120), (5, 16390, 1024), (7, 4100, 4096),
-                                   (8, 3300, 5120), (9, 16390, 1024), (13, 1030, 17408), (16, 3300, 5120), (16, 32800, 512)])
+                                   (8, 3300, 5120), (9, 16390, 1024), (13, 1030, 17408), (16, 3300, 5120), (16, 32800, 512),
+                                   (3, 33, 524288), (2, 17, 1048576)])      # the last two: a few very long rows
 @pytest.mark.parametrize("kind", ["f32", "bf16_outliers"])
 def test_rows_match_oracle(backend, m, n, k, kind):
     g = synth.rng(5100 * m + n + k)
@@ -39,7 +40,7 @@ def test_rows_match_oracle(backend, m, n, k, kind):
     a = {"f32": synth.activations_f32, "bf16_outliers": synth.activations_bf16_outliers}[kind](g, m, k)
     ref = oracle.gemm_fp8(a, codes, scales, m, n, k)
     got = fp8_gemm(backend, a, codes, scales, m, n, k)
-    tol, tol_norm = (2e-3, 1e-4) if kind == "bf16_outliers" else (2e-4, 2e-5)
+    tol, tol_norm = (2e-3, 1e-4) if kind == "bf16_outliers" else (2e-4, 2e-5 if k <= 65536 else 4e-5)   # (the oracle's own fp32 sum over half a million terms)
     print(f"gemm_fp8 {m}x{n}x{k} {kind}: max|d|/rms {rms_err(got, ref):.2e}, 2-norm {norm_err(got, ref):.2e}")
     assert rms_err(got, ref) <= tol and norm_err(got, ref) <= tol_norm
 
@@ -132,7 +133,8 @@ def fp8_block_gemm(backend, a, codes, scales, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(2, 4096, 4096), (3, 8192, 2048), (4, 3328, 5120), (5, 16384, 1024), (8, 3328, 5120),
-                                   (9, 4224, 4096), (13, 1024, 17408), (16, 3328, 5120), (16, 32768, 512)])
+                                   (9, 4224, 4096), (13, 1024, 17408), (16, 3328, 5120), (16, 32768, 512),
+                                   (3, 128, 262144)])
 @pytest.mark.parametrize("kind", ["f32", "bf16_outliers"])
 def test_block_scaled_rows_match_oracle(backend, m, n, k, kind):
     g = synth.rng(5600 * m + n + k)
@@ -140,7 +142,7 @@ def test_block_scaled_rows_match_oracle(backend, m, n, k, kind):
     a = {"f32": synth.activations_f32, "bf16_outliers": synth.activations_bf16_outliers}[kind](g, m, k)
     ref = oracle.gemm_fp8_block(a, codes, scales, m, n, k)
     got = fp8_block_gemm(backend, a, codes, scales, m, n, k)
-    tol, tol_norm = (2e-3, 1e-4) if kind == "bf16_outliers" else (2e-4, 2e-5)
+    tol, tol_norm = (2e-3, 1e-4) if kind == "bf16_outliers" else (2e-4, 2e-5 if k <= 65536 else 4e-5)
     print(f"gemm_fp8_block {m}x{n}x{k} {kind}: max|d|/rms {rms_err(got, ref):.2e}, 2-norm {norm_err(got, ref):.2e}")
     assert rms_err(got, ref) <= tol and norm_err(got, ref) <= tol_norm
 

@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per gate/up launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # same counter reads for a device copy of known size (profiles/q4k_gemv_m1_ffn27b_hbm_traffic.md);
 # a counter figure, not measured by this script.
-GATE_UP_HBM_TRAFFIC_BYTES = 50_530_000
+GATE_UP_HBM_TRAFFIC_BYTES = 50_526_000
 N_FF, K_HID = 17408, 5120
 
 
@@ -52,22 +52,42 @@ def vulkan_on_cpu_probe():
 
 
 def gpu_clocks():
-    """Core and memory clocks as rocm-smi reports them right after the timed region (best effort: None
-    where the tool is missing or refuses an ordinary user)."""
+    """Core and memory clocks right after the timed region, from the driver's sysfs tables (the level
+    marked current), else from rocm-smi (best effort: None where neither answers).  rocm-smi is a
+    script, i.e. a chain of exec calls: it is left alone when a profiler's preloaded library would
+    initialise the GPU in every process of that chain."""
+    import glob
+    import os
     import re
     import shutil
     import subprocess
 
+    clocks = {}
+    for dev in sorted(glob.glob("/sys/class/drm/card*/device")):
+        for name in ("sclk", "mclk", "fclk"):
+            try:
+                with open(os.path.join(dev, "pp_dpm_" + name)) as f:
+                    m = re.search(r"(\d+)\s*[Mm][Hh]z\s*\*", f.read())
+            except OSError:
+                m = None
+            if m:
+                clocks[name + "_MHz"] = int(m.group(1))
+        if clocks:
+            clocks["source"] = "sysfs"
+            return clocks
+    if any("rocprof" in v.lower() for k, v in os.environ.items() if k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB")):
+        return None
     smi = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
     try:
         out = subprocess.run([smi, "--showclocks"], capture_output=True, text=True, timeout=20).stdout
     except (OSError, subprocess.SubprocessError):
         return None
-    clocks = {}
     for name in ("sclk", "mclk", "fclk"):
         m = re.search(name + r" clock level: \S+: \((\d+)Mhz\)", out)
         if m:
             clocks[name + "_MHz"] = int(m.group(1))
+    if clocks:
+        clocks["source"] = "rocm-smi"
     return clocks or None
 
 

@@ -106,20 +106,22 @@ __device__ __forceinline__ BlockHead load_block_head(const uint8_t* raw) {
 }
 
 // The B operands of sub-block SB (32 weights of one row) for a lane of K half `kg`: b[t] holds
-// the weights 16t + 8kg + [0,8) in the order 0,2,1,3,4,6,5,7.  Sub-block SB lives in the low
-// (even SB) or high nibbles of bytes (SB/2)*32 + [0,32) (src/core/numerics/quant.cpp:656-675);
-// an odd SB decodes the bytes its even predecessor loaded, so `qw` (the words) and `qs8` (the
-// same shifted down one byte, for bytes 1 and 3) are carried from that call.
+// the weights 16kg + 8t + [0,8) in the order 0,2,1,3,4,6,5,7 (any assignment of the sub-block's K
+// positions to matrix steps and lane halves will do as long as the activation fragments follow it;
+// this one lets a lane take its sixteen bytes with ONE 16-byte LDS read, which sixteen lanes 144
+// bytes apart make without a bank conflict, where two 8-byte reads a lane put lanes l and l + 16 on
+// the same banks).  Sub-block SB lives in the low (even SB) or high nibbles of bytes
+// (SB/2)*32 + [0,32) (src/core/numerics/quant.cpp:656-675); an odd SB decodes the bytes its even
+// predecessor loaded, so `qw` (the words) and `qs8` (the same shifted down one byte, for bytes 1
+// and 3) are carried from that call.
 template <int SB>
 __device__ __forceinline__ void decode_subblock(const uint8_t* raw, uint32_t kg, const BlockHead& h, uint32_t (&qw)[4],
                                                 uint32_t (&qs8)[4], half8_t (&b)[2]) {
   constexpr int kHi = SB & 1;
   const ScaleMin sm = scale_min_f32<SB>(h.sbytes, h.d, h.ndmin);
   if (kHi == 0) {
-    const uint8_t* qp = raw + 16 + (SB >> 1) * 32 + kg * 8u;
-    const uint2 q0 = *reinterpret_cast<const uint2*>(qp);
-    const uint2 q1 = *reinterpret_cast<const uint2*>(qp + 16);
-    qw[0] = q0.x, qw[1] = q0.y, qw[2] = q1.x, qw[3] = q1.y;
+    const uint4 q = *reinterpret_cast<const uint4*>(raw + 16 + (SB >> 1) * 32 + kg * 16u);
+    qw[0] = q.x, qw[1] = q.y, qw[2] = q.z, qw[3] = q.w;
 #pragma unroll
     for (int x = 0; x < 4; ++x) qs8[x] = qw[x] >> 8;
   }
@@ -202,12 +204,12 @@ __device__ __forceinline__ void q4k_gemm_tile(
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // This lane's first weight row inside a raw stage (column tile j is 32 rows further), and its
-  // activation fragment offsets: MFMA step t of a slice takes chunk 2t + kg of the row
-  // (k = 16t + 8kg + [0,8)).
+  // activation fragment offsets: MFMA step t of a slice takes chunk 2kg + t of the row
+  // (k = 16kg + 8t + [0,8), the positions decode_subblock gives the step).
   const uint32_t w_row = (wave_n * WN + l32) * 144u;
   uint32_t a_fr[2];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) a_fr[tt] = (wave_m * WM + l32) * 64u + (((tt * 2u + kg) ^ ((l32 >> 2) & 3u)) * 16u);
+  for (int tt = 0; tt < 2; ++tt) a_fr[tt] = (wave_m * WM + l32) * 64u + (((kg * 2u + tt) ^ ((l32 >> 2) & 3u)) * 16u);
 
   const uint32_t slices = k / 32;
 

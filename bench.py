@@ -319,20 +319,6 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
             del wf_list, wf
         out[f"{fmt}_gemv"] = res
 
-    # ---- the matrix-core ceiling as measured here: a register-only loop of each GEMM's instruction
-    # ("mfma_probe"), constant operands and hashed ones (the part's power limit prices the toggling bits)
-    kmp = backend.LoadKernel("mfma_probe")
-    probe_wgs, probe_iters = 1024, 4000
-    pout = torch.empty(probe_wgs * 256, dtype=torch.float32, device=dev)
-    ceiling = {}
-    for kind, label, flop in ((0, "f16_32x32x16", 2 * 32 * 32 * 16), (1, "f8f4_scaled_32x32x64", 2 * 32 * 32 * 64),
-                              (2, "i8_16x16x64", 2 * 16 * 16 * 64)):
-        for rnd in (0, 1):
-            us = timed_us([(kmp, KernelLaunch(grid_x=probe_wgs, buffers=[wrap(pout)], scalars=[kind, rnd, probe_iters, probe_wgs]))],
-                          3, graph=False)
-            tflops = probe_wgs * 16 * probe_iters * flop / us / 1e6
-            ceiling[f"{label}_{'random' if rnd else 'constant'}"] = {"TFLOPs": round(tflops, 1)}
-    out["mfma_ceiling"] = ceiling
 
     # ---- configs[3]: prefill GEMM M=2048 ---------------------------------------------------
     m = 2048
@@ -388,10 +374,6 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
         prefill[f"{fmt}_n17408"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * n * k / us / 1e6, 1),
                                     "frac_fp16_peak": round(2 * m * n * k / us / 1e6 / 2500.0, 4)}
         del wf
-    for key, val in prefill.items():
-        ref_key = "f8f4_scaled_32x32x64_random" if key.startswith("mxfp4") else "f16_32x32x16_random"
-        mult = val.get("e4m3_terms", 1)          # the fp32-row form does `terms` times the fp8 work per product flop
-        val["frac_of_measured_ceiling"] = round(val["TFLOPs"] * mult / ceiling[ref_key]["TFLOPs"], 4)
     out["prefill_gemm_m2048_k5120"] = prefill
 
     # ---- the same prefill at the down-projection shape (N=5120, K=17408) ---------------------------
@@ -411,6 +393,27 @@ def other_cases(backend, torch, np, synth, KernelLaunch, dev, args):
     down["mxfp4"] = {"ms": round(us / 1e3, 4), "TFLOPs": round(2 * m * n * k / us / 1e6, 1),
                      "frac_fp8_peak": round(2 * m * n * k / us / 1e6 / 5000.0, 4)}
     out["prefill_gemm_m2048_n5120_k17408"] = down
+
+    # ---- the matrix-core ceiling as measured here (after the GEMMs it is compared with: the probe runs the
+    # part at its power limit, and what follows it within milliseconds runs at the clock that leaves): a
+    # register-only loop of each GEMM's instruction
+    # ("mfma_probe"), constant operands and hashed ones (the part's power limit prices the toggling bits)
+    kmp = backend.LoadKernel("mfma_probe")
+    probe_wgs, probe_iters = 1024, 4000
+    pout = torch.empty(probe_wgs * 256, dtype=torch.float32, device=dev)
+    ceiling = {}
+    for kind, label, flop in ((0, "f16_32x32x16", 2 * 32 * 32 * 16), (1, "f8f4_scaled_32x32x64", 2 * 32 * 32 * 64),
+                              (2, "i8_16x16x64", 2 * 16 * 16 * 64)):
+        for rnd in (0, 1):
+            us = timed_us([(kmp, KernelLaunch(grid_x=probe_wgs, buffers=[wrap(pout)], scalars=[kind, rnd, probe_iters, probe_wgs]))],
+                          3, graph=False)
+            tflops = probe_wgs * 16 * probe_iters * flop / us / 1e6
+            ceiling[f"{label}_{'random' if rnd else 'constant'}"] = {"TFLOPs": round(tflops, 1)}
+    out["mfma_ceiling"] = ceiling
+    for key, val in prefill.items():
+        ref_key = "f8f4_scaled_32x32x64_random" if key.startswith("mxfp4") else "f16_32x32x16_random"
+        mult = val.get("e4m3_terms", 1)          # the fp32-row form does `terms` times the fp8 work per product flop
+        val["frac_of_measured_ceiling"] = round(val["TFLOPs"] * mult / ceiling[ref_key]["TFLOPs"], 4)
     del a, w_q, w_mx, a8, y
 
     # ---- configs[4]: routed Q4_K experts ---------------------------------------------------

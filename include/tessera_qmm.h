@@ -141,6 +141,10 @@ const char* qmm_kernel_name(size_t index);
  *     matrix of 16 M weights or more with k a multiple of 512; from 17 rows with k a multiple of 128)
  *     each activation is carried to 16 significant bits under its row's largest magnitude (exactly,
  *     when it has no more); one row and the small shapes carry the full fp32 value.
+ *   - "gemm_fp8" and "gemm_fp8_block" likewise: 2..16 rows of a matrix of 16 M weights or more with k a
+ *     multiple of 512 run on the matrix cores (E4M3 weights as stored, activations to 16 significant
+ *     bits, the matrix core's own accumulation: within 2e-4 of the rms output of the reference's fp32
+ *     loop, 2e-3 with x20 outlier channels); other shapes on the vector unit in fp32.
  *   - "mfma_probe": buffer Out (workgroups * 256 floats); scalars kind (0 fp16 32x32x16, 1 scaled
  *     fp8 x fp4 32x32x64, 2 int8 16x16x64), random (0 constant operands, 1 hashed), iterations,
  *     workgroups.  "read_probe": a plain read of a buffer.  Measurement ids: the matrix-core and the
